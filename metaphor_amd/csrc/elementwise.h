@@ -1,0 +1,108 @@
+/*
+ * Flat elementwise engine: NIN read streams, NOUT write streams, one fused functor.
+ *
+ * The reference runs one thread per element with 4-byte accesses and a 32x over-sized grid
+ * (src/cuda/nvcc_src/addition.cu:3-14 with GRID_1D, src/cuda/kernel_header.h:100), and its
+ * 32-bit thread index wraps at 2^28 elements. Here every lane moves UNROLL 128-bit packs per
+ * stream, all loads are issued before the first use, indices are 64-bit, and the grid is
+ * exactly ceil(packs / (256*UNROLL)) workgroups.
+ *
+ * Aliasing: the reference's callers pass an output that aliases an input (c == b in
+ * src/ops/addition.zig:67-73). Each lane reads all of its elements before it writes any of
+ * them and no two lanes share an element, so any output may alias any input exactly.
+ */
+#ifndef MP_ELEMENTWISE_H
+#define MP_ELEMENTWISE_H
+
+#include "kernel_header.h"
+
+#if defined(__cplusplus) && defined(__HIPCC__)
+
+namespace mp {
+
+template <int NIN, int NOUT> struct EwPtrs {
+  const void* in[NIN];
+  void* out[NOUT];
+};
+
+constexpr int EW_BLOCK = 256;
+
+/* F::apply(const P (&in)[NIN], P (&out)[NOUT]) computes one element. */
+template <class T, int W, int NIN, int NOUT, int UNROLL, class F>
+__global__ __launch_bounds__(EW_BLOCK) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, size_t n, F f) {
+  using P = typename precision<T>::type;
+  const size_t npacks = n / W;
+  const size_t base = (size_t)blockIdx.x * (EW_BLOCK * UNROLL) + threadIdx.x;
+
+  P in[UNROLL][NIN][W];
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const size_t p = base + (size_t)u * EW_BLOCK;
+    if (p < npacks) {
+#pragma unroll
+      for (int s = 0; s < NIN; ++s)
+        load_pack_nt<T, W>(static_cast<const T*>(ptrs.in[s]) + p * W, in[u][s]);
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < UNROLL; ++u) {
+    const size_t p = base + (size_t)u * EW_BLOCK;
+    if (p < npacks) {
+      P out[NOUT][W];
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        P a[NIN], r[NOUT];
+#pragma unroll
+        for (int s = 0; s < NIN; ++s) a[s] = in[u][s][i];
+        f.apply(a, r);
+#pragma unroll
+        for (int s = 0; s < NOUT; ++s) out[s][i] = r[s];
+      }
+#pragma unroll
+      for (int s = 0; s < NOUT; ++s)
+        store_pack_nt<T, W>(static_cast<T*>(ptrs.out[s]) + p * W, out[s]);
+    }
+  }
+
+  /* the n % W elements after the last whole pack */
+  if (W > 1 && blockIdx.x == 0) {
+    const size_t e = npacks * W + threadIdx.x;
+    if (e < n) {
+      P a[NIN], r[NOUT];
+#pragma unroll
+      for (int s = 0; s < NIN; ++s) a[s] = (P) static_cast<const T*>(ptrs.in[s])[e];
+      f.apply(a, r);
+#pragma unroll
+      for (int s = 0; s < NOUT; ++s) static_cast<T*>(ptrs.out[s])[e] = (T)r[s];
+    }
+  }
+}
+
+/* Enqueue f over n elements. Operands that are all 16-byte aligned take the packed path;
+ * anything else takes the same kernel with one-element packs. n == 0 enqueues nothing. */
+template <class T, int NIN, int NOUT, int UNROLL, class F>
+inline void ew_launch(const EwPtrs<NIN, NOUT>& ptrs, size_t n, F f, hipStream_t stream) {
+  if (n == 0) return;
+  require(n / EW_BLOCK < 0x7fffffffull, "elementwise launch: too many elements for one grid");
+  bool packed = true;
+  for (int s = 0; s < NIN; ++s) packed = packed && aligned16(ptrs.in[s]);
+  for (int s = 0; s < NOUT; ++s) packed = packed && aligned16(ptrs.out[s]);
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  if (packed) {
+    const size_t npacks = n / W;
+    const size_t per_block = (size_t)EW_BLOCK * UNROLL;
+    size_t blocks = (npacks + per_block - 1) / per_block;
+    if (blocks == 0) blocks = 1; /* only a scalar tail */
+    ew_kernel<T, W, NIN, NOUT, UNROLL, F><<<dim3((unsigned)blocks), dim3(EW_BLOCK), 0, stream>>>(ptrs, n, f);
+  } else {
+    const size_t per_block = (size_t)EW_BLOCK * UNROLL;
+    const size_t blocks = (n + per_block - 1) / per_block;
+    ew_kernel<T, 1, NIN, NOUT, UNROLL, F><<<dim3((unsigned)blocks), dim3(EW_BLOCK), 0, stream>>>(ptrs, n, f);
+  }
+  MP_CHECK_LAUNCH();
+}
+
+}  // namespace mp
+
+#endif
+#endif

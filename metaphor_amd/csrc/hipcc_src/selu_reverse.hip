@@ -1,0 +1,21 @@
+#include "../elementwise.h"
+
+struct SeluReverseFn_Scalar {
+  template <class P> __device__ __forceinline__ void apply(const P (&in)[3], P (&out)[1]) const {
+    out[0] = in[1] + in[2] * mp::selu_slope(in[0]);
+  }
+};
+
+// a_grads += b_grads * selu'(a_value), selu' = scale for a > 0, scale*alpha*exp(a) otherwise.
+// Argument order and the accumulate-into-gradient convention of
+// src/cuda/nvcc_src/relu_reverse.cu:3-31.
+extern "C" void launch_selu_reverse_Scalar(
+  const void* a_value,
+  void* a_grads,
+  const void* b_grads,
+  len_t N,
+  StreamContext stream
+) {
+  const mp::EwPtrs<3, 1> ptrs{{a_value, a_grads, b_grads}, {a_grads}};
+  mp::ew_launch<Scalar, 3, 1, 2>(ptrs, N, SeluReverseFn_Scalar{}, get_stream(stream));
+}

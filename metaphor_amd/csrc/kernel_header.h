@@ -1,0 +1,357 @@
+/*
+ * Shared device header of the gfx950 kernel library.
+ *
+ * Takes the place of the reference's src/cuda/kernel_header.h:1-267 for the HIP build:
+ * the same roles (StreamContext access, error macros, DIMPAD, the up-cast `precision<T>`
+ * rule of src/cuda/tensor_types.h:51-69, reduction helpers), re-designed for CDNA4:
+ *   - wavefronts are 64 lanes; all-reduce is a DPP butterfly inside each 16-lane row
+ *     followed by v_permlane16_swap / v_permlane32_swap across rows, no LDS traffic
+ *     (the reference's warpReduce is a 32-lane __shfl_xor_sync loop, kernel_header.h:201-209);
+ *   - workgroup reductions publish one value per wave in LDS and every thread folds them
+ *     (the reference's blockReduce folds serially on thread 0, kernel_header.h:211-236);
+ *   - every global access of the tuned paths is one 128-bit pack per lane.
+ *
+ * Kernel sources are written against the placeholder type `Scalar`; the generator
+ * replicates each source for r16, r32 and r64 (reference: file_gen.zig:38,228-238).
+ */
+#ifndef MP_KERNEL_HEADER_H
+#define MP_KERNEL_HEADER_H
+
+#include "tensor_types.h"
+
+/* placeholder for editors; the generator rewrites every `Scalar` token before compiling */
+#define Scalar float
+
+#define DIMPAD(M, N) (((M) + ((N) - 1)) / (N))
+
+#if defined(__cplusplus) && defined(__HIPCC__)
+
+#include <hip/hip_runtime.h>
+#include <cmath>
+#include <cstdint>
+#include <cstdio>
+#include <cstdlib>
+
+inline hipStream_t get_stream(StreamContext context) {
+  return static_cast<hipStream_t>(context.hip_stream.ptr);
+}
+
+#define HIP_ASSERT(err) (mpHandleHipError((err), __FILE__, __LINE__))
+inline void mpHandleHipError(hipError_t err, const char* file, int line) {
+  if (err != hipSuccess) {
+    fprintf(stderr, "%s in %s at line %d\n", hipGetErrorString(err), file, line);
+    exit(EXIT_FAILURE);
+  }
+}
+
+/* a launch that the runtime rejects (bad grid, missing code object) must not pass silently */
+#define MP_CHECK_LAUNCH() HIP_ASSERT(hipGetLastError())
+
+namespace mp {
+
+/* argument checks of the launchers: same print-and-exit convention as a HIP error */
+inline void require(bool ok, const char* what) {
+  if (!ok) {
+    fprintf(stderr, "metaphor kernels: %s\n", what);
+    exit(EXIT_FAILURE);
+  }
+}
+
+constexpr int WAVE = MP_WAVE_SIZE;
+constexpr int PACK_BYTES = 16;
+
+/* ---------------------------------------------------------------------------------------
+ * numeric conventions
+ * ------------------------------------------------------------------------------------- */
+
+template <class T> struct precision { using type = float; };          /* r16, r32 -> fp32 */
+template <> struct precision<double> { using type = double; };        /* r64 -> fp64 */
+
+template <class T> constexpr int pack_width() { return PACK_BYTES / (int)sizeof(T); }
+
+template <class P> __device__ __forceinline__ P neg_inf();
+template <> __device__ __forceinline__ float neg_inf<float>() { return -__builtin_inff(); }
+template <> __device__ __forceinline__ double neg_inf<double>() { return -__builtin_inf(); }
+
+/* e^x. fp32: one v_exp_f32 on x*log2(e); fp64: library exp. */
+__device__ __forceinline__ float fast_exp(float x) {
+  return __builtin_amdgcn_exp2f(x * 1.44269504088896340736f);
+}
+__device__ __forceinline__ double fast_exp(double x) { return ::exp(x); }
+
+/* e^(x - m) with one fused multiply-add in fp32: exp2(x*log2e - m*log2e). The rounding of
+ * m*log2e is common to every element of a row, so it cancels in a normalised softmax. */
+__device__ __forceinline__ float exp_shifted(float x, float m_log2e) {
+  return __builtin_amdgcn_exp2f(__builtin_fmaf(x, 1.44269504088896340736f, -m_log2e));
+}
+__device__ __forceinline__ float shift_of(float m) { return m * 1.44269504088896340736f; }
+__device__ __forceinline__ double exp_shifted(double x, double m) { return ::exp(x - m); }
+__device__ __forceinline__ double shift_of(double m) { return m; }
+
+__device__ __forceinline__ float rsqrt_of(float x) { return 1.0f / __builtin_sqrtf(x); }
+__device__ __forceinline__ double rsqrt_of(double x) { return 1.0 / ::sqrt(x); }
+
+/* e^x - 1 for x <= 0, accurate near 0: an 8-term series inside (-0.25, 0], exp-1 below. */
+__device__ __forceinline__ float expm1_nonpos(float x) {
+  float p = 1.0f / 40320.0f;
+  p = __builtin_fmaf(p, x, 1.0f / 5040.0f);
+  p = __builtin_fmaf(p, x, 1.0f / 720.0f);
+  p = __builtin_fmaf(p, x, 1.0f / 120.0f);
+  p = __builtin_fmaf(p, x, 1.0f / 24.0f);
+  p = __builtin_fmaf(p, x, 1.0f / 6.0f);
+  p = __builtin_fmaf(p, x, 0.5f);
+  p = __builtin_fmaf(p * x, x, x);
+  const float big = fast_exp(x) - 1.0f;
+  return x > -0.25f ? p : big;
+}
+__device__ __forceinline__ double expm1_nonpos(double x) { return ::expm1(x); }
+
+template <class P> __device__ __forceinline__ P selu_value(P x) {
+  const P lam = (P)MP_SELU_SCALE, la = (P)(MP_SELU_SCALE * MP_SELU_ALPHA);
+  const P neg = la * expm1_nonpos(x > (P)0 ? (P)0 : x);
+  return x > (P)0 ? lam * x : neg;
+}
+template <class P> __device__ __forceinline__ P selu_slope(P x) {
+  const P lam = (P)MP_SELU_SCALE, la = (P)(MP_SELU_SCALE * MP_SELU_ALPHA);
+  const P neg = la * fast_exp(x > (P)0 ? (P)0 : x);
+  return x > (P)0 ? lam : neg;
+}
+
+/* ---------------------------------------------------------------------------------------
+ * 128-bit packs
+ * ------------------------------------------------------------------------------------- */
+
+template <class T, int W> struct vec_of { typedef T type __attribute__((ext_vector_type(W))); };
+
+/* Load W consecutive elements (one pack when W > 1; p must be 16-byte aligned then). */
+template <class T, int W, class P>
+__device__ __forceinline__ void load_pack(const T* p, P (&out)[W]) {
+  if constexpr (W == 1) {
+    out[0] = (P)p[0];
+  } else {
+    using V = typename vec_of<T, W>::type;
+    const V v = *reinterpret_cast<const V*>(p);
+#pragma unroll
+    for (int i = 0; i < W; ++i) out[i] = (P)v[i];
+  }
+}
+
+/* Streaming variant: the data is not needed again by this kernel. */
+template <class T, int W, class P>
+__device__ __forceinline__ void load_pack_nt(const T* p, P (&out)[W]) {
+  if constexpr (W == 1) {
+    out[0] = (P)__builtin_nontemporal_load(p);
+  } else {
+    using V = typename vec_of<T, W>::type;
+    const V v = __builtin_nontemporal_load(reinterpret_cast<const V*>(p));
+#pragma unroll
+    for (int i = 0; i < W; ++i) out[i] = (P)v[i];
+  }
+}
+
+template <class T, int W, class P>
+__device__ __forceinline__ void store_pack(T* p, const P (&in)[W]) {
+  if constexpr (W == 1) {
+    p[0] = (T)in[0];
+  } else {
+    using V = typename vec_of<T, W>::type;
+    V v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) v[i] = (T)in[i];
+    *reinterpret_cast<V*>(p) = v;
+  }
+}
+
+/* Write-once output: non-temporal so it does not evict what is still to be read. */
+template <class T, int W, class P>
+__device__ __forceinline__ void store_pack_nt(T* p, const P (&in)[W]) {
+  if constexpr (W == 1) {
+    __builtin_nontemporal_store((T)in[0], p);
+  } else {
+    using V = typename vec_of<T, W>::type;
+    V v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) v[i] = (T)in[i];
+    __builtin_nontemporal_store(v, reinterpret_cast<V*>(p));
+  }
+}
+
+inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
+inline unsigned misalign16(const void* p) { return (unsigned)(reinterpret_cast<uintptr_t>(p) & 15u); }
+
+/* ---------------------------------------------------------------------------------------
+ * cross-lane reductions (all 64 lanes must be active)
+ * ------------------------------------------------------------------------------------- */
+
+struct AddOP { template <class P> static __device__ __forceinline__ P apply(P a, P b) { return a + b; } };
+struct MaxOP { template <class P> static __device__ __forceinline__ P apply(P a, P b) { return a > b ? a : b; } };
+
+/* DPP controls: quad_perm [1,0,3,2], quad_perm [2,3,0,1], row_half_mirror, row_mirror */
+constexpr int DPP_XOR1 = 0xB1, DPP_XOR2 = 0x4E, DPP_HALF_MIRROR = 0x141, DPP_MIRROR = 0x140;
+
+template <int CTRL> __device__ __forceinline__ float dpp_move(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int CTRL> __device__ __forceinline__ double dpp_move(double v) {
+  const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+  const unsigned lo = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)b, CTRL, 0xF, 0xF, true);
+  const unsigned hi = (unsigned)__builtin_amdgcn_update_dpp(0, (int)(unsigned)(b >> 32), CTRL, 0xF, 0xF, true);
+  return __builtin_bit_cast(double, ((unsigned long long)hi << 32) | lo);
+}
+
+typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
+
+/* After the four DPP steps every lane of a 16-lane row holds that row's result; the two
+ * swaps exchange odd/even rows and then the wave halves, returning both values to fold. */
+template <class OP> __device__ __forceinline__ float fold_rows(float v) {
+  /* the two results are copied to scalars before the bit cast: casting the vector element
+   * expression itself reads element 0 twice with this compiler */
+  uint2_t r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+  unsigned kept = r[0], swapped = r[1];
+  v = OP::apply(__builtin_bit_cast(float, kept), __builtin_bit_cast(float, swapped));
+  r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+  kept = r[0];
+  swapped = r[1];
+  return OP::apply(__builtin_bit_cast(float, kept), __builtin_bit_cast(float, swapped));
+}
+template <class OP> __device__ __forceinline__ double fold_rows(double v) {
+  unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+  uint2_t lo = __builtin_amdgcn_permlane16_swap((unsigned)b, (unsigned)b, false, false);
+  uint2_t hi = __builtin_amdgcn_permlane16_swap((unsigned)(b >> 32), (unsigned)(b >> 32), false, false);
+  v = OP::apply(__builtin_bit_cast(double, ((unsigned long long)hi[0] << 32) | lo[0]),
+                __builtin_bit_cast(double, ((unsigned long long)hi[1] << 32) | lo[1]));
+  b = __builtin_bit_cast(unsigned long long, v);
+  lo = __builtin_amdgcn_permlane32_swap((unsigned)b, (unsigned)b, false, false);
+  hi = __builtin_amdgcn_permlane32_swap((unsigned)(b >> 32), (unsigned)(b >> 32), false, false);
+  return OP::apply(__builtin_bit_cast(double, ((unsigned long long)hi[0] << 32) | lo[0]),
+                   __builtin_bit_cast(double, ((unsigned long long)hi[1] << 32) | lo[1]));
+}
+
+/* Every lane of the wave returns OP folded over all 64 lanes. */
+template <class OP, class P> __device__ __forceinline__ P wave_allreduce(P v) {
+  v = OP::apply(v, dpp_move<DPP_XOR1>(v));
+  v = OP::apply(v, dpp_move<DPP_XOR2>(v));
+  v = OP::apply(v, dpp_move<DPP_HALF_MIRROR>(v));
+  v = OP::apply(v, dpp_move<DPP_MIRROR>(v));
+  return fold_rows<OP>(v);
+}
+
+/* Every thread of a G-thread group (G/64 consecutive waves of the workgroup) returns OP
+ * folded over the group. `slots` points at the group's G/64 LDS words for THIS reduction;
+ * two reductions in flight must use different slots, and a loop that reuses slots must
+ * alternate between two sets, which makes the single barrier below sufficient. */
+template <class OP, int G, class P>
+__device__ __forceinline__ P group_allreduce(P v, P* slots, int lane_in_group) {
+  v = wave_allreduce<OP>(v);
+  if constexpr (G == WAVE) {
+    return v;
+  } else {
+    if ((lane_in_group & (WAVE - 1)) == 0) slots[lane_in_group / WAVE] = v;
+    __syncthreads();
+    P r = slots[0];
+#pragma unroll
+    for (int i = 1; i < G / WAVE; ++i) r = OP::apply(r, slots[i]);
+    return r;
+  }
+}
+
+/* ---------------------------------------------------------------------------------------
+ * row geometry: [head scalars][nvec aligned packs][tail scalars]
+ * ------------------------------------------------------------------------------------- */
+
+template <class T, int W> struct RowGeom {
+  int head;  /* elements before the first 16-byte boundary */
+  int nvec;  /* whole packs */
+  int tail;  /* elements after the last whole pack */
+  __device__ __forceinline__ RowGeom(const T* row, size_t n, bool ragged) {
+    if (W == 1 || !ragged) {
+      head = 0;
+      nvec = (int)(n / W);
+      tail = (int)(n - (size_t)nvec * W);
+    } else {
+      const unsigned mis = (unsigned)(reinterpret_cast<uintptr_t>(row) & 15u);
+      int h = (int)(((16u - mis) & 15u) / sizeof(T));
+      if ((size_t)h > n) h = (int)n;
+      head = h;
+      nvec = (int)((n - h) / W);
+      tail = (int)(n - h - (size_t)nvec * W);
+    }
+  }
+};
+
+/* A row held in registers by a group of G threads: NV packs per thread plus, for ragged
+ * rows, one edge element on the group's first head+tail threads. */
+template <class T, int W, int G, int NV, bool RAGGED> struct RowTile {
+  using P = typename precision<T>::type;
+  P v[NV][W];
+  P edge;
+
+  __device__ __forceinline__ void load(const T* row, const RowGeom<T, W>& g, int lane, P fill) {
+    const T* body = row + g.head;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      if (p < g.nvec) {
+        load_pack<T, W>(body + (size_t)p * W, v[k]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) v[k][i] = fill;
+      }
+    }
+    edge = fill;
+    if constexpr (RAGGED) {
+      if (lane < g.head) edge = (P)row[lane];
+      else if (lane - g.head < g.tail) edge = (P)body[(size_t)g.nvec * W + (lane - g.head)];
+    }
+  }
+
+  __device__ __forceinline__ void store(T* row, const RowGeom<T, W>& g, int lane) const {
+    T* body = row + g.head;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      if (p < g.nvec) store_pack_nt<T, W>(body + (size_t)p * W, v[k]);
+    }
+    if constexpr (RAGGED) {
+      if (lane < g.head) row[lane] = (T)edge;
+      else if (lane - g.head < g.tail) body[(size_t)g.nvec * W + (lane - g.head)] = (T)edge;
+    }
+  }
+
+  /* f(value&, k, i) over pack elements; i == -1 marks the edge element */
+  template <class F> __device__ __forceinline__ void each(F f) {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+#pragma unroll
+      for (int i = 0; i < W; ++i) f(v[k][i]);
+    }
+    if constexpr (RAGGED) f(edge);
+  }
+};
+
+/* ---------------------------------------------------------------------------------------
+ * row-regime selection shared by the softmax and RMSNorm launchers
+ * ------------------------------------------------------------------------------------- */
+
+/* Packs a thread must hold so that a G-thread group covers `packs` packs; 0 = too long. */
+inline int packs_per_thread(size_t packs, int G, int max_nv) {
+  for (int nv = 1; nv <= max_nv; nv *= 2)
+    if ((size_t)nv * G >= packs) return nv;
+  return 0;
+}
+
+/* The GPU's compute-unit count, read once per process. */
+inline int compute_units() {
+  static int cus = [] {
+    int dev = 0, n = 0;
+    HIP_ASSERT(hipGetDevice(&dev));
+    HIP_ASSERT(hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev));
+    return n > 0 ? n : 256;
+  }();
+  return cus;
+}
+
+}  // namespace mp
+
+#endif  /* __cplusplus && __HIPCC__ */
+#endif  /* MP_KERNEL_HEADER_H */

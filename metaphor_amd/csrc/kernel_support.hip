@@ -1,0 +1,26 @@
+/*
+ * Exports of the kernel library that are not per-dtype launchers: workspace sizing and the
+ * diagnostic row-regime override. Compiled once (no `Scalar` replication).
+ */
+#include "row_rmsnorm.h"
+
+// Bytes of caller-owned scratch that launch_rmsnorm_ij_j_reverse_<dtype> needs for an [m, n]
+// problem: one row of n accumulators (fp32 for r16/r32, fp64 for r64) per workgroup, at most
+// one workgroup per compute unit. dtype is the dispatch key 0 = r16, 1 = r32, 2 = r64
+// (the order of the reference's scalar.Tag, src/core/scalar.zig:35-40).
+extern "C" len_t mpRmsnormReverseScratchBytes(len_t dtype, len_t m, len_t n) {
+  switch (dtype) {
+    case MP_R16: return mp::rmsnorm_reverse_scratch_bytes<r16>(m, n);
+    case MP_R32: return mp::rmsnorm_reverse_scratch_bytes<r32>(m, n);
+    case MP_R64: return mp::rmsnorm_reverse_scratch_bytes<r64>(m, n);
+    default: mp::require(false, "mpRmsnormReverseScratchBytes: dtype must be 0, 1 or 2"); return 0;
+  }
+}
+
+// Diagnostic: force the row regime of the softmax / RMSNorm launchers (0 auto, 1 wave,
+// 2 block, 3 wide, 4 stream). A regime that cannot hold a row falls through to the next wider
+// one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
+extern "C" void mpSetRowRegime(len_t regime) {
+  mp::require(regime <= mp::REGIME_STREAM, "mpSetRowRegime: regime must be 0..4");
+  mp::row_regime_override() = (int)regime;
+}

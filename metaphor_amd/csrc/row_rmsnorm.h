@@ -1,0 +1,446 @@
+/*
+ * RMSNorm over the last dimension, forward and reverse.
+ *
+ * The reference has no RMSNorm kernel; its row-reduce (src/cuda/nvcc_src/reduce_ij_i.cu:3-54)
+ * and column-reduce (src/cuda/nvcc_src/reduce_ij_j.cu:3-66) are the nearest patterns. Math:
+ *   forward   r_i   = (mean_j x_ij^2 + eps)^(-1/2),   y_ij = x_ij * r_i * g_j
+ *   reverse   c_i   = mean_j(dy_ij * g_j * x_ij)
+ *             dx_ij = r_i * (dy_ij*g_j - x_ij * r_i^2 * c_i) + alpha * dx_ij
+ *             dg_j  = sum_i dy_ij * x_ij * r_i               + alpha * dg_j
+ * Accumulation is in precision<T>; the last stage of dg sums in fp64.
+ *
+ * Workgroups are persistent: 1024 threads hold 1024/G rows at a time and walk the rows with
+ * the gain vector (and, in reverse, the per-column dg sums) resident in registers. The
+ * reverse reads x and dy once, folds both row reductions into one barrier, writes dx, and at
+ * the end combines the workgroup's dg sums through LDS into ONE partial row per workgroup;
+ * a second small kernel adds the partial rows in a fixed order, so dg is deterministic.
+ */
+#ifndef MP_ROW_RMSNORM_H
+#define MP_ROW_RMSNORM_H
+
+#include "row_dispatch.h"
+
+#if defined(__cplusplus) && defined(__HIPCC__)
+
+namespace mp {
+
+constexpr int NORM_BLOCK = 1024;
+
+/* Both values folded over a G-thread group with a single barrier. */
+template <int G, class P>
+__device__ __forceinline__ void group_allreduce_sum2(P& a, P& b, P* slots_a, P* slots_b, int lane) {
+  a = wave_allreduce<AddOP>(a);
+  b = wave_allreduce<AddOP>(b);
+  if constexpr (G > WAVE) {
+    if ((lane & (WAVE - 1)) == 0) {
+      slots_a[lane / WAVE] = a;
+      slots_b[lane / WAVE] = b;
+    }
+    __syncthreads();
+    a = slots_a[0];
+    b = slots_b[0];
+#pragma unroll
+    for (int i = 1; i < G / WAVE; ++i) {
+      a += slots_a[i];
+      b += slots_b[i];
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ resident forward */
+
+template <class T, int W, int G, int NV, bool RAGGED>
+__global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_fwd_resident(
+    const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  constexpr int RPB = NORM_BLOCK / G;
+  __shared__ P slots[2][RPB][G / WAVE];
+
+  const int sub = threadIdx.x / G, lane = threadIdx.x % G;
+
+  P gv[NV][W];
+  if constexpr (!RAGGED) { /* aligned rows: a thread's columns are the same in every row */
+    const int nvec = (int)(n / W);
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      if (p < nvec) {
+        load_pack<T, W>(gain + (size_t)p * W, gv[k]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) gv[k][i] = (P)0;
+      }
+    }
+  }
+
+  int parity = 0;
+  for (size_t base = (size_t)blockIdx.x * RPB; base < m; base += (size_t)gridDim.x * RPB, parity ^= 1) {
+    const size_t row = base + sub;
+    const bool live = row < m; /* uniform per wave; dead groups still meet the barrier */
+    const T* xr = x + (live ? row : 0) * n;
+    const RowGeom<T, W> g(xr, n, RAGGED);
+    RowTile<T, W, G, NV, RAGGED> t;
+    t.load(xr, g, live ? lane : 0x3fffffff, (P)0);
+
+    P ss = (P)0;
+    t.each([&](P& e) { ss += e * e; });
+    ss = group_allreduce<AddOP, G>(ss, slots[parity][sub], lane);
+    const P r = rsqrt_of(ss / (P)n + eps);
+
+    if (live) {
+      if constexpr (!RAGGED) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
+#pragma unroll
+          for (int i = 0; i < W; ++i) t.v[k][i] *= r * gv[k][i];
+      } else {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+          const int p = k * G + lane;
+          if (p < g.nvec) {
+#pragma unroll
+            for (int i = 0; i < W; ++i) t.v[k][i] *= r * (P)gain[(size_t)g.head + (size_t)p * W + i];
+          }
+        }
+        if (lane < g.head) t.edge *= r * (P)gain[lane];
+        else if (lane - g.head < g.tail) t.edge *= r * (P)gain[(size_t)g.head + (size_t)g.nvec * W + (lane - g.head)];
+      }
+      t.store(y + row * n, g, lane);
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ streaming forward */
+
+template <class T, int W>
+__global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_fwd_stream(
+    const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  constexpr int G = STREAM_THREADS, U = 4;
+  __shared__ P slots[2][G / WAVE];
+  const int lane = threadIdx.x;
+  int parity = 0;
+
+  for (size_t row = blockIdx.x; row < m; row += gridDim.x, parity ^= 1) {
+    const T* xr = x + row * n;
+    T* yr = y + row * n;
+    const RowGeom<T, W> g(xr, n, true);
+    const T* body = xr + g.head;
+    T* ybody = yr + g.head;
+
+    P ss = (P)0;
+    for (int p0 = lane; p0 < g.nvec; p0 += G * U) {
+      P buf[U][W];
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const int p = p0 + u * G;
+        if (p < g.nvec) {
+          load_pack<T, W>(body + (size_t)p * W, buf[u]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < W; ++i) buf[u][i] = (P)0;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < W; ++i) ss += buf[u][i] * buf[u][i];
+    }
+    size_t edge = (size_t)-1;
+    if (W > 1) {
+      if (lane < g.head) edge = (size_t)lane;
+      else if (lane - g.head < g.tail) edge = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
+      if (edge != (size_t)-1) ss += (P)xr[edge] * (P)xr[edge];
+    }
+    ss = group_allreduce<AddOP, G>(ss, slots[parity], lane);
+    const P r = rsqrt_of(ss / (P)n + eps);
+
+    for (int p = lane; p < g.nvec; p += G) {
+      P buf[W];
+      load_pack_nt<T, W>(body + (size_t)p * W, buf);
+#pragma unroll
+      for (int i = 0; i < W; ++i) buf[i] *= r * (P)gain[(size_t)g.head + (size_t)p * W + i];
+      store_pack_nt<T, W>(ybody + (size_t)p * W, buf);
+    }
+    if (W > 1 && edge != (size_t)-1) yr[edge] = (T)((P)xr[edge] * r * (P)gain[edge]);
+  }
+}
+
+/* ------------------------------------------------------------------ resident reverse */
+
+/* Rows must be pack-aligned (n % W == 0, every base 16-byte aligned) or W must be 1, so that
+ * a thread owns the same columns in every row and can keep their dg sums in registers.
+ * partials holds gridDim.x rows of n values of precision<T>. */
+template <class T, int W, int G, int NV, bool BLEND>
+__global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
+    const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
+    typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  constexpr int RPB = NORM_BLOCK / G;
+  __shared__ P slots[2][2][RPB][G / WAVE];
+  __shared__ P comb[RPB > 1 ? G * NV * W : 1];
+
+  const int sub = threadIdx.x / G, lane = threadIdx.x % G;
+  const int nvec = (int)(n / W);
+
+  P gv[NV][W], acc[NV][W];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
+#pragma unroll
+    for (int i = 0; i < W; ++i) acc[k][i] = gv[k][i] = (P)0;
+    if (p < nvec) load_pack<T, W>(gain + (size_t)p * W, gv[k]);
+  }
+
+  int parity = 0;
+  for (size_t base = (size_t)blockIdx.x * RPB; base < m; base += (size_t)gridDim.x * RPB, parity ^= 1) {
+    const size_t row = base + sub;
+    const bool live = row < m;
+    const size_t off = (live ? row : 0) * n;
+
+    P xv[NV][W], dv[NV][W];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      if (live && p < nvec) {
+        load_pack_nt<T, W>(x + off + (size_t)p * W, xv[k]);
+        load_pack_nt<T, W>(dy + off + (size_t)p * W, dv[k]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) xv[k][i] = dv[k][i] = (P)0;
+      }
+    }
+
+    P ss = (P)0, c = (P)0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        ss += xv[k][i] * xv[k][i];
+        c += dv[k][i] * gv[k][i] * xv[k][i];
+      }
+    group_allreduce_sum2<G>(ss, c, slots[parity][0][sub], slots[parity][1][sub], lane);
+    const P r = rsqrt_of(ss / (P)n + eps);
+    const P cc = c / (P)n * r * r;
+
+    if (live) {
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        const int p = k * G + lane;
+        if (p < nvec) {
+          P out[W];
+#pragma unroll
+          for (int i = 0; i < W; ++i) {
+            out[i] = r * (dv[k][i] * gv[k][i] - xv[k][i] * cc);
+            acc[k][i] += dv[k][i] * xv[k][i] * r;
+          }
+          if constexpr (BLEND) {
+            P old[W];
+            load_pack<T, W>(dx + off + (size_t)p * W, old);
+#pragma unroll
+            for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+          }
+          store_pack_nt<T, W>(dx + off + (size_t)p * W, out);
+        }
+      }
+    }
+  }
+
+  /* one partial row per workgroup */
+  P* mine = partials + (size_t)blockIdx.x * n;
+  if constexpr (RPB > 1) {
+    for (int s = 0; s < RPB; ++s) {
+      if (sub == s) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k)
+#pragma unroll
+          for (int i = 0; i < W; ++i) {
+            const int idx = (k * G + lane) * W + i;
+            comb[idx] = (s == 0 ? (P)0 : comb[idx]) + acc[k][i];
+          }
+      }
+      __syncthreads();
+    }
+    for (size_t col = threadIdx.x; col < n; col += NORM_BLOCK) mine[col] = comb[col];
+  } else {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      if (p < nvec) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) mine[(size_t)p * W + i] = acc[k][i];
+      }
+    }
+  }
+}
+
+/* ------------------------------------------------------------------ streaming reverse */
+
+/* Rows too long for registers. Same alignment rule as the resident reverse. Each workgroup
+ * owns one partial row and adds every row it processes into it (first row: overwrite). */
+template <class T, int W, bool BLEND>
+__global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
+    const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
+    typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  constexpr int G = STREAM_THREADS;
+  __shared__ P slots[2][2][G / WAVE];
+  const int lane = threadIdx.x;
+  const int nvec = (int)(n / W);
+  P* mine = partials + (size_t)blockIdx.x * n;
+  int parity = 0;
+  bool first = true;
+
+  for (size_t row = blockIdx.x; row < m; row += gridDim.x, parity ^= 1, first = false) {
+    const size_t off = row * n;
+    P ss = (P)0, c = (P)0;
+    for (int p = lane; p < nvec; p += G) {
+      P xv[W], dv[W], gv[W];
+      load_pack<T, W>(x + off + (size_t)p * W, xv);
+      load_pack<T, W>(dy + off + (size_t)p * W, dv);
+      load_pack<T, W>(gain + (size_t)p * W, gv);
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        ss += xv[i] * xv[i];
+        c += dv[i] * gv[i] * xv[i];
+      }
+    }
+    group_allreduce_sum2<G>(ss, c, slots[parity][0], slots[parity][1], lane);
+    const P r = rsqrt_of(ss / (P)n + eps);
+    const P cc = c / (P)n * r * r;
+
+    for (int p = lane; p < nvec; p += G) {
+      P xv[W], dv[W], gv[W], out[W];
+      load_pack_nt<T, W>(x + off + (size_t)p * W, xv);
+      load_pack_nt<T, W>(dy + off + (size_t)p * W, dv);
+      load_pack<T, W>(gain + (size_t)p * W, gv);
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        out[i] = r * (dv[i] * gv[i] - xv[i] * cc);
+        const P t = dv[i] * xv[i] * r;
+        P* slot = mine + (size_t)p * W + i;
+        *slot = first ? t : *slot + t;
+      }
+      if constexpr (BLEND) {
+        P old[W];
+        load_pack<T, W>(dx + off + (size_t)p * W, old);
+#pragma unroll
+        for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+      }
+      store_pack_nt<T, W>(dx + off + (size_t)p * W, out);
+    }
+  }
+}
+
+/* dg_j = sum over partial rows (fixed order, fp64) + alpha * dg_j. 64 columns per workgroup,
+ * 16 waves split the partial rows. */
+template <class T>
+__global__ __launch_bounds__(1024) void rmsnorm_dgain_finish(
+    const typename precision<T>::type* partials, T* dg, double alpha, int rows, size_t n) {
+  __shared__ double part[16][WAVE];
+  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
+  const size_t col = (size_t)blockIdx.x * WAVE + lane;
+  double s = 0.0;
+  if (col < n)
+    for (int p = w; p < rows; p += 16) s += (double)partials[(size_t)p * n + col];
+  part[w][lane] = s;
+  __syncthreads();
+  if (w == 0 && col < n) {
+    double t = 0.0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t += part[i][lane];
+    if (alpha != 0.0) t += alpha * (double)dg[col];
+    dg[col] = (T)t;
+  }
+}
+
+/* ------------------------------------------------------------------ host dispatch */
+
+/* Partial rows the reverse may write: one per workgroup, at most one workgroup per CU. */
+inline size_t rmsnorm_reverse_partial_rows(size_t m) {
+  const size_t cus = (size_t)compute_units();
+  return m < cus ? (m ? m : 1) : cus;
+}
+
+template <class T>
+inline size_t rmsnorm_reverse_scratch_bytes(size_t m, size_t n) {
+  return rmsnorm_reverse_partial_rows(m) * n * sizeof(typename precision<T>::type);
+}
+
+template <class T>
+inline void rmsnorm_forward(const T* x, const T* gain, T* y, double eps, size_t m, size_t n,
+                            hipStream_t stream) {
+  if (m == 0 || n == 0) return;
+  using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  require(n <= 0x40000000ull, "rmsnorm: row length must not exceed 2^30");
+  const size_t cap = (size_t)compute_units() * 2;
+  if (misalign16(x) != misalign16(y)) {
+    const size_t grid = m < cap ? m : cap;
+    rmsnorm_fwd_stream<T, 1><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
+    MP_CHECK_LAUNCH();
+    return;
+  }
+  const bool ragged = !(aligned16(x) && aligned16(gain) && (n % W) == 0);
+  constexpr int MAXNV = max_nv_for<T>(32);
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV);
+  const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
+    const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
+    const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
+    if (ragged) rmsnorm_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+    else rmsnorm_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+  });
+  if (!resident) {
+    const size_t grid = m < cap ? m : cap;
+    rmsnorm_fwd_stream<T, W><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
+  }
+  MP_CHECK_LAUNCH();
+}
+
+template <class T, int W>
+inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* dg, void* scratch,
+                              double eps, double alpha, size_t m, size_t n, hipStream_t stream) {
+  using P = typename precision<T>::type;
+  P* partials = static_cast<P*>(scratch);
+  const size_t max_rows = rmsnorm_reverse_partial_rows(m);
+  const bool blend = alpha != 0.0;
+  unsigned rows = 0;
+  /* four register arrays per thread (x, dy, gain, dg sums): 16 registers each when packed,
+   * 8 elements each on the element-wise path */
+  constexpr int MAXNV = W == 1 ? 8 : max_nv_for<T>(16);
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV);
+  const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
+    const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
+    rows = (unsigned)(need < max_rows ? need : max_rows);
+    const dim3 grid(rows), block(NORM_BLOCK);
+    if (blend) rmsnorm_rev_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+    else rmsnorm_rev_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+  });
+  if (!resident) {
+    rows = (unsigned)max_rows;
+    const dim3 grid(rows), block(STREAM_THREADS);
+    if (blend) rmsnorm_rev_stream<T, W, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+    else rmsnorm_rev_stream<T, W, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+  }
+  MP_CHECK_LAUNCH();
+  const unsigned fin = (unsigned)((n + WAVE - 1) / WAVE);
+  rmsnorm_dgain_finish<T><<<dim3(fin), dim3(1024), 0, stream>>>(partials, dg, alpha, (int)rows, n);
+  MP_CHECK_LAUNCH();
+}
+
+template <class T>
+inline void rmsnorm_reverse(const T* x, const T* gain, const T* dy, T* dx, T* dg, void* scratch,
+                            double eps, double alpha, size_t m, size_t n, hipStream_t stream) {
+  if (m == 0 || n == 0) return;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  require(n <= 0x40000000ull, "rmsnorm reverse: row length must not exceed 2^30");
+  require(scratch != nullptr, "rmsnorm reverse: scratch must hold mpRmsnormReverseScratchBytes bytes");
+  const bool packed = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gain) && (n % W) == 0;
+  if (packed) rmsnorm_reverse_w<T, W>(x, gain, dy, dx, dg, scratch, eps, alpha, m, n, stream);
+  else rmsnorm_reverse_w<T, 1>(x, gain, dy, dx, dg, scratch, eps, alpha, m, n, stream);
+}
+
+}  // namespace mp
+
+#endif
+#endif

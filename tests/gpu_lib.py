@@ -1,0 +1,202 @@
+"""Helpers of the GPU parity tests: call the launchers through the C-ABI on torch-owned
+device memory, guard every buffer with canaries, and compare against the fp64 oracle with
+the tolerances stated for this path."""
+import sys
+
+import numpy as np
+import torch
+
+from metaphor_amd import ffi
+
+KEY = {torch.float16: ffi.R16, torch.float32: ffi.R32, torch.float64: ffi.R64}
+NP_OF = {torch.float16: np.float16, torch.float32: np.float32, torch.float64: np.float64}
+
+# r32: 1e-5 relative (softmax outputs: 1e-6 absolute); r16: 2e-3 relative with a floor of one
+# r16 subnormal ulp; r64 is held to 1e-12 relative. "Relative" is against
+# max(|ref|, RMS of the reference row or tensor), which keeps cancellation-prone entries
+# (dx of softmax, dg of RMSNorm) meaningful.
+RTOL = {torch.float16: 2e-3, torch.float32: 1e-5, torch.float64: 1e-12}
+FLOOR = {torch.float16: 2.0 ** -24, torch.float32: 0.0, torch.float64: 0.0}
+SOFTMAX_ATOL = {torch.float16: 2e-3, torch.float32: 1e-6, torch.float64: 1e-13}
+
+GUARD = 64
+_SENTINEL = 12345.0
+
+
+def say(msg):
+    """Name the case before each GPU step, so a lost box still tells which one it was."""
+    print(f"[gpu-case] {msg}", flush=True)
+    sys.stdout.flush()
+
+
+def lib():
+    kernels, utils = ffi.load()
+    return kernels, utils
+
+
+def ctx():
+    return ffi.StreamContext.from_handle(torch.cuda.current_stream().cuda_stream)
+
+
+class Guarded:
+    """A device tensor inside a larger buffer whose margins hold a sentinel. `shift`
+    elements move the view off 16-byte alignment."""
+
+    def __init__(self, shape, dtype, shift=0, fill=None):
+        n = int(np.prod(shape)) if len(shape) else 1
+        # keep the interior 16-byte aligned at shift 0: GUARD elements of any dtype are >= 128 bytes
+        self.sentinel = _SENTINEL if dtype.is_floating_point else 165
+        self.buf = torch.full((n + 2 * GUARD + shift,), self.sentinel, dtype=dtype, device="cuda")
+        self.lo = GUARD + shift
+        self.t = self.buf[self.lo:self.lo + n].view(*shape) if n else self.buf[self.lo:self.lo].view(*shape)
+        if fill is not None:
+            self.t.copy_(fill)
+
+    def check(self, what):
+        lo = self.buf[:self.lo]
+        hi = self.buf[self.lo + self.t.numel():]
+        ok = bool((lo == self.sentinel).all()) and bool((hi == self.sentinel).all())
+        assert ok, f"{what}: wrote outside its buffer"
+
+
+def dev(a, dtype, shift=0):
+    """numpy -> guarded device tensor of `dtype` (values rounded to the storage type first)."""
+    t = torch.from_numpy(np.ascontiguousarray(a)).to(dtype)
+    g = Guarded(tuple(t.shape), dtype, shift)
+    g.t.copy_(t)
+    return g
+
+
+def host(t):
+    """device tensor -> numpy in its storage dtype (what the oracle must read)."""
+    return t.detach().cpu().numpy()
+
+
+def compare(got, ref, dtype, what, rowwise=True, rtol=None, atol=None, scale=None):
+    """|got - ref| <= rtol * max(|ref|, RMS(ref row|tensor), scale) + floor (or a plain atol).
+
+    `scale` is the magnitude of the terms an entry is the difference of (see
+    softmax_reverse_scale / rmsnorm_reverse_scales): where two terms of size s cancel to a
+    result far below s, no fp32 kernel can be closer than a few ulp of s."""
+    g = got.detach().double().cpu().numpy()
+    ref = np.asarray(ref, dtype=np.float64)
+    assert g.shape == ref.shape, f"{what}: shape {g.shape} vs {ref.shape}"
+    if g.size == 0:
+        return
+    both_nan = np.isnan(g) & np.isnan(ref)
+    fin = np.where(np.isfinite(ref), ref, 0.0)
+    if atol is not None:
+        bound = np.full_like(ref, atol)
+    else:
+        rtol = RTOL[dtype] if rtol is None else rtol
+        if rowwise and ref.ndim >= 2:
+            rms = np.sqrt((fin ** 2).mean(axis=-1, keepdims=True))
+        else:
+            rms = np.sqrt((fin ** 2).mean())
+        mag = np.maximum(np.abs(fin), rms)
+        if scale is not None:
+            mag = np.maximum(mag, np.asarray(scale, dtype=np.float64))
+        bound = rtol * mag + FLOOR[dtype]
+    with np.errstate(invalid="ignore"):
+        err = np.abs(g - ref)
+    bad = ~(err <= bound) & ~both_nan
+    if bad.any():
+        idx = np.unravel_index(np.argmax(np.where(bad, err / np.maximum(bound, 1e-300), 0)), ref.shape)
+        raise AssertionError(
+            f"{what}: {int(bad.sum())} of {ref.size} outside tolerance; worst at {idx}: "
+            f"got {g[idx]!r} ref {ref[idx]!r} err {err[idx]:.3e} bound {bound[idx]:.3e}")
+
+
+def softmax_reverse_scale(y, dy, dx_in=None, alpha=0.0):
+    """dx = y*dy - y*dot (+ alpha*old): size of the terms that cancel."""
+    y, dy = np.asarray(y, np.float64), np.asarray(dy, np.float64)
+    s = np.abs(y) * (np.abs(dy) + np.abs(y * dy).sum(axis=-1, keepdims=True))
+    if dx_in is not None:
+        s = s + abs(alpha) * np.abs(np.asarray(dx_in, np.float64))
+    return s
+
+
+def rmsnorm_reverse_scales(x, g, dy, eps, dx_in=None, dg_in=None, alpha=0.0):
+    """dx = r*dy*g - r^3*x*c: size of its two terms; dg = sum_i dy*x*r: sum of |terms|."""
+    x, g, dy = (np.asarray(a, np.float64) for a in (x, g, dy))
+    n = x.shape[-1]
+    r = 1.0 / np.sqrt((x * x).mean(axis=-1, keepdims=True) + eps)
+    c_abs = np.abs(dy * g * x).sum(axis=-1, keepdims=True) / n
+    sdx = r * (np.abs(dy * g) + np.abs(x) * r * r * c_abs)
+    sdg = np.abs(dy * x * r).sum(axis=0)
+    if dx_in is not None:
+        sdx = sdx + abs(alpha) * np.abs(np.asarray(dx_in, np.float64))
+    if dg_in is not None:
+        sdg = sdg + abs(alpha) * np.abs(np.asarray(dg_in, np.float64))
+    return sdx, sdg
+
+
+# ---------------------------------------------------------------- launcher wrappers
+
+def _call(stem, dtype, *args):
+    kernels, _ = lib()
+    ffi.invoke(getattr(kernels, stem), KEY[dtype], *args, ctx())
+
+
+def addition(a, b, c):
+    _call("addition", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(), a.numel())
+
+
+def hadamard(a, b, c):
+    _call("hadamard", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(), a.numel())
+
+
+def hadamard_reverse(a, b, c):
+    _call("hadamard_reverse", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(), a.numel())
+
+
+def selu(a, b):
+    _call("selu", a.dtype, a.data_ptr(), b.data_ptr(), a.numel())
+
+
+def selu_reverse(a_value, a_grads, b_grads):
+    _call("selu_reverse", a_value.dtype, a_value.data_ptr(), a_grads.data_ptr(), b_grads.data_ptr(),
+          a_value.numel())
+
+
+def fused(a, b, c, d, e):
+    _call("fused_selu_hadamard_add_add", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(),
+          d.data_ptr(), e.data_ptr(), a.numel())
+
+
+def fused_reverse(a, b, c, d, de, da, db, dc, dd, alpha=0.0):
+    _call("fused_selu_hadamard_add_add_reverse", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(),
+          d.data_ptr(), de.data_ptr(), da.data_ptr(), db.data_ptr(), dc.data_ptr(), dd.data_ptr(),
+          float(alpha), a.numel())
+
+
+def softmax(x, y):
+    m, n = x.shape
+    _call("softmax_ij_j", x.dtype, x.data_ptr(), y.data_ptr(), m, n)
+
+
+def softmax_reverse(y, dy, dx, alpha=0.0):
+    m, n = y.shape
+    _call("softmax_ij_j_reverse", y.dtype, y.data_ptr(), dy.data_ptr(), dx.data_ptr(), float(alpha), m, n)
+
+
+def rmsnorm(x, g, y, eps):
+    m, n = x.shape
+    _call("rmsnorm_ij_j", x.dtype, x.data_ptr(), g.data_ptr(), y.data_ptr(), float(eps), m, n)
+
+
+def rmsnorm_scratch(dtype, m, n):
+    kernels, _ = lib()
+    nbytes = int(kernels.mpRmsnormReverseScratchBytes(KEY[dtype], m, n))
+    return Guarded((max(nbytes, 1),), torch.uint8), nbytes
+
+
+def rmsnorm_reverse(x, g, dy, dx, dg, scratch, eps, alpha=0.0):
+    m, n = x.shape
+    _call("rmsnorm_ij_j_reverse", x.dtype, x.data_ptr(), g.data_ptr(), dy.data_ptr(), dx.data_ptr(),
+          dg.data_ptr(), scratch.data_ptr(), float(eps), float(alpha), m, n)
+
+
+def set_regime(r):
+    kernels, _ = lib()
+    kernels.mpSetRowRegime(int(r))

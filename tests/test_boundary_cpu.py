@@ -1,0 +1,75 @@
+"""CPU-side checks of the boundary: the libraries load, export every symbol the headers
+declare, and the generator's outputs are consistent. No compute call is made."""
+import ctypes
+import os
+import re
+
+import pytest
+
+from metaphor_amd import ffi, kernelgen
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_kernel_library_exports_every_declared_symbol():
+    lib = ctypes.CDLL(os.path.join(ffi.LIB_DIR, "libmp_kernels.so"))
+    protos = ffi.parse_declarations()
+    assert len(protos) >= 35
+    for _, name, _ in protos:
+        assert hasattr(lib, name), name
+
+
+def test_device_utils_exports_the_eleven_reference_names():
+    lib = ctypes.CDLL(os.path.join(ffi.LIB_DIR, "libdev_utils.so"))
+    names = [n for _, n, _ in ffi.parse_declarations(os.path.join(ROOT, "include", "device_utils.h"))]
+    assert names == ["mpInitDevice", "mpMemAlloc", "mpMemcpyHtoD", "mpMemcpyDtoH", "mpMemFree",
+                     "mpDeviceSynchronize", "mpStreamSynchronize", "mpInitStream", "mpDeinitStream",
+                     "mpCheckLastError", "mpDeviceTotalMemory"]
+    for n in names:
+        assert hasattr(lib, n), n
+
+
+def test_static_archive_holds_the_same_launchers():
+    import subprocess
+    out = subprocess.run(["nm", "--defined-only", os.path.join(ffi.LIB_DIR, "mp_kernels.a")],
+                         capture_output=True, text=True, check=True).stdout
+    defined = set(re.findall(r" T (launch_\w+|mp\w+)", out))
+    for _, name, _ in ffi.parse_declarations():
+        assert name in defined, name
+
+
+def test_dispatch_arrays_are_r16_r32_r64_in_scalar_tag_order():
+    table = kernelgen.kernel_table()
+    for stem, arr in table.items():
+        assert arr == [f"launch_{stem}_r16", f"launch_{stem}_r32", f"launch_{stem}_r64"]
+    kernels, _ = ffi.load()
+    assert set(table) == set(kernels.stems())
+    for stem in table:
+        assert len(getattr(kernels, stem)) == 3
+
+
+def test_every_launcher_takes_the_stream_context_last_and_returns_void():
+    for ret, name, args in ffi.parse_declarations():
+        if name.startswith("launch_"):
+            assert ret == "void"
+            assert args[-1][0] == "StreamContext"
+            assert all(t in ("const void*", "void*", "double", "len_t") for t, _ in args[:-1])
+
+
+def test_stream_context_layout_is_two_pointers_by_value():
+    assert ctypes.sizeof(ffi.StreamContext) == 16
+    assert ffi.StreamContext.hip_stream.offset == 0 and ffi.StreamContext.blas_handle.offset == 8
+
+
+def test_generated_header_is_current():
+    before = open(kernelgen.DECLS).read()
+    kernelgen.make_kernel_declarations()
+    assert open(kernelgen.DECLS).read() == before
+
+
+def test_config_rejects_non_gfx_architectures(tmp_path, monkeypatch):
+    cfg = tmp_path / "config.json"
+    cfg.write_text('{"gpu-architecture": "sm_89"}')
+    monkeypatch.setattr(kernelgen, "CONFIG", str(cfg))
+    with pytest.raises(ValueError):
+        kernelgen.load_config()

@@ -1,0 +1,398 @@
+"""GPU parity: every launcher, through the C-ABI, against the fp64 CPU oracle on the same
+seeded inputs, at sizes the oracle finishes in seconds. Buffers carry canaries; ragged,
+unaligned, aliased, empty and masked inputs are covered, and the softmax / RMSNorm launchers
+are driven through each row regime."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_lib as G
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float16, torch.float32, torch.float64]
+IDS = ["r16", "r32", "r64"]
+REGIMES = [0, 1, 2, 3, 4]  # auto, wave, block, wide, stream
+
+
+@pytest.fixture(autouse=True)
+def _auto_regime():
+    G.set_regime(0)
+    yield
+    G.set_regime(0)
+    torch.cuda.synchronize()
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# ------------------------------------------------------------------ elementwise
+
+EW_SIZES = [0, 1, 3, 8, 255, 1024, 4099, (1 << 20) + 5]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shift", [0, 1])
+def test_add_hadamard_and_reverse(dtype, shift):
+    r = rng(10)
+    for n in EW_SIZES:
+        G.say(f"add/hadamard dtype={dtype} n={n} shift={shift}")
+        a, b = G.dev(r.normal(0, 1, n), dtype, shift), G.dev(r.normal(0, 1, n), dtype, shift)
+        c = G.Guarded((n,), dtype, shift)
+        G.addition(a.t, b.t, c.t)
+        G.compare(c.t, O.addition(G.host(a.t), G.host(b.t)), dtype, f"addition n={n}", rowwise=False)
+        G.hadamard(a.t, b.t, c.t)
+        G.compare(c.t, O.hadamard(G.host(a.t), G.host(b.t)), dtype, f"hadamard n={n}", rowwise=False)
+        c0 = G.dev(r.normal(0, 1, n), dtype, shift)
+        before = G.host(c0.t).copy()
+        G.hadamard_reverse(a.t, b.t, c0.t)
+        G.compare(c0.t, O.hadamard_reverse(G.host(a.t), G.host(b.t), before), dtype,
+                  f"hadamard_reverse n={n}", rowwise=False)
+        for g in (a, b, c, c0):
+            g.check(f"elementwise n={n}")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_addition_in_place_as_the_reference_reverse_calls_it(dtype):
+    # src/ops/addition.zig:67-73: gx = gz + gx with the output aliasing the second input
+    r = rng(11)
+    n = 70001
+    gz, gx = G.dev(r.normal(0, 1, n), dtype), G.dev(r.normal(0, 1, n), dtype)
+    want = O.addition(G.host(gz.t), G.host(gx.t))
+    G.say(f"addition in place dtype={dtype}")
+    G.addition(gz.t, gx.t, gx.t)
+    G.compare(gx.t, want, dtype, "in-place addition", rowwise=False)
+    gx.check("in-place addition")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shift", [0, 1])
+def test_selu_forward_and_reverse(dtype, shift):
+    r = rng(12)
+    for n in EW_SIZES:
+        G.say(f"selu dtype={dtype} n={n} shift={shift}")
+        x = r.uniform(-9, 9, n)
+        x[: min(n, 6)] = [0.0, -0.0, 1e-4, -1e-4, -0.25, -0.2500001][: min(n, 6)]
+        a = G.dev(x, dtype, shift)
+        b = G.Guarded((n,), dtype, shift)
+        G.selu(a.t, b.t)
+        G.compare(b.t, O.selu(G.host(a.t)), dtype, f"selu n={n}", rowwise=False)
+        gb, ga = G.dev(r.normal(0, 1, n), dtype, shift), G.dev(r.normal(0, 1, n), dtype, shift)
+        before = G.host(ga.t).copy()
+        G.selu_reverse(a.t, ga.t, gb.t)
+        G.compare(ga.t, O.selu_reverse(G.host(a.t), G.host(gb.t), before), dtype,
+                  f"selu_reverse n={n}", rowwise=False)
+        for g in (a, b, ga, gb):
+            g.check(f"selu n={n}")
+
+
+def test_selu_relative_accuracy_near_zero_r32():
+    # the expm1 branch must keep relative accuracy where exp(x)-1 cancels
+    x = -np.logspace(-8, 0.5, 4000)
+    a = G.dev(x, torch.float32)
+    b = G.Guarded(a.t.shape, torch.float32)
+    G.say("selu near zero r32")
+    G.selu(a.t, b.t)
+    ref = O.selu(G.host(a.t))
+    got = b.t.double().cpu().numpy()
+    assert np.max(np.abs(got - ref) / np.abs(ref)) < 1e-6
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shift", [0, 1])
+def test_fused_chain_forward_and_reverse(dtype, shift):
+    r = rng(13)
+    for n in EW_SIZES:
+        G.say(f"fused dtype={dtype} n={n} shift={shift}")
+        ins = [G.dev(r.uniform(-2, 2, n), dtype, shift) for _ in range(4)]
+        de = G.dev(r.normal(0, 1, n), dtype, shift)
+        e = G.Guarded((n,), dtype, shift)
+        G.fused(*[g.t for g in ins], e.t)
+        hin = [G.host(g.t) for g in ins]
+        G.compare(e.t, O.fused_selu_hadamard_add_add(*hin), dtype, f"fused fwd n={n}", rowwise=False)
+        outs = [G.Guarded((n,), dtype, shift) for _ in range(4)]
+        G.fused_reverse(*[g.t for g in ins], de.t, *[g.t for g in outs], alpha=0.0)
+        refs = O.fused_selu_hadamard_add_add_reverse(*hin, G.host(de.t))
+        for name, g, ref in zip("abcd", outs, refs):
+            G.compare(g.t, ref, dtype, f"fused rev d{name} n={n}", rowwise=False)
+        if n:
+            assert torch.equal(outs[0].t, outs[1].t) and torch.equal(outs[2].t, outs[3].t)
+        # accumulate mode: out = val + alpha*old
+        olds = [G.dev(r.normal(0, 1, n), dtype, shift) for _ in range(4)]
+        hold = tuple(G.host(g.t).copy() for g in olds)
+        G.fused_reverse(*[g.t for g in ins], de.t, *[g.t for g in olds], alpha=1.0)
+        refs = O.fused_selu_hadamard_add_add_reverse(*hin, G.host(de.t), hold, alpha=1.0)
+        for name, g, ref in zip("abcd", olds, refs):
+            G.compare(g.t, ref, dtype, f"fused rev accumulate d{name} n={n}", rowwise=False)
+        for g in ins + outs + olds + [de, e]:
+            g.check(f"fused n={n}")
+
+
+# ------------------------------------------------------------------ softmax
+
+SOFTMAX_SHAPES = [(1, 1), (3, 7), (5, 64), (4, 65), (9, 256), (7, 1000), (256, 1024), (6, 2048),
+                  (3, 5000), (5, 8192), (2, 20000), (2, 50257), (1, 151936), (1030, 33)]
+
+
+def _softmax_inputs(r, m, n, dtype, masked):
+    x = r.normal(0, 2, (m, n))
+    if masked:
+        rows, cols = np.indices((m, n))
+        x[cols > (rows % max(n, 1))] = -np.inf
+    return x
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("regime", REGIMES)
+def test_softmax_forward_all_regimes(dtype, regime):
+    r = rng(20 + regime)
+    G.set_regime(regime)
+    for (m, n) in SOFTMAX_SHAPES:
+        for masked in (False, True):
+            G.say(f"softmax fwd dtype={dtype} regime={regime} shape=({m},{n}) masked={masked}")
+            x = G.dev(_softmax_inputs(r, m, n, dtype, masked), dtype)
+            y = G.Guarded((m, n), dtype)
+            G.softmax(x.t, y.t)
+            ref = O.softmax_ij_j(G.host(x.t))
+            G.compare(y.t, ref, dtype, f"softmax ({m},{n}) regime {regime}", atol=G.SOFTMAX_ATOL[dtype])
+            if masked:
+                assert bool((y.t[torch.isinf(x.t)] == 0).all()), "-inf must map to exactly 0"
+            x.check("softmax x")
+            y.check("softmax y")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("regime", [0, 4])
+def test_softmax_unaligned_bases_and_in_place(dtype, regime):
+    r = rng(30)
+    G.set_regime(regime)
+    for (m, n) in [(5, 100), (3, 1027), (2, 50257), (4, 4096)]:
+        for sx, sy in [(1, 1), (1, 0), (3, 2)]:
+            G.say(f"softmax unaligned dtype={dtype} regime={regime} shape=({m},{n}) shifts=({sx},{sy})")
+            x = G.dev(r.normal(0, 3, (m, n)), dtype, sx)
+            y = G.Guarded((m, n), dtype, sy)
+            G.softmax(x.t, y.t)
+            ref = O.softmax_ij_j(G.host(x.t))
+            G.compare(y.t, ref, dtype, f"softmax unaligned ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
+            x.check("x")
+            y.check("y")
+        x = G.dev(r.normal(0, 3, (m, n)), dtype)
+        ref = O.softmax_ij_j(G.host(x.t))
+        G.say(f"softmax in place dtype={dtype} shape=({m},{n})")
+        G.softmax(x.t, x.t)
+        G.compare(x.t, ref, dtype, f"softmax in place ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
+        x.check("in place")
+
+
+def test_softmax_vocabulary_spike_rows_r32():
+    # the sampling-path input: N(0,3) logits with +12 on one random column per row
+    r = rng(31)
+    for (m, n) in [(3, 151936), (4, 50257)]:
+        x = r.normal(0, 3, (m, n))
+        x[np.arange(m), r.integers(0, n, m)] += 12.0
+        xd = G.dev(x, torch.float32)
+        y = G.Guarded((m, n), torch.float32)
+        G.say(f"softmax vocabulary rows ({m},{n})")
+        G.softmax(xd.t, y.t)
+        G.compare(y.t, O.softmax_ij_j(G.host(xd.t)), torch.float32, f"vocab ({m},{n})", atol=1e-6)
+        y.check("vocab")
+
+
+def test_softmax_all_masked_row_is_nan_like_the_closed_form():
+    x = torch.full((2, 128), float("-inf"), device="cuda", dtype=torch.float32)
+    x[1, 5] = 0.0
+    y = torch.empty_like(x)
+    G.say("softmax all -inf row")
+    G.softmax(x, y)
+    assert bool(torch.isnan(y[0]).all())
+    assert float(y[1, 5]) == 1.0 and float(y[1].sum()) == 1.0
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("regime", REGIMES)
+def test_softmax_reverse_all_regimes(dtype, regime):
+    r = rng(40 + regime)
+    G.set_regime(regime)
+    for (m, n) in SOFTMAX_SHAPES:
+        for alpha in (0.0, 1.0, 0.5):
+            if alpha == 0.5 and n > 5000:
+                continue
+            G.say(f"softmax rev dtype={dtype} regime={regime} shape=({m},{n}) alpha={alpha}")
+            xs = _softmax_inputs(r, m, n, dtype, masked=(m % 2 == 0))
+            y64 = O.softmax_ij_j(xs)
+            y = G.dev(y64, dtype)
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dx = G.dev(r.normal(0, 1, (m, n)), dtype)
+            before = G.host(dx.t).copy()
+            G.softmax_reverse(y.t, dy.t, dx.t, alpha)
+            ref = O.softmax_ij_j_reverse(G.host(y.t), G.host(dy.t), before if alpha else None, alpha)
+            scale = G.softmax_reverse_scale(G.host(y.t), G.host(dy.t), before if alpha else None, alpha)
+            G.compare(dx.t, ref, dtype, f"softmax rev ({m},{n}) regime {regime} alpha {alpha}", scale=scale)
+            for g in (y, dy, dx):
+                g.check("softmax rev")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_softmax_reverse_unaligned(dtype):
+    r = rng(41)
+    for (m, n) in [(5, 100), (3, 1027), (2, 50257)]:
+        for shifts in [(1, 1, 1), (1, 0, 2)]:
+            G.say(f"softmax rev unaligned dtype={dtype} shape=({m},{n}) shifts={shifts}")
+            y = G.dev(O.softmax_ij_j(r.normal(0, 2, (m, n))), dtype, shifts[0])
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[1])
+            dx = G.Guarded((m, n), dtype, shifts[2])
+            G.softmax_reverse(y.t, dy.t, dx.t, 0.0)
+            ref = O.softmax_ij_j_reverse(G.host(y.t), G.host(dy.t))
+            G.compare(dx.t, ref, dtype, f"softmax rev unaligned ({m},{n})",
+                      scale=G.softmax_reverse_scale(G.host(y.t), G.host(dy.t)))
+            dx.check("dx")
+
+
+# ------------------------------------------------------------------ RMSNorm
+
+NORM_SHAPES = [(1, 1), (3, 7), (17, 64), (33, 256), (64, 4096), (5, 1000), (300, 1024), (3, 50257),
+               (2, 70001), (1025, 128), (40, 8192)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("regime", REGIMES)
+def test_rmsnorm_forward_all_regimes(dtype, regime):
+    r = rng(50 + regime)
+    G.set_regime(regime)
+    eps = 1e-6
+    for (m, n) in NORM_SHAPES:
+        G.say(f"rmsnorm fwd dtype={dtype} regime={regime} shape=({m},{n})")
+        x = G.dev(r.normal(0, 1, (m, n)), dtype)
+        g = G.dev(r.normal(1, 0.02, n), dtype)
+        y = G.Guarded((m, n), dtype)
+        G.rmsnorm(x.t, g.t, y.t, eps)
+        G.compare(y.t, O.rmsnorm_ij_j(G.host(x.t), G.host(g.t), eps), dtype, f"rmsnorm ({m},{n}) regime {regime}")
+        y.check("rmsnorm y")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rmsnorm_forward_unaligned_and_in_place(dtype):
+    r = rng(51)
+    eps = 1e-6
+    for (m, n) in [(5, 100), (3, 1027), (2, 50257), (4, 4096)]:
+        for sx, sg, sy in [(1, 0, 1), (1, 1, 0), (0, 1, 0)]:
+            G.say(f"rmsnorm unaligned dtype={dtype} shape=({m},{n}) shifts=({sx},{sg},{sy})")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype, sx)
+            g = G.dev(r.normal(1, 0.02, n), dtype, sg)
+            y = G.Guarded((m, n), dtype, sy)
+            G.rmsnorm(x.t, g.t, y.t, eps)
+            G.compare(y.t, O.rmsnorm_ij_j(G.host(x.t), G.host(g.t), eps), dtype, f"rmsnorm unaligned ({m},{n})")
+            y.check("y")
+        x = G.dev(r.normal(0, 1, (m, n)), dtype)
+        g = G.dev(r.normal(1, 0.02, n), dtype)
+        ref = O.rmsnorm_ij_j(G.host(x.t), G.host(g.t), eps)
+        G.rmsnorm(x.t, g.t, x.t, eps)
+        G.compare(x.t, ref, dtype, f"rmsnorm in place ({m},{n})")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("regime", REGIMES)
+def test_rmsnorm_reverse_all_regimes(dtype, regime):
+    r = rng(60 + regime)
+    G.set_regime(regime)
+    eps = 1e-6
+    for (m, n) in NORM_SHAPES:
+        for alpha in (0.0, 1.0):
+            G.say(f"rmsnorm rev dtype={dtype} regime={regime} shape=({m},{n}) alpha={alpha}")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype)
+            g = G.dev(r.normal(1, 0.02, n), dtype)
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dx = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dg = G.dev(r.normal(0, 1, n), dtype)
+            hdx, hdg = G.host(dx.t).copy(), G.host(dg.t).copy()
+            scratch, nbytes = G.rmsnorm_scratch(dtype, m, n)
+            G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, eps, alpha)
+            rdx, rdg = O.rmsnorm_ij_j_reverse(G.host(x.t), G.host(g.t), G.host(dy.t), eps,
+                                              hdx if alpha else None, hdg if alpha else None, alpha)
+            sdx, sdg = G.rmsnorm_reverse_scales(G.host(x.t), G.host(g.t), G.host(dy.t), eps,
+                                                hdx if alpha else None, hdg if alpha else None, alpha)
+            G.compare(dx.t, rdx, dtype, f"rmsnorm rev dx ({m},{n}) regime {regime} alpha {alpha}", scale=sdx)
+            G.compare(dg.t, rdg, dtype, f"rmsnorm rev dg ({m},{n}) regime {regime} alpha {alpha}",
+                      rowwise=False, scale=sdg)
+            for gd in (x, g, dy, dx, dg, scratch):
+                gd.check("rmsnorm rev")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rmsnorm_reverse_unaligned(dtype):
+    r = rng(61)
+    eps = 1e-6
+    for (m, n) in [(5, 100), (3, 1027), (4, 4096)]:
+        for shifts in [(1, 0, 1, 1), (0, 1, 0, 0)]:
+            G.say(f"rmsnorm rev unaligned dtype={dtype} shape=({m},{n}) shifts={shifts}")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[0])
+            g = G.dev(r.normal(1, 0.02, n), dtype, shifts[1])
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[2])
+            dx = G.Guarded((m, n), dtype, shifts[3])
+            dg = G.Guarded((n,), dtype)
+            scratch, _ = G.rmsnorm_scratch(dtype, m, n)
+            G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, eps, 0.0)
+            rdx, rdg = O.rmsnorm_ij_j_reverse(G.host(x.t), G.host(g.t), G.host(dy.t), eps)
+            sdx, sdg = G.rmsnorm_reverse_scales(G.host(x.t), G.host(g.t), G.host(dy.t), eps)
+            G.compare(dx.t, rdx, dtype, f"rmsnorm rev unaligned dx ({m},{n})", scale=sdx)
+            G.compare(dg.t, rdg, dtype, f"rmsnorm rev unaligned dg ({m},{n})", rowwise=False, scale=sdg)
+            for gd in (dx, dg, scratch):
+                gd.check("rmsnorm rev unaligned")
+
+
+def test_rmsnorm_reverse_is_deterministic():
+    r = rng(62)
+    m, n = 2048, 4096
+    x = G.dev(r.normal(0, 1, (m, n)), torch.float32)
+    g = G.dev(r.normal(1, 0.02, n), torch.float32)
+    dy = G.dev(r.normal(0, 1, (m, n)), torch.float32)
+    scratch, _ = G.rmsnorm_scratch(torch.float32, m, n)
+    outs = []
+    for rep in range(3):
+        dx = G.Guarded((m, n), torch.float32)
+        dg = G.Guarded((n,), torch.float32)
+        G.say(f"rmsnorm rev determinism rep {rep}")
+        G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, 1e-6, 0.0)
+        outs.append((dx.t.clone(), dg.t.clone()))
+    for dx, dg in outs[1:]:
+        assert torch.equal(dx, outs[0][0]) and torch.equal(dg, outs[0][1])
+
+
+# ------------------------------------------------------------------ streams
+
+def test_launchers_follow_the_stream_of_the_context():
+    kernels, utils = G.lib()
+    sc = utils.mpInitStream()
+    assert sc.blas_handle.ptr is None and sc.hip_stream.ptr
+    r = rng(70)
+    n = 1 << 20
+    a, b = G.dev(r.normal(0, 1, n), torch.float32), G.dev(r.normal(0, 1, n), torch.float32)
+    c = G.Guarded((n,), torch.float32)
+    torch.cuda.synchronize()
+    G.say("addition on an mpInitStream stream")
+    kernels.addition[1](a.t.data_ptr(), b.t.data_ptr(), c.t.data_ptr(), n, sc)
+    utils.mpStreamSynchronize(sc)
+    G.compare(c.t, O.addition(G.host(a.t), G.host(b.t)), torch.float32, "addition on own stream", rowwise=False)
+    utils.mpDeinitStream(sc)
+
+
+def test_device_utils_roundtrip():
+    kernels, utils = G.lib()
+    utils.mpInitDevice(0)
+    assert utils.mpDeviceTotalMemory(0) > (100 << 30)
+    sc = utils.mpInitStream()
+    src = np.arange(100003, dtype=np.float32)
+    dst = np.zeros_like(src)
+    G.say("mpMemAlloc / HtoD / DtoH / Free")
+    d = utils.mpMemAlloc(src.nbytes, sc)
+    assert d
+    utils.mpMemcpyHtoD(d, src.ctypes.data, src.nbytes, sc)
+    utils.mpMemcpyDtoH(dst.ctypes.data, d, src.nbytes, sc)  # returns with the bytes landed
+    assert np.array_equal(src, dst)
+    utils.mpMemFree(d, sc)
+    utils.mpStreamSynchronize(sc)
+    utils.mpDeviceSynchronize()
+    utils.mpCheckLastError()
+    utils.mpDeinitStream(sc)
