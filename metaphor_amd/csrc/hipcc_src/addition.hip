@@ -16,5 +16,5 @@ extern "C" void launch_addition_Scalar(
   StreamContext stream
 ) {
   const mp::EwPtrs<2, 1> ptrs{{a, b}, {c}};
-  mp::ew_launch<Scalar, 2, 1, 4>(ptrs, N, AdditionFn_Scalar{}, get_stream(stream));
+  mp::ew_launch<Scalar, 2, 1, 1>(ptrs, N, AdditionFn_Scalar{}, get_stream(stream));
 }

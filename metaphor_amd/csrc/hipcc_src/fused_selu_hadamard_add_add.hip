@@ -19,5 +19,5 @@ extern "C" void launch_fused_selu_hadamard_add_add_Scalar(
   StreamContext stream
 ) {
   const mp::EwPtrs<4, 1> ptrs{{a, b, c, d}, {e}};
-  mp::ew_launch<Scalar, 4, 1, 2>(ptrs, N, FusedSeluHadamardAddAddFn_Scalar{}, get_stream(stream));
+  mp::ew_launch<Scalar, 4, 1, 1>(ptrs, N, FusedSeluHadamardAddAddFn_Scalar{}, get_stream(stream));
 }

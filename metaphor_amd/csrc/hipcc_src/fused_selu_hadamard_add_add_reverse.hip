@@ -43,7 +43,7 @@ extern "C" void launch_fused_selu_hadamard_add_add_reverse_Scalar(
 ) {
   if (alpha == 0.0) {
     const mp::EwPtrs<5, 4> ptrs{{a, b, c, d, e_grads}, {a_grads, b_grads, c_grads, d_grads}};
-    mp::ew_launch<Scalar, 5, 4, 2>(ptrs, N, FusedReverseOverwriteFn_Scalar{}, get_stream(stream));
+    mp::ew_launch<Scalar, 5, 4, 1>(ptrs, N, FusedReverseOverwriteFn_Scalar{}, get_stream(stream));
   } else {
     const mp::EwPtrs<9, 4> ptrs{{a, b, c, d, e_grads, a_grads, b_grads, c_grads, d_grads},
                                 {a_grads, b_grads, c_grads, d_grads}};

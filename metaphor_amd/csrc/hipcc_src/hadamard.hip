@@ -15,5 +15,5 @@ extern "C" void launch_hadamard_Scalar(
   StreamContext stream
 ) {
   const mp::EwPtrs<2, 1> ptrs{{a, b}, {c}};
-  mp::ew_launch<Scalar, 2, 1, 4>(ptrs, N, HadamardFn_Scalar{}, get_stream(stream));
+  mp::ew_launch<Scalar, 2, 1, 1>(ptrs, N, HadamardFn_Scalar{}, get_stream(stream));
 }

@@ -16,5 +16,5 @@ extern "C" void launch_hadamard_reverse_Scalar(
   StreamContext stream
 ) {
   const mp::EwPtrs<3, 1> ptrs{{a, b, c}, {c}};
-  mp::ew_launch<Scalar, 3, 1, 2>(ptrs, N, HadamardReverseFn_Scalar{}, get_stream(stream));
+  mp::ew_launch<Scalar, 3, 1, 1>(ptrs, N, HadamardReverseFn_Scalar{}, get_stream(stream));
 }

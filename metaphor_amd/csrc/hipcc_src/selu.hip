@@ -16,5 +16,5 @@ extern "C" void launch_selu_Scalar(
   StreamContext stream
 ) {
   const mp::EwPtrs<1, 1> ptrs{{a}, {b}};
-  mp::ew_launch<Scalar, 1, 1, 4>(ptrs, N, SeluFn_Scalar{}, get_stream(stream));
+  mp::ew_launch<Scalar, 1, 1, 1>(ptrs, N, SeluFn_Scalar{}, get_stream(stream));
 }

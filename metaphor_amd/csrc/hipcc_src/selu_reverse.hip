@@ -17,5 +17,5 @@ extern "C" void launch_selu_reverse_Scalar(
   StreamContext stream
 ) {
   const mp::EwPtrs<3, 1> ptrs{{a_value, a_grads, b_grads}, {a_grads}};
-  mp::ew_launch<Scalar, 3, 1, 2>(ptrs, N, SeluReverseFn_Scalar{}, get_stream(stream));
+  mp::ew_launch<Scalar, 3, 1, 1>(ptrs, N, SeluReverseFn_Scalar{}, get_stream(stream));
 }

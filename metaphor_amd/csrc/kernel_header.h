@@ -292,7 +292,7 @@ template <class T, int W, int G, int NV, bool RAGGED> struct RowTile {
     for (int k = 0; k < NV; ++k) {
       const int p = k * G + lane;
       if (p < g.nvec) {
-        load_pack<T, W>(body + (size_t)p * W, v[k]);
+        load_pack_nt<T, W>(body + (size_t)p * W, v[k]); /* a resident row is read exactly once */
       } else {
 #pragma unroll
         for (int i = 0; i < W; ++i) v[k][i] = fill;

@@ -6,7 +6,7 @@
 
 // Bytes of caller-owned scratch that launch_rmsnorm_ij_j_reverse_<dtype> needs for an [m, n]
 // problem: one row of n accumulators (fp32 for r16/r32, fp64 for r64) per workgroup, at most
-// one workgroup per compute unit. dtype is the dispatch key 0 = r16, 1 = r32, 2 = r64
+// two workgroups per compute unit. dtype is the dispatch key 0 = r16, 1 = r32, 2 = r64
 // (the order of the reference's scalar.Tag, src/core/scalar.zig:35-40).
 extern "C" len_t mpRmsnormReverseScratchBytes(len_t dtype, len_t m, len_t n) {
   switch (dtype) {
@@ -17,10 +17,10 @@ extern "C" len_t mpRmsnormReverseScratchBytes(len_t dtype, len_t m, len_t n) {
   }
 }
 
-// Diagnostic: force the row regime of the softmax / RMSNorm launchers (0 auto, 1 wave,
-// 2 block, 3 wide, 4 stream). A regime that cannot hold a row falls through to the next wider
-// one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
+// Diagnostic: force the row regime of the softmax / RMSNorm launchers (0 auto; 1..5 = groups of
+// 64, 128, 256, 512, 1024 threads per row; 6 = streaming). A group that cannot hold a row falls
+// through to the next wider one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
 extern "C" void mpSetRowRegime(len_t regime) {
-  mp::require(regime <= mp::REGIME_STREAM, "mpSetRowRegime: regime must be 0..4");
+  mp::require(regime <= mp::REGIME_STREAM, "mpSetRowRegime: regime must be 0..6");
   mp::row_regime_override() = (int)regime;
 }

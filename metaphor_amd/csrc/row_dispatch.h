@@ -1,15 +1,15 @@
 /*
  * Row-regime selection shared by the softmax and RMSNorm launchers.
  *
- * A row of `packs` 128-bit packs is processed by a group of G threads, each holding NV packs
- * in registers between the reduction and the write, so the row is read from HBM once:
- *   wave   G = 64    one wavefront per row, four rows per 256-thread workgroup, cross-lane
- *                    reductions only (rows up to 4 KiB by default);
- *   block  G = 256   one workgroup per row, per-wave partials combined through LDS
- *                    (rows up to 32 KiB);
- *   wide   G = 1024  one 16-wave workgroup per row (rows up to 256 KiB);
- *   stream           rows too long for registers: an online first pass and a second pass that
- *                    re-reads the row (served by L2 / the memory-side cache where it fits).
+ * A row of `packs` 128-bit packs is processed by a group of G threads (G = 64 ... 1024), each
+ * holding NV packs in registers between the reduction and the write, so the row is read from
+ * HBM once. HBM streams fastest here with many small waves each moving one or two packs, so
+ * the plan takes the narrowest group that covers the row at a target NV (2 for softmax, 1 for
+ * RMSNorm) and only lets NV grow once the group is 1024 threads wide:
+ *   G = 64             one wavefront per row, cross-lane (DPP / permlane-swap) reductions only;
+ *   G = 128 ... 1024   per-wave partials combined through LDS with one barrier per reduction;
+ *   stream             rows too long for registers: an online first pass and a second pass that
+ *                      re-reads the row (served by L2 / the memory-side cache where it fits).
  * The reference has one regime only: a 32-lane warp per row striding the row with 4-byte loads
  * (src/cuda/nvcc_src/reduce_ij_i.cu:13-32).
  */
@@ -22,9 +22,11 @@
 
 namespace mp {
 
-enum RowRegime { REGIME_AUTO = 0, REGIME_WAVE = 1, REGIME_BLOCK = 2, REGIME_WIDE = 3, REGIME_STREAM = 4 };
+/* 0 = automatic; 1..5 force G = 64, 128, 256, 512, 1024; 6 forces the streaming kernels. */
+enum RowRegime { REGIME_AUTO = 0, REGIME_G64 = 1, REGIME_G128 = 2, REGIME_G256 = 3, REGIME_G512 = 4,
+                 REGIME_G1024 = 5, REGIME_STREAM = 6 };
 
-/* Diagnostic override set through mpSetRowRegime (device_utils); AUTO in normal use. */
+/* Diagnostic override set through mpSetRowRegime; AUTO in normal use. */
 inline int& row_regime_override() {
   static int regime = REGIME_AUTO;
   return regime;
@@ -45,17 +47,23 @@ struct RowPlan {
   int NV;  /* packs per thread */
 };
 
-/* Default regime limits, in packs per thread: a wave takes rows up to 4 KiB, a 256-thread
- * group up to 32 KiB, a 1024-thread group up to 256 KiB, each clipped to max_nv. */
-inline RowPlan plan_row(size_t packs, int max_nv) {
-  static const int group_of[] = {0, 64, 256, 1024};
-  static const int auto_cap[] = {0, 4, 8, 16};
+/* nv_target: packs per thread the automatic plan aims for before it widens the group. */
+inline RowPlan plan_row(size_t packs, int max_nv, int nv_target) {
+  static const int group_of[] = {0, 64, 128, 256, 512, 1024};
   const int forced = row_regime_override();
   if (forced == REGIME_STREAM) return RowPlan{0, 0};
-  /* a forced regime that cannot hold the row moves on to the next wider one */
-  for (int r = (forced == REGIME_AUTO ? REGIME_WAVE : forced); r <= REGIME_WIDE; ++r) {
-    const int cap = forced == REGIME_AUTO && auto_cap[r] < max_nv ? auto_cap[r] : max_nv;
-    const int nv = packs_per_thread(packs, group_of[r], cap);
+  if (forced == REGIME_AUTO) {
+    const int want = nv_target < max_nv ? nv_target : max_nv;
+    for (int r = REGIME_G64; r <= REGIME_G1024; ++r) {
+      const int nv = packs_per_thread(packs, group_of[r], want);
+      if (nv) return RowPlan{group_of[r], nv};
+    }
+    const int nv = packs_per_thread(packs, 1024, max_nv);
+    return nv ? RowPlan{1024, nv} : RowPlan{0, 0};
+  }
+  /* a forced group that cannot hold the row moves on to the next wider one */
+  for (int r = forced; r <= REGIME_G1024; ++r) {
+    const int nv = packs_per_thread(packs, group_of[r], max_nv);
     if (nv) return RowPlan{group_of[r], nv};
   }
   return RowPlan{0, 0};
@@ -70,7 +78,9 @@ template <int MAXNV, class F> inline bool for_row_plan(const RowPlan& plan, F&& 
 #define MP_PLAN_GROUP(G_) \
   MP_PLAN_CASE(G_, 1) MP_PLAN_CASE(G_, 2) MP_PLAN_CASE(G_, 4) MP_PLAN_CASE(G_, 8) MP_PLAN_CASE(G_, 16)
   MP_PLAN_GROUP(64)
+  MP_PLAN_GROUP(128)
   MP_PLAN_GROUP(256)
+  MP_PLAN_GROUP(512)
   MP_PLAN_GROUP(1024)
 #undef MP_PLAN_GROUP
 #undef MP_PLAN_CASE
@@ -79,13 +89,9 @@ template <int MAXNV, class F> inline bool for_row_plan(const RowPlan& plan, F&& 
 
 constexpr int STREAM_THREADS = 1024;
 
-template <int G> constexpr int block_threads() { return G < 256 ? 256 : G; }
-
-inline unsigned row_grid(size_t m, int G) {
-  const size_t rows_per_block = G < 256 ? 256 / G : 1;
-  const size_t blocks = (m + rows_per_block - 1) / rows_per_block;
-  require(blocks < 0x7fffffffull, "row launch: too many rows for one grid");
-  return (unsigned)blocks;
+inline unsigned row_grid(size_t m) {
+  require(m < 0x7fffffffull, "row launch: too many rows for one grid");
+  return (unsigned)m;
 }
 
 }  // namespace mp

@@ -332,23 +332,34 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
   }
 }
 
-/* dg_j = sum over partial rows (fixed order, fp64) + alpha * dg_j. 64 columns per workgroup,
- * 16 waves split the partial rows. */
+/* dg_j = sum over partial rows (fixed order, fp64) + alpha * dg_j. A workgroup owns 32 columns;
+ * its 32 half-wave slices split the partial rows and keep eight loads in flight each. */
+constexpr int FINISH_COLS = 32, FINISH_SLICES = 32;
 template <class T>
-__global__ __launch_bounds__(1024) void rmsnorm_dgain_finish(
+__global__ __launch_bounds__(FINISH_COLS * FINISH_SLICES) void rmsnorm_dgain_finish(
     const typename precision<T>::type* partials, T* dg, double alpha, int rows, size_t n) {
-  __shared__ double part[16][WAVE];
-  const int lane = threadIdx.x & (WAVE - 1), w = threadIdx.x / WAVE;
-  const size_t col = (size_t)blockIdx.x * WAVE + lane;
+  using P = typename precision<T>::type;
+  __shared__ double part[FINISH_SLICES][FINISH_COLS + 1];
+  const int c = threadIdx.x % FINISH_COLS, slice = threadIdx.x / FINISH_COLS;
+  const size_t col = (size_t)blockIdx.x * FINISH_COLS + c;
   double s = 0.0;
-  if (col < n)
-    for (int p = w; p < rows; p += 16) s += (double)partials[(size_t)p * n + col];
-  part[w][lane] = s;
+  if (col < n) {
+    int p = slice;
+    for (; p + 7 * FINISH_SLICES < rows; p += 8 * FINISH_SLICES) {
+      P v[8];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) v[u] = partials[(size_t)(p + u * FINISH_SLICES) * n + col];
+#pragma unroll
+      for (int u = 0; u < 8; ++u) s += (double)v[u];
+    }
+    for (; p < rows; p += FINISH_SLICES) s += (double)partials[(size_t)p * n + col];
+  }
+  part[slice][c] = s;
   __syncthreads();
-  if (w == 0 && col < n) {
+  if (slice == 0 && col < n) {
     double t = 0.0;
 #pragma unroll
-    for (int i = 0; i < 16; ++i) t += part[i][lane];
+    for (int i = 0; i < FINISH_SLICES; ++i) t += part[i][c];
     if (alpha != 0.0) t += alpha * (double)dg[col];
     dg[col] = (T)t;
   }
@@ -356,10 +367,10 @@ __global__ __launch_bounds__(1024) void rmsnorm_dgain_finish(
 
 /* ------------------------------------------------------------------ host dispatch */
 
-/* Partial rows the reverse may write: one per workgroup, at most one workgroup per CU. */
+/* Partial rows the reverse may write: one per workgroup, at most two workgroups per CU. */
 inline size_t rmsnorm_reverse_partial_rows(size_t m) {
-  const size_t cus = (size_t)compute_units();
-  return m < cus ? (m ? m : 1) : cus;
+  const size_t cap = (size_t)compute_units() * 2;
+  return m < cap ? (m ? m : 1) : cap;
 }
 
 template <class T>
@@ -383,7 +394,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, double eps, size_t 
   }
   const bool ragged = !(aligned16(x) && aligned16(gain) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV);
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 1);
   const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
@@ -408,7 +419,7 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
   /* four register arrays per thread (x, dy, gain, dg sums): 16 registers each when packed,
    * 8 elements each on the element-wise path */
   constexpr int MAXNV = W == 1 ? 8 : max_nv_for<T>(16);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV);
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 1);
   const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     rows = (unsigned)(need < max_rows ? need : max_rows);
@@ -423,8 +434,8 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
     else rmsnorm_rev_stream<T, W, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
   }
   MP_CHECK_LAUNCH();
-  const unsigned fin = (unsigned)((n + WAVE - 1) / WAVE);
-  rmsnorm_dgain_finish<T><<<dim3(fin), dim3(1024), 0, stream>>>(partials, dg, alpha, (int)rows, n);
+  const unsigned fin = (unsigned)((n + FINISH_COLS - 1) / FINISH_COLS);
+  rmsnorm_dgain_finish<T><<<dim3(fin), dim3(FINISH_COLS * FINISH_SLICES), 0, stream>>>(partials, dg, alpha, (int)rows, n);
   MP_CHECK_LAUNCH();
 }
 

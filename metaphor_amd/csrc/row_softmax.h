@@ -26,15 +26,13 @@ namespace mp {
 /* ------------------------------------------------------------------ resident forward */
 
 template <class T, int W, int G, int NV, bool RAGGED>
-__global__ __launch_bounds__(block_threads<G>()) void softmax_fwd_resident(
+__global__ __launch_bounds__(G) void softmax_fwd_resident(
     const T* x, T* y, size_t m, size_t n) {
   using P = typename precision<T>::type;
-  constexpr int RPB = block_threads<G>() / G;
   __shared__ P slots[2][G / WAVE];
 
-  const int sub = threadIdx.x / G, lane = threadIdx.x % G;
-  const size_t row = (size_t)blockIdx.x * RPB + sub;
-  if (row >= m) return; /* whole waves leave; groups wider than a wave own one row per block */
+  const int lane = threadIdx.x; /* one row per workgroup of G threads */
+  const size_t row = blockIdx.x;
 
   const T* xr = x + row * n;
   const RowGeom<T, W> g(xr, n, RAGGED);
@@ -58,15 +56,13 @@ __global__ __launch_bounds__(block_threads<G>()) void softmax_fwd_resident(
 /* ------------------------------------------------------------------ resident reverse */
 
 template <class T, int W, int G, int NV, bool RAGGED, bool BLEND>
-__global__ __launch_bounds__(block_threads<G>()) void softmax_rev_resident(
+__global__ __launch_bounds__(G) void softmax_rev_resident(
     const T* y, const T* dy, T* dx, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
-  constexpr int RPB = block_threads<G>() / G;
   __shared__ P slots[G / WAVE];
 
-  const int sub = threadIdx.x / G, lane = threadIdx.x % G;
-  const size_t row = (size_t)blockIdx.x * RPB + sub;
-  if (row >= m) return;
+  const int lane = threadIdx.x;
+  const size_t row = blockIdx.x;
 
   const T* yr = y + row * n;
   const T* gr = dy + row * n;
@@ -311,9 +307,9 @@ inline void softmax_forward(const T* x, T* y, size_t m, size_t n, hipStream_t st
   }
   const bool ragged = !(aligned16(x) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(64);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV);
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 2);
   const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
-    const dim3 grid(row_grid(m, G)), block(block_threads<G>());
+    const dim3 grid(row_grid(m)), block(G);
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n);
     else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n);
   });
@@ -340,9 +336,9 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, double alpha, size_t
   }
   const bool ragged = !(aligned16(y) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV);
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 2);
   const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
-    const dim3 grid(row_grid(m, G)), block(block_threads<G>());
+    const dim3 grid(row_grid(m)), block(G);
     if (ragged) {
       if (blend) softmax_rev_resident<T, W, G, NV, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
       else softmax_rev_resident<T, W, G, NV, true, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);

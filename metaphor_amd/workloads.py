@@ -1,0 +1,239 @@
+"""The seeded synthetic workloads this path is measured and checked on, and thin Python
+wrappers that enqueue the launchers of the C-ABI on torch-owned device memory.
+
+torch is plumbing here (device buffers, the current stream, the seeded generators); every
+computation is one of the ``launch_*`` entry points of include/kernel_decls.h.
+
+Workloads (N(mu, s) = mean mu, standard deviation s; seed 0 unless a set index is added):
+  cfg1  softmax forward, r32, [256, 1024], inputs 4*N(0,1)
+  cfg2  RMSNorm forward + reverse, r32, X and dY [8192, 4096] ~ N(0,1), gain ~ N(1, 0.02), eps 1e-6
+  cfg3  softmax forward + reverse, r16, [8*32*2048, 2048] ~ N(0,2) with -inf strictly above the
+        diagonal of every 2048-row block, dY ~ N(0,1)
+  cfg4  fused e = selu((a+b)*(c+d)) forward + reverse, r32, flat 2^28, inputs U(-2,2), de ~ N(0,1)
+  cfg5a softmax forward, r32, [512, 151936], N(0,3) + 12 on one random column per row
+  cfg5b softmax forward, r32, [2048, 50257], same distribution
+"""
+import torch
+
+from . import ffi
+
+KEY = {torch.float16: ffi.R16, torch.float32: ffi.R32, torch.float64: ffi.R64}
+DTYPE_NAME = {torch.float16: "r16", torch.float32: "r32", torch.float64: "r64"}
+
+
+def _ctx():
+    return ffi.StreamContext.from_handle(torch.cuda.current_stream().cuda_stream)
+
+
+def _launch(stem, dtype, *args):
+    kernels, _ = ffi.load()
+    ffi.invoke(getattr(kernels, stem), KEY[dtype], *args, _ctx())
+
+
+# ------------------------------------------------------------------ launch wrappers
+
+def softmax_forward(x, y):
+    m, n = x.shape
+    _launch("softmax_ij_j", x.dtype, x.data_ptr(), y.data_ptr(), m, n)
+
+
+def softmax_reverse(y, dy, dx, alpha=0.0):
+    m, n = y.shape
+    _launch("softmax_ij_j_reverse", y.dtype, y.data_ptr(), dy.data_ptr(), dx.data_ptr(), float(alpha), m, n)
+
+
+def rmsnorm_forward(x, gain, y, eps):
+    m, n = x.shape
+    _launch("rmsnorm_ij_j", x.dtype, x.data_ptr(), gain.data_ptr(), y.data_ptr(), float(eps), m, n)
+
+
+def rmsnorm_reverse_scratch(dtype, m, n):
+    kernels, _ = ffi.load()
+    nbytes = int(kernels.mpRmsnormReverseScratchBytes(KEY[dtype], m, n))
+    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device="cuda")
+
+
+def rmsnorm_reverse(x, gain, dy, dx, dgain, scratch, eps, alpha=0.0):
+    m, n = x.shape
+    _launch("rmsnorm_ij_j_reverse", x.dtype, x.data_ptr(), gain.data_ptr(), dy.data_ptr(), dx.data_ptr(),
+            dgain.data_ptr(), scratch.data_ptr(), float(eps), float(alpha), m, n)
+
+
+def fused_forward(a, b, c, d, e):
+    _launch("fused_selu_hadamard_add_add", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(),
+            d.data_ptr(), e.data_ptr(), a.numel())
+
+
+def fused_reverse(a, b, c, d, de, da, db, dc, dd, alpha=0.0):
+    _launch("fused_selu_hadamard_add_add_reverse", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(),
+            d.data_ptr(), de.data_ptr(), da.data_ptr(), db.data_ptr(), dc.data_ptr(), dd.data_ptr(),
+            float(alpha), a.numel())
+
+
+# ------------------------------------------------------------------ workload definitions
+
+def _gen(seed):
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    return g
+
+
+class Workload:
+    """One buffer set of one config. `forward()` / `reverse()` enqueue the launchers;
+    `fwd_bytes` / `rev_bytes` are the algorithmic HBM bytes of one call (each input read once,
+    each output written once); `rows` is rows (elements for cfg4) per call."""
+    name = ""
+    dtype = torch.float32
+    has_reverse = True
+
+    def forward(self):
+        raise NotImplementedError
+
+    def reverse(self):
+        raise NotImplementedError
+
+
+class Cfg1(Workload):
+    name, dtype, has_reverse = "cfg1", torch.float32, False
+    shape = (256, 1024)
+
+    def __init__(self, seed=0, shape=None):
+        self.shape = shape or self.shape
+        g = _gen(seed)
+        self.x = 4.0 * torch.randn(self.shape, generator=g, device="cuda", dtype=torch.float32)
+        self.y = torch.empty_like(self.x)
+        self.rows = self.shape[0]
+        self.fwd_bytes = 2 * self.x.numel() * 4
+        self.rev_bytes = 0
+
+    def forward(self):
+        softmax_forward(self.x, self.y)
+
+
+class Cfg2(Workload):
+    name, dtype = "cfg2", torch.float32
+    shape = (8192, 4096)
+    eps = 1e-6
+
+    def __init__(self, seed=0, shape=None):
+        self.shape = shape or self.shape
+        m, n = self.shape
+        g = _gen(seed)
+        self.x = torch.randn(self.shape, generator=g, device="cuda", dtype=torch.float32)
+        self.gain = 1.0 + 0.02 * torch.randn((n,), generator=g, device="cuda", dtype=torch.float32)
+        self.dy = torch.randn(self.shape, generator=g, device="cuda", dtype=torch.float32)
+        self.y = torch.empty_like(self.x)
+        self.dx = torch.empty_like(self.x)
+        self.dgain = torch.empty_like(self.gain)
+        self.scratch = rmsnorm_reverse_scratch(torch.float32, m, n)
+        self.rows = m
+        self.fwd_bytes = 2 * m * n * 4
+        self.rev_bytes = 3 * m * n * 4
+
+    def forward(self):
+        rmsnorm_forward(self.x, self.gain, self.y, self.eps)
+
+    def reverse(self):
+        rmsnorm_reverse(self.x, self.gain, self.dy, self.dx, self.dgain, self.scratch, self.eps, 0.0)
+
+
+class Cfg3(Workload):
+    name, dtype = "cfg3", torch.float16
+    shape = (8 * 32 * 2048, 2048)
+    block = 2048
+
+    def __init__(self, seed=0, shape=None, block=None):
+        self.shape = shape or self.shape
+        self.block = block or self.block
+        m, n = self.shape
+        g = _gen(seed)
+        self.x = torch.empty(self.shape, device="cuda", dtype=torch.float16)
+        self.dy = torch.empty(self.shape, device="cuda", dtype=torch.float16)
+        cols = torch.arange(n, device="cuda").view(1, n)
+        step = min(m, 1 << 15)
+        for lo in range(0, m, step):  # chunked so the fp32 staging stays small
+            hi = min(m, lo + step)
+            t = 2.0 * torch.randn((hi - lo, n), generator=g, device="cuda", dtype=torch.float32)
+            rows = (torch.arange(lo, hi, device="cuda") % self.block).view(-1, 1)
+            t.masked_fill_(cols > rows, float("-inf"))
+            self.x[lo:hi] = t.to(torch.float16)
+            self.dy[lo:hi] = torch.randn((hi - lo, n), generator=g, device="cuda", dtype=torch.float32).to(torch.float16)
+        self.y = torch.empty_like(self.x)
+        self.dx = torch.empty_like(self.x)
+        self.rows = m
+        self.fwd_bytes = 2 * m * n * 2
+        self.rev_bytes = 3 * m * n * 2
+
+    def forward(self):
+        softmax_forward(self.x, self.y)
+
+    def reverse(self):
+        # consumes the forward output of this set
+        softmax_reverse(self.y, self.dy, self.dx, 0.0)
+
+
+class Cfg4(Workload):
+    name, dtype = "cfg4", torch.float32
+    n = 1 << 28
+
+    def __init__(self, seed=0, n=None):
+        self.n = n or self.n
+        g = _gen(seed)
+
+        def unif():
+            return torch.rand((self.n,), generator=g, device="cuda", dtype=torch.float32).mul_(4.0).sub_(2.0)
+
+        self.a, self.b, self.c, self.d = unif(), unif(), unif(), unif()
+        self.de = torch.randn((self.n,), generator=g, device="cuda", dtype=torch.float32)
+        self.e = torch.empty_like(self.a)
+        self.da, self.db, self.dc, self.dd = (torch.empty_like(self.a) for _ in range(4))
+        self.rows = self.n
+        self.fwd_bytes = 20 * self.n
+        self.rev_bytes = 36 * self.n
+
+    def forward(self):
+        fused_forward(self.a, self.b, self.c, self.d, self.e)
+
+    def reverse(self):
+        fused_reverse(self.a, self.b, self.c, self.d, self.de, self.da, self.db, self.dc, self.dd, 0.0)
+
+
+class _Vocab(Workload):
+    dtype, has_reverse = torch.float32, False
+
+    def __init__(self, seed=0, shape=None):
+        self.shape = shape or self.shape
+        m, n = self.shape
+        g = _gen(seed)
+        self.x = 3.0 * torch.randn(self.shape, generator=g, device="cuda", dtype=torch.float32)
+        spike = torch.randint(0, n, (m,), generator=g, device="cuda")
+        self.x[torch.arange(m, device="cuda"), spike] += 12.0
+        self.y = torch.empty_like(self.x)
+        self.rows = m
+        self.fwd_bytes = 2 * m * n * 4
+        self.rev_bytes = 0
+
+    def forward(self):
+        softmax_forward(self.x, self.y)
+
+
+class Cfg5a(_Vocab):
+    name = "cfg5a"
+    shape = (512, 151936)
+
+
+class Cfg5b(_Vocab):
+    name = "cfg5b"
+    shape = (2048, 50257)
+
+
+WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b)}
+
+DESCRIPTION = {
+    "cfg1": "softmax fwd r32 [256,1024]",
+    "cfg2": "RMSNorm fwd+rev r32 [8192,4096], gain [4096], eps 1e-6",
+    "cfg3": "causal attention-score softmax fwd+rev r16 [524288,2048]",
+    "cfg4": "fused selu((a+b)*(c+d)) fwd+rev r32 flat 2^28",
+    "cfg5a": "vocabulary softmax fwd r32 [512,151936]",
+    "cfg5b": "vocabulary softmax fwd r32 [2048,50257]",
+}

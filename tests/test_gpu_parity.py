@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 DTYPES = [torch.float16, torch.float32, torch.float64]
 IDS = ["r16", "r32", "r64"]
-REGIMES = [0, 1, 2, 3, 4]  # auto, wave, block, wide, stream
+REGIMES = [0, 1, 2, 3, 4, 5, 6]  # auto, G = 64/128/256/512/1024, stream
 
 
 @pytest.fixture(autouse=True)
@@ -164,7 +164,7 @@ def test_softmax_forward_all_regimes(dtype, regime):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
-@pytest.mark.parametrize("regime", [0, 4])
+@pytest.mark.parametrize("regime", [0, 6])
 def test_softmax_unaligned_bases_and_in_place(dtype, regime):
     r = rng(30)
     G.set_regime(regime)
