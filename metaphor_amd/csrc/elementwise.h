@@ -21,9 +21,17 @@
 namespace mp {
 
 template <int NIN, int NOUT> struct EwPtrs {
-  const void* in[NIN];
+  const void* in[NIN > 0 ? NIN : 1]; /* generators (fill, sequence) have no input stream */
   void* out[NOUT];
 };
+
+/* A functor that declares `static constexpr bool needs_index = true` is also handed the
+ * element's flat index: apply(in, out, index). */
+template <class F, class P, int NIN, int NOUT>
+__device__ __forceinline__ void ew_apply(const F& f, const P (&a)[NIN > 0 ? NIN : 1], P (&r)[NOUT], size_t index) {
+  if constexpr (requires { F::needs_index; }) f.apply(a, r, index);
+  else f.apply(a, r);
+}
 
 /* One wavefront per workgroup and one pack per stream per lane measured fastest on MI355X for
  * pure streaming (larger workgroups or deeper unrolling lose 3-8 % of HBM bandwidth). */
@@ -33,10 +41,11 @@ constexpr int EW_BLOCK = 64;
 template <class T, int W, int NIN, int NOUT, int UNROLL, class F>
 __global__ __launch_bounds__(EW_BLOCK) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, size_t n, F f) {
   using P = typename precision<T>::type;
+  constexpr int NA = NIN > 0 ? NIN : 1;
   const size_t npacks = n / W;
   const size_t base = (size_t)blockIdx.x * (EW_BLOCK * UNROLL) + threadIdx.x;
 
-  P in[UNROLL][NIN][W];
+  P in[UNROLL][NA][W];
 #pragma unroll
   for (int u = 0; u < UNROLL; ++u) {
     const size_t p = base + (size_t)u * EW_BLOCK;
@@ -53,10 +62,10 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, si
       P out[NOUT][W];
 #pragma unroll
       for (int i = 0; i < W; ++i) {
-        P a[NIN], r[NOUT];
+        P a[NA], r[NOUT];
 #pragma unroll
         for (int s = 0; s < NIN; ++s) a[s] = in[u][s][i];
-        f.apply(a, r);
+        ew_apply<F, P, NIN, NOUT>(f, a, r, p * W + i);
 #pragma unroll
         for (int s = 0; s < NOUT; ++s) out[s][i] = r[s];
       }
@@ -70,10 +79,10 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, si
   if (W > 1 && blockIdx.x == 0) {
     const size_t e = npacks * W + threadIdx.x;
     if (e < n) {
-      P a[NIN], r[NOUT];
+      P a[NA], r[NOUT];
 #pragma unroll
       for (int s = 0; s < NIN; ++s) a[s] = (P) static_cast<const T*>(ptrs.in[s])[e];
-      f.apply(a, r);
+      ew_apply<F, P, NIN, NOUT>(f, a, r, e);
 #pragma unroll
       for (int s = 0; s < NOUT; ++s) static_cast<T*>(ptrs.out[s])[e] = (T)r[s];
     }

@@ -227,7 +227,25 @@ class Cfg5b(_Vocab):
     shape = (2048, 50257)
 
 
-WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b)}
+class Copy(Workload):
+    """Plain copy of known size (1 GiB in, 1 GiB out): the calibration run for the HBM traffic
+    counters and the practical bandwidth ceiling next to which the other figures are read."""
+    name, dtype, has_reverse = "copy", torch.float32, False
+    n = 1 << 28
+
+    def __init__(self, seed=0, n=None):
+        self.n = n or self.n
+        self.x = torch.randn((self.n,), generator=_gen(seed), device="cuda", dtype=torch.float32)
+        self.y = torch.empty_like(self.x)
+        self.rows = self.n
+        self.fwd_bytes = 8 * self.n
+        self.rev_bytes = 0
+
+    def forward(self):
+        _launch("copy", self.x.dtype, self.x.data_ptr(), self.y.data_ptr(), self.n)
+
+
+WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b, Copy)}
 
 DESCRIPTION = {
     "cfg1": "softmax fwd r32 [256,1024]",
@@ -236,4 +254,5 @@ DESCRIPTION = {
     "cfg4": "fused selu((a+b)*(c+d)) fwd+rev r32 flat 2^28",
     "cfg5a": "vocabulary softmax fwd r32 [512,151936]",
     "cfg5b": "vocabulary softmax fwd r32 [2048,50257]",
+    "copy": "plain copy r32 flat 2^28 (calibration)",
 }

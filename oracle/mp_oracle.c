@@ -14,6 +14,16 @@
  *   oracle_addition          src/cuda/nvcc_src/addition.cu:12           c = a + b
  *   oracle_hadamard          src/cuda/nvcc_src/hadamard.cu:12           c = a * b
  *   oracle_hadamard_reverse  src/cuda/nvcc_src/hadamard_reverse.cu:12   c += a * b
+ *   oracle_subtraction       src/cuda/nvcc_src/subtraction.cu:12        c = a - b
+ *   oracle_negate            src/cuda/nvcc_src/negate.cu:11             b = -a
+ *   oracle_relu / _reverse   src/cuda/nvcc_src/relu.cu:11-12, relu_reverse.cu:12-14   (a >= 0) convention
+ *   oracle_stepwise          the step function (a >= 0) ? 1 : 0 that src/ops/relu.zig:54-57 needs as the
+ *                            derivative of relu (the body of stepwise.cu:11-12 is a copy of relu)
+ *   oracle_dilate / _reverse src/cuda/nvcc_src/dilate.cu:12, dilate_reverse.cu:12     c = a*v ; b += a*v
+ *   oracle_translate         src/cuda/nvcc_src/translate.cu:12          c = a + v
+ *   oracle_fill, _sequence   src/cuda/nvcc_src/fill.cu:11, sequence.cu:13             a = v ; a_i = init + step*i
+ *   oracle_copy              src/cuda/nvcc_src/copy.cu:19-29            dst = src
+ *                            Scalars are narrowed to the storage type first, as the reference launchers do.
  *   oracle_reduce_ij_i       src/cuda/nvcc_src/reduce_ij_i.cu:20-32     dst_i = sum_j + alpha*dst_i
  *   oracle_reduce_ij_j       src/cuda/nvcc_src/reduce_ij_j.cu:10-44     dst_j = sum_i + alpha*dst_j (the intent; the
  *                                                                       reference body mis-indexes dst, :42-43)
@@ -102,6 +112,75 @@ void oracle_hadamard_reverse(int key, const void* a, const void* b, const void* 
 #pragma omp parallel for schedule(static)
   for (size_t i = 0; i < N; ++i)
     c_out[i] = (c_in ? ld(key, c_in, i) : 0.0) + ld(key, a, i) * ld(key, b, i);
+}
+
+/* value rounded to the storage type of the dtype key */
+static double narrow(int key, double v) {
+  switch (key) {
+    case 0: return half_bits_to_double(oracle_double_to_half_bits(v));
+    case 1: return (double)(float)v;
+    default: return v;
+  }
+}
+
+void oracle_subtraction(int key, const void* a, const void* b, double* c, size_t N) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < N; ++i) c[i] = ld(key, a, i) - ld(key, b, i);
+}
+
+void oracle_negate(int key, const void* a, double* b, size_t N) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < N; ++i) b[i] = -ld(key, a, i);
+}
+
+void oracle_relu(int key, const void* a, double* b, size_t N) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < N; ++i) { const double v = ld(key, a, i); b[i] = v >= 0.0 ? v : 0.0; }
+}
+
+void oracle_relu_reverse(int key, const void* a_value, const void* a_grads_in, const void* b_grads,
+                         double* a_grads_out, size_t N) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < N; ++i)
+    a_grads_out[i] = (a_grads_in ? ld(key, a_grads_in, i) : 0.0) +
+                     ld(key, b_grads, i) * (ld(key, a_value, i) >= 0.0 ? 1.0 : 0.0);
+}
+
+void oracle_stepwise(int key, const void* a, double* b, size_t N) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < N; ++i) b[i] = ld(key, a, i) >= 0.0 ? 1.0 : 0.0;
+}
+
+void oracle_dilate(int key, const void* a, double value, double* c, size_t N) {
+  const double v = narrow(key, value);
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < N; ++i) c[i] = ld(key, a, i) * v;
+}
+
+void oracle_dilate_reverse(int key, const void* a, double value, const void* b_in, double* b_out, size_t N) {
+  const double v = narrow(key, value);
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < N; ++i) b_out[i] = (b_in ? ld(key, b_in, i) : 0.0) + ld(key, a, i) * v;
+}
+
+void oracle_translate(int key, const void* a, double value, double* c, size_t N) {
+  const double v = narrow(key, value);
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < N; ++i) c[i] = ld(key, a, i) + v;
+}
+
+void oracle_fill(int key, double value, double* a, size_t N) {
+  const double v = narrow(key, value);
+  for (size_t i = 0; i < N; ++i) a[i] = v;
+}
+
+void oracle_sequence(int key, double init, double step, double* a, size_t N) {
+  const double i0 = narrow(key, init), st = narrow(key, step);
+  for (size_t i = 0; i < N; ++i) a[i] = i0 + st * (double)i;
+}
+
+void oracle_copy(int key, const void* src, double* dst, size_t N) {
+  for (size_t i = 0; i < N; ++i) dst[i] = ld(key, src, i);
 }
 
 /* selu(x) = scale*x for x > 0, scale*alpha*expm1(x) otherwise. */

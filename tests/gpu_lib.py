@@ -150,6 +150,33 @@ def hadamard_reverse(a, b, c):
     _call("hadamard_reverse", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(), a.numel())
 
 
+def subtraction(a, b, c):
+    _call("subtraction", a.dtype, a.data_ptr(), b.data_ptr(), c.data_ptr(), a.numel())
+
+
+def unary(stem, a, b):
+    """negate, relu, stepwise, copy, selu: (src, dst, n)."""
+    _call(stem, a.dtype, a.data_ptr(), b.data_ptr(), a.numel())
+
+
+def relu_reverse(a_value, a_grads, b_grads):
+    _call("relu_reverse", a_value.dtype, a_value.data_ptr(), a_grads.data_ptr(), b_grads.data_ptr(),
+          a_value.numel())
+
+
+def scalar_op(stem, a, value, c):
+    """dilate, dilate_reverse, translate: (a, value, c, n)."""
+    _call(stem, a.dtype, a.data_ptr(), float(value), c.data_ptr(), a.numel())
+
+
+def fill(a, value):
+    _call("fill", a.dtype, a.data_ptr(), float(value), a.numel())
+
+
+def sequence(a, init, step):
+    _call("sequence", a.dtype, a.data_ptr(), float(init), float(step), a.numel())
+
+
 def selu(a, b):
     _call("selu", a.dtype, a.data_ptr(), b.data_ptr(), a.numel())
 

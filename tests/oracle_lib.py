@@ -55,6 +55,17 @@ _rmsnorm = _sig("oracle_rmsnorm_ij_j", _it, _vp, _vp, _vp, _db, _sz, _sz)
 _rmsnorm_rev = _sig("oracle_rmsnorm_ij_j_reverse", _it, *([_vp] * 7), _db, _db, _sz, _sz)
 _rmsnorm_rev_mt = _sig("oracle_rmsnorm_ij_j_reverse_mt", _it, *([_vp] * 5), _db, _sz, _sz)
 _set_threads = _sig("oracle_set_threads", _it)
+_subtraction = _sig("oracle_subtraction", _it, _vp, _vp, _vp, _sz)
+_negate = _sig("oracle_negate", _it, _vp, _vp, _sz)
+_relu = _sig("oracle_relu", _it, _vp, _vp, _sz)
+_relu_reverse = _sig("oracle_relu_reverse", _it, _vp, _vp, _vp, _vp, _sz)
+_stepwise = _sig("oracle_stepwise", _it, _vp, _vp, _sz)
+_dilate = _sig("oracle_dilate", _it, _vp, _db, _vp, _sz)
+_dilate_reverse = _sig("oracle_dilate_reverse", _it, _vp, _db, _vp, _vp, _sz)
+_translate = _sig("oracle_translate", _it, _vp, _db, _vp, _sz)
+_fill = _sig("oracle_fill", _it, _db, _vp, _sz)
+_sequence = _sig("oracle_sequence", _it, _db, _db, _vp, _sz)
+_copy = _sig("oracle_copy", _it, _vp, _vp, _sz)
 
 
 def threads():
@@ -109,6 +120,76 @@ def hadamard_reverse(a, b, c_in=None):
     c = _out(a.shape)
     _hadamard_reverse(k, _p(a), _p(b), _p(c_in), _p(c), a.size)
     return c
+
+
+def subtraction(a, b):
+    k, (a, b) = _prep(a, b)
+    c = _out(a.shape)
+    _subtraction(k, _p(a), _p(b), _p(c), a.size)
+    return c
+
+
+def _unary(fn, a):
+    k, (a,) = _prep(a)
+    b = _out(a.shape)
+    fn(k, _p(a), _p(b), a.size)
+    return b
+
+
+def negate(a):
+    return _unary(_negate, a)
+
+
+def relu(a):
+    return _unary(_relu, a)
+
+
+def stepwise(a):
+    return _unary(_stepwise, a)
+
+
+def copy(a):
+    return _unary(_copy, a)
+
+
+def relu_reverse(a_value, b_grads, a_grads_in=None):
+    k, (a_value, b_grads, a_grads_in) = _prep(a_value, b_grads, a_grads_in)
+    o = _out(a_value.shape)
+    _relu_reverse(k, _p(a_value), _p(a_grads_in), _p(b_grads), _p(o), a_value.size)
+    return o
+
+
+def dilate(a, value):
+    k, (a,) = _prep(a)
+    c = _out(a.shape)
+    _dilate(k, _p(a), float(value), _p(c), a.size)
+    return c
+
+
+def dilate_reverse(a, value, b_in=None):
+    k, (a, b_in) = _prep(a, b_in)
+    b = _out(a.shape)
+    _dilate_reverse(k, _p(a), float(value), _p(b_in), _p(b), a.size)
+    return b
+
+
+def translate(a, value):
+    k, (a,) = _prep(a)
+    c = _out(a.shape)
+    _translate(k, _p(a), float(value), _p(c), a.size)
+    return c
+
+
+def fill(dtype, value, n):
+    a = _out((n,))
+    _fill(_KEY[np.dtype(dtype)], float(value), _p(a), n)
+    return a
+
+
+def sequence(dtype, init, step, n):
+    a = _out((n,))
+    _sequence(_KEY[np.dtype(dtype)], float(init), float(step), _p(a), n)
+    return a
 
 
 def selu(a):

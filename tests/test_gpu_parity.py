@@ -55,6 +55,72 @@ def test_add_hadamard_and_reverse(dtype, shift):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shift", [0, 1])
+def test_remaining_elementwise_launchers(dtype, shift):
+    r = rng(14)
+    npdt = G.NP_OF[dtype]
+    for n in [0, 1, 5, 1000, 65537]:
+        G.say(f"sub/negate/relu/step/dilate/translate/fill/sequence/copy dtype={dtype} n={n} shift={shift}")
+        x = r.normal(0, 1, n)
+        x[: min(n, 2)] = [0.0, -0.0][: min(n, 2)]
+        a, b = G.dev(x, dtype, shift), G.dev(r.normal(0, 1, n), dtype, shift)
+        ha, hb = G.host(a.t), G.host(b.t)
+        c = G.Guarded((n,), dtype, shift)
+        G.subtraction(a.t, b.t, c.t)
+        G.compare(c.t, O.subtraction(ha, hb), dtype, f"subtraction n={n}", rowwise=False)
+        for stem, ref in (("negate", O.negate), ("relu", O.relu), ("stepwise", O.stepwise), ("copy", O.copy)):
+            G.unary(stem, a.t, c.t)
+            G.compare(c.t, ref(ha), dtype, f"{stem} n={n}", rowwise=False, rtol=0.0 if stem != "relu" else None)
+        acc = G.dev(r.normal(0, 1, n), dtype, shift)
+        before = G.host(acc.t).copy()
+        G.relu_reverse(a.t, acc.t, b.t)
+        G.compare(acc.t, O.relu_reverse(ha, hb, before), dtype, f"relu_reverse n={n}", rowwise=False)
+        G.scalar_op("dilate", a.t, 0.3, c.t)
+        G.compare(c.t, O.dilate(ha, 0.3), dtype, f"dilate n={n}", rowwise=False)
+        G.scalar_op("translate", a.t, -1.7, c.t)
+        G.compare(c.t, O.translate(ha, -1.7), dtype, f"translate n={n}", rowwise=False)
+        acc = G.dev(r.normal(0, 1, n), dtype, shift)
+        before = G.host(acc.t).copy()
+        G.scalar_op("dilate_reverse", a.t, 0.3, acc.t)
+        G.compare(acc.t, O.dilate_reverse(ha, 0.3, before), dtype, f"dilate_reverse n={n}", rowwise=False)
+        G.fill(c.t, 1.0)
+        assert bool((c.t == 1).all())
+        G.fill(c.t, 0.1)
+        G.compare(c.t, O.fill(npdt, 0.1, n), dtype, f"fill n={n}", rowwise=False, rtol=0.0)
+        G.sequence(c.t, 0.5, 0.25)
+        G.compare(c.t, O.sequence(npdt, 0.5, 0.25, n), dtype, f"sequence n={n}", rowwise=False)
+        for g in (a, b, c, acc):
+            g.check(f"remaining elementwise n={n}")
+
+
+def test_reference_example_all_ones_through_relu_add():
+    # src/examples/subgraphs.zig:34-45: x = w1 = w2 = 1; z4 = relu(relu(x + w1) + w2) == 3
+    f32 = torch.float32
+    n = 32
+    x, w1, w2 = (G.Guarded((n,), f32) for _ in range(3))
+    for t in (x, w1, w2):
+        G.fill(t.t, 1.0)
+    z1, z2, z3, z4 = (G.Guarded((n,), f32) for _ in range(4))
+    G.say("subgraphs example: relu(add) twice")
+    G.addition(x.t, w1.t, z1.t)
+    G.unary("relu", z1.t, z2.t)
+    G.addition(z2.t, w2.t, z3.t)
+    G.unary("relu", z3.t, z4.t)
+    assert bool((z4.t == 3).all())
+    # reverse: seed dz4 = 1 (graph.zig:116), then relu_reverse / in-place addition as the ops do
+    grads = {k: G.dev(np.zeros(n), f32) for k in ("z4", "z3", "z2", "z1", "x", "w1", "w2")}
+    G.fill(grads["z4"].t, 1.0)
+    G.relu_reverse(z3.t, grads["z3"].t, grads["z4"].t)
+    G.addition(grads["z3"].t, grads["z2"].t, grads["z2"].t)
+    G.addition(grads["z3"].t, grads["w2"].t, grads["w2"].t)
+    G.relu_reverse(z1.t, grads["z1"].t, grads["z2"].t)
+    G.addition(grads["z1"].t, grads["x"].t, grads["x"].t)
+    G.addition(grads["z1"].t, grads["w1"].t, grads["w1"].t)
+    for k in ("x", "w1", "w2"):
+        assert bool((grads[k].t == 1).all()), k
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 def test_addition_in_place_as_the_reference_reverse_calls_it(dtype):
     # src/ops/addition.zig:67-73: gx = gz + gx with the output aliasing the second input
     r = rng(11)

@@ -75,6 +75,35 @@ def test_add_hadamard_and_accumulating_reverse():
     assert np.array_equal(O.hadamard_reverse(a, b, c0), c0.astype(np.float64) + a64 * b64)
 
 
+def test_remaining_elementwise_launchers_closed_forms():
+    a = np.concatenate([RNG.normal(0, 1, 500), [0.0, -0.0]]).astype(np.float32)
+    b = RNG.normal(0, 1, a.size).astype(np.float32)
+    a64, b64 = a.astype(np.float64), b.astype(np.float64)
+    assert np.array_equal(O.subtraction(a, b), a64 - b64)
+    assert np.array_equal(O.negate(a), -a64)
+    assert np.array_equal(O.copy(a), a64)
+    assert np.array_equal(O.relu(a), torch.relu(t64(a)).numpy())
+    assert np.array_equal(O.stepwise(a), (a64 >= 0).astype(np.float64))
+    assert O.stepwise(np.array([-0.0]))[0] == 1.0  # -0.0 >= 0, as in relu.cu:12
+    # relu reverse: subgraphs.zig:34-45 — all-ones through relu(add) gives gradients of 1
+    one = np.ones(8, dtype=np.float32)
+    assert np.all(O.relu_reverse(O.addition(one, one).astype(np.float32), one) == 1.0)
+    at = t64(a).requires_grad_(True)
+    torch.relu(at).backward(t64(b))
+    nz = a64 != 0  # torch takes 0 as the slope at exactly 0; the reference takes 1
+    assert np.array_equal(O.relu_reverse(a, b)[nz], at.grad.numpy()[nz])
+    assert np.array_equal(O.relu_reverse(a, b)[~nz], b64[~nz])
+    assert np.array_equal(O.relu_reverse(a, b, b), b64 + O.relu_reverse(a, b))
+    v = 0.1  # not representable: narrowed to the storage type before use
+    assert np.array_equal(O.dilate(a, v), a64 * float(np.float32(v)))
+    assert np.array_equal(O.translate(a, v), a64 + float(np.float32(v)))
+    assert np.array_equal(O.dilate_reverse(a, v, b), b64 + a64 * float(np.float32(v)))
+    h = a.astype(np.float16)
+    assert np.array_equal(O.dilate(h, v), h.astype(np.float64) * float(np.float16(v)))
+    assert np.array_equal(O.fill(np.float32, v, 5), np.full(5, float(np.float32(v))))
+    assert np.array_equal(O.sequence(np.float64, 1.5, 0.25, 6), 1.5 + 0.25 * np.arange(6))
+
+
 def test_reduce_blend_and_orientation():
     src = RNG.normal(0, 1, (5, 9))
     d_i, d_j = RNG.normal(0, 1, 5), RNG.normal(0, 1, 9)
