@@ -40,8 +40,12 @@ def make_sets(name, count=None):
     return [W.WORKLOADS[name](seed=i) for i in range(count or SETS[name])]
 
 
+EVENT_EVERY = 8  # a pair of events costs ~2-5 us of stream time: sample launches, not every one
+
+
 def time_steps(sets, steps, warmup):
-    """K timed steps; returns (seconds, per-step forward ms, per-step reverse ms)."""
+    """K timed steps. Returns (seconds, durations in ms of the dominant launcher sampled with
+    events inside the timed region on the launch stream)."""
     import torch
     S = len(sets)
     rev_of = lambda i: sets[(i + S // 2) % S]
@@ -52,21 +56,50 @@ def time_steps(sets, steps, warmup):
         sets[i % S].forward()
         if has_rev:
             rev_of(i).reverse()
-    ev = _events(3 * steps)
+    every = EVENT_EVERY if steps >= 4 * EVENT_EVERY else 1
+    sampled = list(range(0, steps, every))
+    ev = {i: _events(2) for i in sampled}
     torch.cuda.synchronize()
     t0 = time.perf_counter()
     for i in range(steps):
-        ev[3 * i].record()
-        sets[i % S].forward()
-        ev[3 * i + 1].record()
         if has_rev:
+            sets[i % S].forward()
+            if i in ev:
+                ev[i][0].record()
             rev_of(i).reverse()
-        ev[3 * i + 2].record()
+            if i in ev:
+                ev[i][1].record()
+        else:
+            if i in ev:
+                ev[i][0].record()
+            sets[i % S].forward()
+            if i in ev:
+                ev[i][1].record()
     torch.cuda.synchronize()
     dt = time.perf_counter() - t0
-    fwd = [ev[3 * i].elapsed_time(ev[3 * i + 1]) for i in range(steps)]
-    rev = [ev[3 * i + 1].elapsed_time(ev[3 * i + 2]) for i in range(steps)] if has_rev else []
-    return dt, fwd, rev
+    return dt, [ev[i][0].elapsed_time(ev[i][1]) for i in sampled]
+
+
+def time_each(sets, iters):
+    """Per-launcher medians outside the headline region: (forward ms list, reverse ms list)."""
+    import torch
+    S = len(sets)
+    has_rev = sets[0].has_reverse
+    fwd, rev = [], []
+    for i in range(iters):
+        a, b = _events(2)
+        a.record()
+        sets[i % S].forward()
+        b.record()
+        fwd.append((a, b))
+        if has_rev:
+            c, d = _events(2)
+            c.record()
+            sets[(i + S // 2) % S].reverse()
+            d.record()
+            rev.append((c, d))
+    torch.cuda.synchronize()
+    return [a.elapsed_time(b) for a, b in fwd], [a.elapsed_time(b) for a, b in rev]
 
 
 def rates(w, fwd_ms, rev_ms):
@@ -141,11 +174,12 @@ def main():
     name = args.workload
     sets = make_sets(name)
     w = sets[0]
-    dt, fwd_ms, rev_ms = time_steps(sets, args.steps, args.warmup)
+    dt, dom_ms = time_steps(sets, args.steps, args.warmup)
     step_bytes = w.fwd_bytes + w.rev_bytes
     value = args.steps * step_bytes / dt / 1e9
+    fwd_ms, rev_ms = time_each(sets, max(20, min(args.steps, 100)))
 
-    dom_ms, dom_bytes, dom_name = (rev_ms, w.rev_bytes, "reverse") if rev_ms else (fwd_ms, w.fwd_bytes, "forward")
+    dom_bytes, dom_name = (w.rev_bytes, "reverse") if w.has_reverse else (w.fwd_bytes, "forward")
     avg_ms = sum(dom_ms) / len(dom_ms)
     achieved = dom_bytes / (avg_ms * 1e-3) / 1e9
     traffic_path = os.path.join(ROOT, "profiles", f"traffic_{name}.json")
@@ -174,7 +208,7 @@ def main():
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
                      "kernel": f"{name} {dom_name} launcher", "bytes_per_launch": dom_bytes,
-                     "avg_launch_ms": round(avg_ms, 5)},
+                     "avg_launch_ms": round(avg_ms, 5), "launches_timed": len(dom_ms)},
         name: rates(w, fwd_ms, rev_ms),
     }
 
@@ -190,7 +224,8 @@ def main():
                 continue
             osets = make_sets(other)
             k = max(10, min(args.steps, 40 if other in ("cfg3", "cfg4") else 100))
-            _, f_ms, r_ms = time_steps(osets, k, 5)
+            time_steps(osets, 5, 2)
+            f_ms, r_ms = time_each(osets, k)
             extra[other] = rates(osets[0], f_ms, r_ms)
             extra[other]["workload"] = W.DESCRIPTION[other]
             del osets
