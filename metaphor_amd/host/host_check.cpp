@@ -1,0 +1,226 @@
+/*
+ * Check program of the C++ host side. Runs on a GPU.
+ *
+ *   host_check <output directory>
+ *
+ * Part 1 replays the reference's own example (src/examples/subgraphs.zig:8-133) with the same
+ * assertions: two relu(add) blocks, detach, reverse(.free) then reverse(.keep).
+ * Part 2 builds e = selu(hadamard(add(a,b), add(c,d))) through mp::ops, checks that forward and
+ * reverse are one kernel each, and writes inputs, outputs and gradients as raw little-endian
+ * files for the Python test to compare with the CPU oracle; the same for softmax and RMSNorm
+ * through the graph, and for an expression that must NOT fuse (a repeated input).
+ */
+#include <cmath>
+#include <cstdio>
+#include <cstdlib>
+#include <string>
+#include <vector>
+
+#include "metaphor.hpp"
+
+#define CHECK(cond)                                                          \
+  do {                                                                       \
+    if (!(cond)) {                                                           \
+      fprintf(stderr, "host_check: %s failed at line %d\n", #cond, __LINE__); \
+      return 1;                                                              \
+    }                                                                        \
+  } while (0)
+
+static std::string out_dir;
+
+template <class T> static void dump(const std::string& name, const std::vector<T>& v) {
+  const std::string path = out_dir + "/" + name + ".bin";
+  FILE* f = fopen(path.c_str(), "wb");
+  if (!f || fwrite(v.data(), sizeof(T), v.size(), f) != v.size()) {
+    fprintf(stderr, "host_check: cannot write %s\n", path.c_str());
+    exit(2);
+  }
+  fclose(f);
+}
+
+/* SplitMix64 -> uniform in [lo, hi) */
+struct Rng {
+  uint64_t s;
+  double next() {
+    uint64_t z = (s += 0x9e3779b97f4a7c15ull);
+    z = (z ^ (z >> 30)) * 0xbf58476d1ce4e5b9ull;
+    z = (z ^ (z >> 27)) * 0x94d049bb133111ebull;
+    z ^= z >> 31;
+    return (double)(z >> 11) / 9007199254740992.0;
+  }
+  std::vector<float> uniform(size_t n, double lo, double hi) {
+    std::vector<float> v(n);
+    for (auto& x : v) x = (float)(lo + (hi - lo) * next());
+    return v;
+  }
+  std::vector<float> normal(size_t n, double mu, double sd) {
+    std::vector<float> v(n);
+    for (auto& x : v) {
+      const double u1 = next() + 1e-300, u2 = next();
+      x = (float)(mu + sd * std::sqrt(-2.0 * std::log(u1)) * std::cos(6.283185307179586 * u2));
+    }
+    return v;
+  }
+};
+
+/* upload an upstream gradient, as a loss would have left it (reverse seeds ones only when none exists) */
+static void set_grad(mp::Tensor t, const std::vector<float>& host) {
+  mp::enable_gradient(t);
+  mpMemcpyHtoD(t.grad_ptr(), host.data(), host.size() * sizeof(float), t.context());
+  mpStreamSynchronize(t.context());
+}
+
+static mp::Tensor leaf(mp::Graph* G, mp::TensorClass cls, const std::vector<size_t>& sizes,
+                       const std::vector<float>& host) {
+  mp::Tensor t = G->tensor(cls, mp::Tag::r32, sizes);
+  mp::util::to_device(host.data(), t, host.size() * sizeof(float));
+  return t;
+}
+
+static int subgraphs_example(mp::Stream stream) {
+  mp::Graph* G = mp::Graph::init({stream, mp::Mode::train});
+  const size_t M = 32;
+  mp::Tensor x = G->tensor(mp::TensorClass::inp, mp::Tag::r32, {M});
+  mp::Tensor w1 = G->tensor(mp::TensorClass::wgt, mp::Tag::r32, {M});
+  mp::Tensor w2 = G->tensor(mp::TensorClass::wgt, mp::Tag::r32, {M});
+  mp::algo::fill(x, 1.0);
+  mp::algo::fill(w1, 1.0);
+  mp::algo::fill(w2, 1.0);
+
+  mp::Tensor z1 = mp::ops::add(x, w1);
+  mp::Tensor z2 = mp::ops::relu(z1);
+  mp::Tensor z3 = mp::ops::add(z2, w2);
+  mp::Tensor z4 = mp::ops::relu(z3);
+  for (float v : z4.native<float>()) CHECK(v == 3.0f);
+
+  z2.detach();
+  z4.reverse(mp::ReverseCleanup::free);
+  CHECK(z4.len() == 0);
+  CHECK(z3.len() == 0);
+  CHECK(!z4.has_grad());
+  CHECK(!z3.has_grad());
+  CHECK(z2.len() != 0);
+  CHECK(w2.len() != 0);
+  CHECK(z2.has_grad());
+  CHECK(w2.has_grad());
+  CHECK(z1.len() != 0);
+  CHECK(w1.len() != 0);
+  CHECK(!z1.has_grad());
+  CHECK(!w1.has_grad());
+  for (float v : w2.native_grad<float>()) CHECK(v == 1.0f);
+
+  z2.reverse(mp::ReverseCleanup::keep);
+  CHECK(x.len() != 0);
+  CHECK(z1.len() != 0);
+  CHECK(w1.len() != 0);
+  CHECK(z1.has_grad());
+  CHECK(w1.has_grad());
+  CHECK(x.has_grad());
+  for (float v : w1.native_grad<float>()) CHECK(v == 1.0f);
+  for (float v : x.native_grad<float>()) CHECK(v == 1.0f);
+  G->deinit();
+  return 0;
+}
+
+static int fused_chain(mp::Stream stream) {
+  mp::Graph* G = mp::Graph::init({stream, mp::Mode::train});
+  const size_t n = 100003;
+  Rng r{7};
+  const auto ha = r.uniform(n, -2, 2), hb = r.uniform(n, -2, 2), hc = r.uniform(n, -2, 2), hd = r.uniform(n, -2, 2);
+  mp::Tensor a = leaf(G, mp::TensorClass::wgt, {n}, ha), b = leaf(G, mp::TensorClass::wgt, {n}, hb);
+  mp::Tensor c = leaf(G, mp::TensorClass::wgt, {n}, hc), d = leaf(G, mp::TensorClass::inp, {n}, hd);
+  dump("fused_a", ha); dump("fused_b", hb); dump("fused_c", hc); dump("fused_d", hd);
+
+  const size_t before = G->launches;
+  mp::Tensor e = mp::ops::selu(mp::ops::hadamard(mp::ops::add(a, b), mp::ops::add(c, d)));
+  CHECK(G->launches == before);                 /* nothing ran yet */
+  dump("fused_e", e.native<float>());
+  CHECK(G->launches == before + 1);             /* the whole chain was one kernel */
+
+  const size_t before_rev = G->launches;
+  e.reverse(mp::ReverseCleanup::keep);          /* seeds de = 1 */
+  CHECK(G->launches == before_rev + 1 + 1);     /* the seed fill of de, then ONE reverse kernel */
+  dump("fused_da", a.native_grad<float>()); dump("fused_db", b.native_grad<float>());
+  dump("fused_dc", c.native_grad<float>()); dump("fused_dd", d.native_grad<float>());
+
+  /* second pass over the same leaves: gradients accumulate (alpha = 1 path) */
+  mp::Tensor e2 = mp::ops::selu(mp::ops::hadamard(mp::ops::add(a, b), mp::ops::add(c, d)));
+  e2.reverse(mp::ReverseCleanup::free);
+  CHECK(e2.len() == 0);
+  dump("fused_da2", a.native_grad<float>());
+
+  /* a repeated input must not fuse: selu((a+a)*(c+d)) runs per op and still differentiates right */
+  G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+  const size_t l0 = G->launches;
+  mp::Tensor f = mp::ops::selu(mp::ops::hadamard(mp::ops::add(a, a), mp::ops::add(c, d)));
+  dump("rep_f", f.native<float>());
+  CHECK(G->launches == l0 + 4);
+  f.reverse(mp::ReverseCleanup::keep);
+  dump("rep_da", a.native_grad<float>()); dump("rep_dc", c.native_grad<float>());
+
+  /* eval mode attaches nothing and reverse is refused by construction: only forward here */
+  mp::Graph* E = mp::Graph::init({stream, mp::Mode::eval});
+  mp::Tensor ea = leaf(E, mp::TensorClass::inp, {n}, ha), eb = leaf(E, mp::TensorClass::inp, {n}, hb);
+  mp::Tensor ec = leaf(E, mp::TensorClass::inp, {n}, hc), ed = leaf(E, mp::TensorClass::inp, {n}, hd);
+  mp::Tensor ee = mp::ops::selu(mp::ops::hadamard(mp::ops::add(ea, eb), mp::ops::add(ec, ed)));
+  dump("eval_e", ee.native<float>());
+  E->deinit();
+  G->deinit();
+  return 0;
+}
+
+static int row_ops(mp::Stream stream) {
+  mp::Graph* G = mp::Graph::init({stream, mp::Mode::train});
+  const size_t m = 37, n = 1000;
+  Rng r{11};
+  const auto hx = r.normal(m * n, 0, 1), hg = r.normal(n, 1, 0.02), hs = r.normal(m * n, 0, 2);
+  mp::Tensor x = leaf(G, mp::TensorClass::inp, {m, n}, hx);
+  mp::Tensor g = leaf(G, mp::TensorClass::wgt, {n}, hg);
+  mp::Tensor s = leaf(G, mp::TensorClass::inp, {m, n}, hs);
+  dump("row_x", hx); dump("row_g", hg); dump("row_s", hs);
+
+  const auto hdy = r.normal(m * n, 0, 1), hdp = r.normal(m * n, 0, 1);
+  dump("row_dy", hdy); dump("row_dp", hdp);
+
+  mp::Tensor y = mp::ops::rmsnorm(x, g, 1e-6);
+  dump("row_y", y.native<float>());
+  set_grad(y, hdy);
+  y.reverse(mp::ReverseCleanup::keep);
+  dump("row_dx", x.native_grad<float>()); dump("row_dg", g.native_grad<float>());
+
+  /* p = softmax(s + s) exercises a pending add feeding a row op */
+  mp::Tensor p = mp::ops::softmax(mp::ops::add(s, s));
+  dump("row_p", p.native<float>());
+  set_grad(p, hdp);
+  p.reverse(mp::ReverseCleanup::keep);
+  dump("row_ds", s.native_grad<float>());
+  G->deinit();
+  return 0;
+}
+
+int main(int argc, char** argv) {
+  if (argc != 2) {
+    fprintf(stderr, "usage: host_check <output directory>\n");
+    return 2;
+  }
+  out_dir = argv[1];
+  mp::device::init(0);
+  CHECK(mp::device::total_memory(0) > 0);
+  mp::Stream stream = mp::stream::init();
+  mp::Stream second = mp::stream::init();
+  CHECK(stream->ID == 0 && second->ID == 1);
+  mp::stream::deinit(second);
+
+  if (subgraphs_example(stream)) return 1;
+  printf("host_check: subgraphs example ok\n");
+  if (fused_chain(stream)) return 1;
+  printf("host_check: fused chain ok (one kernel forward, one kernel reverse)\n");
+  if (row_ops(stream)) return 1;
+  printf("host_check: softmax / rmsnorm through the graph ok\n");
+
+  mp::stream::sync(stream);
+  mp::stream::deinit(stream);
+  mp::device::check();
+  printf("host_check: done\n");
+  return 0;
+}

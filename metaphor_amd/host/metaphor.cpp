@@ -1,0 +1,554 @@
+/*
+ * Host side of the hot path: stream registry, tensor allocator, graph / autograd walk, op
+ * modules and the deferred-elementwise fusion. See metaphor.hpp for the map to the reference.
+ * Everything device-side goes through the C-ABI (mp* utilities and launch_* kernels); no HIP
+ * header is needed to build this file.
+ */
+#include "metaphor.hpp"
+
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+
+#include "kernels.hpp"
+
+namespace mp {
+
+void panic(const char* what) {
+  fprintf(stderr, "metaphor: %s\n", what);
+  abort();
+}
+
+/* ------------------------------------------------------------------ streams / device */
+
+static std::mutex stream_mutex;
+static StreamEntry stream_array[MAX_STREAMS];
+static bool stream_used[MAX_STREAMS];
+
+void* StreamEntry::get_scratch(size_t bytes) {
+  if (scratch_bytes < bytes) {
+    if (scratch_head) mpMemFree(scratch_head, context);
+    scratch_head = mpMemAlloc(bytes, context);
+    if (!scratch_head) panic("get_scratch: device allocation failed");
+    scratch_bytes = bytes;
+  }
+  return scratch_head;
+}
+
+namespace device {
+void init(uint32_t device_number) { mpInitDevice(device_number); }
+void sync() { mpDeviceSynchronize(); }
+void check() { mpCheckLastError(); }
+size_t total_memory(uint32_t device_number) { return mpDeviceTotalMemory(device_number); }
+}  // namespace device
+
+namespace stream {
+Stream init() {
+  std::lock_guard<std::mutex> lock(stream_mutex);
+  for (size_t i = 0; i < MAX_STREAMS; ++i) {
+    if (!stream_used[i]) {
+      stream_used[i] = true;
+      stream_array[i] = StreamEntry{};
+      stream_array[i].ID = i;
+      stream_array[i].context = mpInitStream();
+      return &stream_array[i];
+    }
+  }
+  panic("stream limit reached - increase streams");
+}
+
+void deinit(Stream s) {
+  if (s->scratch_head) {
+    mpMemFree(s->scratch_head, s->context);
+    mpStreamSynchronize(s->context);
+  }
+  mpDeinitStream(s->context);
+  mpDeviceSynchronize();
+  std::lock_guard<std::mutex> lock(stream_mutex);
+  stream_used[s->ID] = false;
+}
+
+void sync(Stream s) { mpStreamSynchronize(s->context); }
+}  // namespace stream
+
+/* ------------------------------------------------------------------ tensor allocator */
+
+TensorData TensorAllocator::alloc(Tag dtype, size_t n, Stream s) {
+  const size_t bytes = n * tag_size(dtype);
+  auto it = cache_.find(bytes);
+  void* p = nullptr;
+  if (it != cache_.end() && !it->second.empty()) {
+    p = it->second.back();
+    it->second.pop_back();
+  } else {
+    p = mpMemAlloc(bytes, s->context);
+    if (!p) panic("TensorAllocator.alloc: device allocation failed");
+  }
+  return TensorData{p, n, dtype};
+}
+
+void TensorAllocator::free(TensorData d, Stream) {
+  if (!d.ptr) return;
+  cache_[d.len * tag_size(d.dtype)].push_back(d.ptr);
+}
+
+void TensorAllocator::deinit(Stream s) {
+  for (auto& kv : cache_)
+    for (void* p : kv.second) mpMemFree(p, s->context);
+  cache_.clear();
+}
+
+/* ------------------------------------------------------------------ graph */
+
+Graph* Graph::init(GraphConfig config) {
+  if (!config.stream) panic("Graph.init: a stream is required");
+  Graph* g = new Graph();
+  g->stream = config.stream;
+  g->mode = config.mode;
+  return g;
+}
+
+void Graph::deinit() {
+  reset(ResetGroup::node, ResetComponent::all);
+  reset(ResetGroup::leaf, ResetComponent::all);
+  allocator_.deinit(stream);
+  mpStreamSynchronize(stream->context);
+  delete this;
+}
+
+TensorData& Graph::data_of(Tensor t) {
+  return t.cls == TensorClass::hid ? nodes_[t.idx].data : leaves_[t.idx].data;
+}
+TensorData& Graph::grad_of(Tensor t) {
+  return t.cls == TensorClass::hid ? nodes_[t.idx].grad : leaves_[t.idx].grad;
+}
+
+Tensor Graph::tensor(TensorClass cls, Tag dtype, const std::vector<size_t>& sizes) {
+  if (sizes.empty()) panic("Graph.tensor: sizes must not be empty");
+  size_t n = 1;
+  for (size_t s : sizes) n *= s;
+  if (n == 0) panic("Graph.tensor: every size must be positive");
+  if (cls == TensorClass::hid) {
+    Node node;
+    node.data = allocator_.alloc(dtype, n, stream);
+    node.sizes = sizes;
+    nodes_.push_back(std::move(node));
+    return Tensor{this, nodes_.size() - 1, cls};
+  }
+  Leaf leaf;
+  leaf.data = allocator_.alloc(dtype, n, stream);
+  leaf.sizes = sizes;
+  leaf.cls = cls;
+  leaves_.push_back(std::move(leaf));
+  return Tensor{this, leaves_.size() - 1, cls};
+}
+
+void Graph::free_gradient(Tensor t) {
+  TensorData& g = grad_of(t);
+  if (g.ptr) {
+    allocator_.free(g, stream);
+    g = TensorData{};
+  }
+}
+
+void Graph::free_tensor(Tensor t) {
+  TensorData& d = data_of(t);
+  if (d.len == 0) return;
+  if (d.ptr) allocator_.free(d, stream);
+  d.ptr = nullptr;
+  d.len = 0;
+  if (t.cls == TensorClass::hid) nodes_[t.idx].pending = Pending::none;
+  free_gradient(t);
+}
+
+void Graph::reset(ResetGroup group, ResetComponent component) {
+  if (group == ResetGroup::leaf) {
+    for (size_t i = 0; i < leaves_.size(); ++i) {
+      Tensor t{this, i, leaves_[i].cls};
+      if (component == ResetComponent::grd) free_gradient(t);
+      else free_tensor(t);
+    }
+    if (component == ResetComponent::all) leaves_.clear();
+  } else {
+    for (size_t i = 0; i < nodes_.size(); ++i) {
+      Tensor t{this, i, TensorClass::hid};
+      if (component == ResetComponent::grd) {
+        free_gradient(t);
+        nodes_[i].deps = 0;
+      } else {
+        free_tensor(t);
+      }
+    }
+    if (component == ResetComponent::all) nodes_.clear();
+  }
+}
+
+void enable_gradient(Tensor t) {
+  Graph* g = t.ptr;
+  TensorData& grd = g->grad_of(t);
+  if (!grd.ptr) {
+    grd = g->allocator_.alloc(t.dtype(), t.len(), g->stream);
+    /* the reference leaves new gradient storage unwritten (src/core/graph.zig:710-722) although
+     * every reverse kernel accumulates into it; here it starts at zero */
+    kernels::fill(dkey(t), grd.ptr, 0.0, (len_t)grd.len, g->stream->context);
+    g->launches++;
+  }
+}
+
+void attach_op(Tensor t, void (*rev)(const std::vector<OpDatum>&), std::vector<OpDatum> args) {
+  if (t.cls != TensorClass::hid) panic("attach_op: only computed tensors carry an op");
+  Graph* g = t.ptr;
+  for (size_t i = 0; i + 1 < args.size(); ++i) { /* the last argument is the output itself */
+    const OpDatum& a = args[i];
+    if (a.kind == OpDatum::tensor && a.t.cls == TensorClass::hid) g->nodes_[a.t.idx].deps += 1;
+  }
+  OpInterface& op = g->nodes_[t.idx].op;
+  op.reverse = rev;
+  op.args = std::move(args);
+  op.live = true;
+}
+
+/* src/core/graph.zig:552-631 */
+void Graph::reverse(size_t idx, ReverseCleanup cleanup) {
+  if (mode == Mode::eval) panic("Graph.reverse: graph is in eval mode");
+  if (nodes_.empty()) return;
+  std::vector<size_t> node_stack{idx}, free_stack;
+  while (!node_stack.empty()) {
+    const size_t last = node_stack.back();
+    node_stack.pop_back();
+    OpInterface& op = nodes_[last].op;
+    if (!op.live) continue;
+    if (cleanup == ReverseCleanup::free) free_stack.push_back(last);
+    op.reverse(op.args);
+    for (const OpDatum& arg : op.args) {
+      if (arg.kind != OpDatum::tensor) continue;
+      if (arg.t.cls != TensorClass::hid || arg.t.idx == last) continue;
+      if (!nodes_[arg.t.idx].attached) continue;
+      if (--nodes_[arg.t.idx].deps == 0) node_stack.push_back(arg.t.idx);
+    }
+    op.args.clear();
+    op.live = false;
+  }
+  if (cleanup == ReverseCleanup::free) {
+    mpStreamSynchronize(stream->context);
+    for (size_t node : free_stack) free_tensor(Tensor{this, node, TensorClass::hid});
+  }
+}
+
+/* ------------------------------------------------------------------ tensor */
+
+Tag Tensor::dtype() const { return ptr->data_of(*this).dtype; }
+const std::vector<size_t>& Tensor::sizes() const {
+  return cls == TensorClass::hid ? ptr->nodes_[idx].sizes : ptr->leaves_[idx].sizes;
+}
+size_t Tensor::len() const { return ptr->data_of(*this).len; }
+Stream Tensor::stream() const { return ptr->stream; }
+StreamContext Tensor::context() const { return ptr->stream->context; }
+void* Tensor::grad_ptr() const { return ptr->grad_of(*this).ptr; }
+void Tensor::detach() const {
+  if (cls == TensorClass::hid) ptr->nodes_[idx].attached = false;
+}
+void Tensor::free() const { ptr->free_tensor(*this); }
+
+void* Tensor::data_ptr() const {
+  materialise(*this);
+  return ptr->data_of(*this).ptr;
+}
+
+void Tensor::reverse(ReverseCleanup cleanup) const {
+  materialise(*this);
+  if (!has_grad()) {
+    /* no loss applied: d self / d self = 1 (src/core/graph.zig:112-117) */
+    ptr->grad_of(*this) = ptr->allocator_.alloc(dtype(), len(), ptr->stream);
+    kernels::fill(dkey(*this), grad_ptr(), 1.0, (len_t)len(), context());
+    ptr->launches++;
+  }
+  if (cls != TensorClass::hid) return;
+  ptr->reverse(idx, cleanup);
+}
+
+void Tensor::copy_out(void* dst, size_t bytes, bool grad) const {
+  const void* src = grad ? grad_ptr() : data_ptr();
+  mpMemcpyDtoH(dst, src, bytes, context()); /* returns with the bytes on the host */
+}
+
+/* ------------------------------------------------------------------ deferred elementwise */
+
+bool is_pending(Tensor t) {
+  return t.cls == TensorClass::hid && t.ptr->nodes_[t.idx].pending != Pending::none;
+}
+
+/* A pending node owns no bytes yet: its buffer is taken from the allocator when it is computed. */
+Tensor defer(Graph* g, Pending op, Tensor x, Tensor y) {
+  Graph::Node node;
+  node.data = TensorData{nullptr, x.len(), x.dtype()};
+  node.sizes = x.sizes();
+  node.pending = op;
+  node.in0 = x;
+  node.in1 = y;
+  g->nodes_.push_back(std::move(node));
+  return Tensor{g, g->nodes_.size() - 1, TensorClass::hid};
+}
+
+static void addition_reverse(const std::vector<OpDatum>& a);
+static void hadamard_reverse(const std::vector<OpDatum>& a);
+static void selu_reverse(const std::vector<OpDatum>& a);
+static void fused_reverse(const std::vector<OpDatum>& a);
+
+void materialise(Tensor t) {
+  if (!is_pending(t)) return;
+  Graph* g = t.ptr;
+  const Pending op = g->nodes_[t.idx].pending;
+  const Tensor in0 = g->nodes_[t.idx].in0, in1 = g->nodes_[t.idx].in1;
+  const size_t n = g->nodes_[t.idx].data.len;
+  const Tag dt = g->nodes_[t.idx].data.dtype;
+  const size_t key = (size_t)dt;
+  const StreamContext ctx = g->stream->context;
+
+  auto take_buffer = [&]() {
+    TensorData d = g->allocator_.alloc(dt, n, g->stream);
+    g->nodes_[t.idx].data = d;
+    g->nodes_[t.idx].pending = Pending::none;
+    return d.ptr;
+  };
+
+  /* selu(hadamard(add(a,b), add(c,d))) with the three inner nodes still pending and owned by
+   * the same graph: one launch, and the inner nodes stay unmaterialised */
+  if (op == Pending::selu && is_pending(in0) && in0.ptr == g && g->nodes_[in0.idx].pending == Pending::hadamard) {
+    const Tensor u = g->nodes_[in0.idx].in0, v = g->nodes_[in0.idx].in1;
+    if (is_pending(u) && is_pending(v) && u.ptr == g && v.ptr == g && !u.same(v) &&
+        g->nodes_[u.idx].pending == Pending::add && g->nodes_[v.idx].pending == Pending::add) {
+      const Tensor a = g->nodes_[u.idx].in0, b = g->nodes_[u.idx].in1;
+      const Tensor c = g->nodes_[v.idx].in0, d = g->nodes_[v.idx].in1;
+      const bool distinct = !a.same(b) && !a.same(c) && !a.same(d) && !b.same(c) && !b.same(d) && !c.same(d);
+      if (distinct) {
+      void* pa = a.data_ptr();
+      void* pb = b.data_ptr();
+      void* pc = c.data_ptr();
+      void* pd = d.data_ptr();
+      void* pe = take_buffer();
+      kernels::fused_selu_hadamard_add_add(key, pa, pb, pc, pd, pe, (len_t)n, ctx);
+      g->launches++;
+      if (g->mode == Mode::train) attach_op(t, fused_reverse, {a, b, c, d, t});
+      return;
+      } /* a repeated input needs its contributions added up: per-op path below */
+    }
+  }
+  if (in0.len() == 0 || in1.len() == 0) panic("materialise: an input of a pending node was freed");
+
+  /* anything else: one launch per op, as the reference's forward_impl does */
+  void* p0 = in0.data_ptr();
+  if (op == Pending::selu) {
+    void* pz = take_buffer();
+    kernels::selu(key, p0, pz, (len_t)n, ctx);
+    g->launches++;
+    if (g->mode == Mode::train) attach_op(t, selu_reverse, {in0, t});
+    return;
+  }
+  void* p1 = in1.data_ptr();
+  void* pz = take_buffer();
+  if (op == Pending::add) {
+    kernels::addition(key, p0, p1, pz, (len_t)n, ctx);
+    if (g->mode == Mode::train) attach_op(t, addition_reverse, {in0, in1, t});
+  } else {
+    kernels::hadamard(key, p0, p1, pz, (len_t)n, ctx);
+    if (g->mode == Mode::train) attach_op(t, hadamard_reverse, {in0, in1, t});
+  }
+  g->launches++;
+}
+
+void Graph::flush() {
+  for (size_t i = 0; i < nodes_.size(); ++i) materialise(Tensor{this, i, TensorClass::hid});
+}
+
+/* ------------------------------------------------------------------ op modules */
+
+static void check_pair(Tensor x, Tensor y, const char* what) {
+  if (x.dtype() != y.dtype()) panic(what);
+  if (x.sizes() != y.sizes()) panic(what);
+}
+
+/* src/ops/addition.zig:60-82: gx = gz + gx, gy = gz + gy, in place */
+static void addition_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, y = a[1].t, z = a[2].t;
+  enable_gradient(x);
+  enable_gradient(y);
+  const size_t key = dkey(z);
+  kernels::addition(key, z.grad_ptr(), x.grad_ptr(), x.grad_ptr(), (len_t)x.len(), x.context());
+  kernels::addition(key, z.grad_ptr(), y.grad_ptr(), y.grad_ptr(), (len_t)y.len(), y.context());
+  z.ptr->launches += 2;
+}
+
+/* src/ops/hadamard.zig:58-80 */
+static void hadamard_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, y = a[1].t, z = a[2].t;
+  enable_gradient(x);
+  enable_gradient(y);
+  const size_t key = dkey(z);
+  kernels::hadamard_reverse(key, z.grad_ptr(), y.data_ptr(), x.grad_ptr(), (len_t)x.len(), x.context());
+  kernels::hadamard_reverse(key, z.grad_ptr(), x.data_ptr(), y.grad_ptr(), (len_t)y.len(), y.context());
+  z.ptr->launches += 2;
+}
+
+/* the shape of src/ops/relu.zig:39-52 */
+static void selu_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, z = a[1].t;
+  enable_gradient(x);
+  kernels::selu_reverse(dkey(z), x.data_ptr(), x.grad_ptr(), z.grad_ptr(), (len_t)x.len(), x.context());
+  z.ptr->launches++;
+}
+
+static void relu_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, z = a[1].t;
+  enable_gradient(x);
+  kernels::relu_reverse(dkey(z), x.data_ptr(), x.grad_ptr(), z.grad_ptr(), (len_t)x.len(), x.context());
+  z.ptr->launches++;
+}
+
+/* One launch writes all four leaf gradients (the four inputs are distinct tensors: materialise
+ * only fuses then). If none of them has a gradient yet the launch creates them (alpha = 0
+ * overwrites); otherwise the missing ones are zero-filled and all four are blended (alpha = 1). */
+static void fused_reverse(const std::vector<OpDatum>& a) {
+  const Tensor ins[4] = {a[0].t, a[1].t, a[2].t, a[3].t};
+  const Tensor te = a[4].t;
+  Graph* g = te.ptr;
+  bool any = false;
+  for (const Tensor& t : ins) any = any || t.has_grad();
+  for (const Tensor& t : ins) {
+    if (any) enable_gradient(t);
+    else t.ptr->grad_of(t) = t.ptr->allocator_.alloc(t.dtype(), t.len(), t.ptr->stream);
+  }
+  kernels::fused_selu_hadamard_add_add_reverse(dkey(te), ins[0].data_ptr(), ins[1].data_ptr(), ins[2].data_ptr(),
+                                               ins[3].data_ptr(), te.grad_ptr(), ins[0].grad_ptr(),
+                                               ins[1].grad_ptr(), ins[2].grad_ptr(), ins[3].grad_ptr(),
+                                               any ? 1.0 : 0.0, (len_t)te.len(), te.context());
+  g->launches++;
+}
+
+static void softmax_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, z = a[1].t;
+  const bool fresh = !x.has_grad();
+  if (fresh) {
+    TensorData& grd = x.ptr->grad_of(x);
+    grd = x.ptr->allocator_.alloc(x.dtype(), x.len(), x.ptr->stream);
+  }
+  const size_t n = z.sizes().back(), m = z.len() / n;
+  kernels::softmax_ij_j_reverse(dkey(z), z.data_ptr(), z.grad_ptr(), x.grad_ptr(), fresh ? 0.0 : 1.0,
+                                (len_t)m, (len_t)n, z.context());
+  z.ptr->launches++;
+}
+
+static void rmsnorm_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, gain = a[1].t, z = a[3].t;
+  const double eps = a[2].s;
+  const bool fresh = !x.has_grad() && !gain.has_grad();
+  if (fresh) {
+    x.ptr->grad_of(x) = x.ptr->allocator_.alloc(x.dtype(), x.len(), x.ptr->stream);
+    gain.ptr->grad_of(gain) = gain.ptr->allocator_.alloc(gain.dtype(), gain.len(), gain.ptr->stream);
+  } else {
+    enable_gradient(x);
+    enable_gradient(gain);
+  }
+  const size_t n = z.sizes().back(), m = z.len() / n;
+  void* scratch = z.stream()->get_scratch(mpRmsnormReverseScratchBytes((len_t)dkey(z), (len_t)m, (len_t)n));
+  kernels::rmsnorm_ij_j_reverse(dkey(z), x.data_ptr(), gain.data_ptr(), z.grad_ptr(), x.grad_ptr(),
+                                gain.grad_ptr(), scratch, eps, fresh ? 0.0 : 1.0, (len_t)m, (len_t)n,
+                                z.context());
+  z.ptr->launches += 2;
+}
+
+namespace ops {
+
+Tensor add(Tensor x, Tensor y) {
+  check_pair(x, y, "add: operands must agree in dtype and sizes");
+  return defer(x.ptr, Pending::add, x, y);
+}
+
+Tensor hadamard(Tensor x, Tensor y) {
+  check_pair(x, y, "hadamard: operands must agree in dtype and sizes");
+  return defer(x.ptr, Pending::hadamard, x, y);
+}
+
+Tensor selu(Tensor x) { return defer(x.ptr, Pending::selu, x, x); }
+
+/* src/ops/relu.zig:13-37 */
+Tensor relu(Tensor x) {
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
+  kernels::relu(dkey(z), px, z.data_ptr(), (len_t)z.len(), z.context());
+  g->launches++;
+  if (g->mode == Mode::train) attach_op(z, relu_reverse, {x, z});
+  return z;
+}
+
+Tensor softmax(Tensor x, const char* expr) {
+  if (std::strcmp(expr, "ij|j") != 0) panic("softmax: only the row form \"ij|j\" exists");
+  if (x.rank() < 1) panic("softmax: tensor has no axis");
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
+  const size_t n = x.sizes().back(), m = x.len() / n;
+  kernels::softmax_ij_j(dkey(z), px, z.data_ptr(), (len_t)m, (len_t)n, z.context());
+  g->launches++;
+  if (g->mode == Mode::train) attach_op(z, softmax_reverse, {x, z});
+  return z;
+}
+
+Tensor rmsnorm(Tensor x, Tensor gain, double eps) {
+  if (x.dtype() != gain.dtype()) panic("rmsnorm: x and gain must agree in dtype");
+  if (gain.len() != x.sizes().back()) panic("rmsnorm: gain must have one entry per column");
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  void* pg = gain.data_ptr();
+  Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
+  const size_t n = x.sizes().back(), m = x.len() / n;
+  kernels::rmsnorm_ij_j(dkey(z), px, pg, z.data_ptr(), eps, (len_t)m, (len_t)n, z.context());
+  g->launches++;
+  if (g->mode == Mode::train) attach_op(z, rmsnorm_reverse, {x, gain, eps, z});
+  return z;
+}
+
+}  // namespace ops
+
+namespace algo {
+
+void fill(Tensor t, double value) {
+  t.ptr->flush(); /* pending nodes may read these bytes */
+  kernels::fill(dkey(t), t.data_ptr(), value, (len_t)t.len(), t.context());
+  t.ptr->launches++;
+}
+
+void copy(Tensor src, Tensor dst) {
+  check_pair(src, dst, "copy: operands must agree in dtype and sizes");
+  dst.ptr->flush();
+  kernels::copy(dkey(src), src.data_ptr(), dst.data_ptr(), (len_t)src.len(), src.context());
+  dst.ptr->launches++;
+}
+
+void sequence(Tensor t, double init, double step) {
+  t.ptr->flush();
+  kernels::sequence(dkey(t), t.data_ptr(), init, step, (len_t)t.len(), t.context());
+  t.ptr->launches++;
+}
+
+}  // namespace algo
+
+namespace util {
+
+void to_device(const void* src, Tensor dst, size_t bytes) {
+  if (bytes != dst.len() * tag_size(dst.dtype())) panic("to_device: byte count does not match the tensor");
+  dst.ptr->flush();
+  mpMemcpyHtoD(dst.data_ptr(), src, bytes, dst.context());
+  mpStreamSynchronize(dst.context()); /* the host buffer may go away right after this call */
+}
+
+void from_device(Tensor src, void* dst, size_t bytes) {
+  if (bytes != src.len() * tag_size(src.dtype())) panic("from_device: byte count does not match the tensor");
+  mpMemcpyDtoH(dst, src.data_ptr(), bytes, src.context());
+}
+
+}  // namespace util
+
+}  // namespace mp
