@@ -25,6 +25,22 @@ HBM_PEAK_GBPS = 8000.0
 SETS = {"cfg1": 16, "cfg2": 4, "cfg3": 2, "cfg4": 2, "cfg5a": 3, "cfg5b": 3, "copy": 2}
 
 
+PROFILE_OF = {"cfg1": "cfg1_softmax", "cfg2": "cfg2_rmsnorm", "cfg3": "cfg3_softmax_r16",
+              "cfg4": "cfg4_fused_chain", "cfg5a": "cfg5a_softmax_vocab", "cfg5b": "cfg5b_softmax_vocab"}
+
+
+def traffic_from_profile(name):
+    """HBM bytes per launch of the dominant launcher, as derived from the rocprofv3 FETCH_SIZE /
+    WRITE_SIZE runs summarised under profiles/ (None when no summary is committed)."""
+    import re
+    path = os.path.join(ROOT, "profiles", f"{PROFILE_OF.get(name, name)}_hbm_traffic.md")
+    if not os.path.exists(path):
+        return None
+    with open(path) as f:
+        m = re.search(r"roofline_traffic_bytes_per_launch\s*=\s*(\d+)", f.read())
+    return int(m.group(1)) if m else None
+
+
 def _events(n):
     import torch
     return [torch.cuda.Event(enable_timing=True) for _ in range(n)]
@@ -182,11 +198,7 @@ def main():
     dom_bytes, dom_name = (w.rev_bytes, "reverse") if w.has_reverse else (w.fwd_bytes, "forward")
     avg_ms = sum(dom_ms) / len(dom_ms)
     achieved = dom_bytes / (avg_ms * 1e-3) / 1e9
-    traffic_path = os.path.join(ROOT, "profiles", f"traffic_{name}.json")
-    traffic = None
-    if os.path.exists(traffic_path):
-        with open(traffic_path) as f:
-            traffic = json.load(f).get("bytes_per_launch")
+    traffic = traffic_from_profile(name)
 
     line = {
         "metric": "achieved HBM GB/s (% of peak) + rows/s, softmax/RMSNorm/elementwise fwd+rev",
