@@ -332,36 +332,50 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
   }
 }
 
-/* dg_j = sum over partial rows (fixed order, fp64) + alpha * dg_j. A workgroup owns 32 columns;
- * its 32 half-wave slices split the partial rows and keep eight loads in flight each. */
-constexpr int FINISH_COLS = 32, FINISH_SLICES = 32;
-template <class T>
-__global__ __launch_bounds__(FINISH_COLS * FINISH_SLICES) void rmsnorm_dgain_finish(
+/* dg_j = sum over partial rows (fixed order, fp64) + alpha * dg_j. A workgroup owns
+ * FINISH_LANES * CW columns; its FINISH_SLICES slices split the partial rows, and a thread keeps
+ * up to eight CW-wide loads in flight (CW = 4 when the partial rows are 16-byte aligned). */
+constexpr int FINISH_LANES = 16, FINISH_SLICES = 64;
+template <class T, int CW>
+__global__ __launch_bounds__(FINISH_LANES * FINISH_SLICES) void rmsnorm_dgain_finish(
     const typename precision<T>::type* partials, T* dg, double alpha, int rows, size_t n) {
   using P = typename precision<T>::type;
-  __shared__ double part[FINISH_SLICES][FINISH_COLS + 1];
-  const int c = threadIdx.x % FINISH_COLS, slice = threadIdx.x / FINISH_COLS;
-  const size_t col = (size_t)blockIdx.x * FINISH_COLS + c;
-  double s = 0.0;
-  if (col < n) {
+  __shared__ double part[FINISH_SLICES][FINISH_LANES * CW + 1];
+  const int c = threadIdx.x % FINISH_LANES, slice = threadIdx.x / FINISH_LANES;
+  const size_t col = ((size_t)blockIdx.x * FINISH_LANES + c) * CW;
+  double s[CW];
+#pragma unroll
+  for (int i = 0; i < CW; ++i) s[i] = 0.0;
+  if (col < n) { /* n is a multiple of CW, so a thread's CW columns are all in range */
     int p = slice;
     for (; p + 7 * FINISH_SLICES < rows; p += 8 * FINISH_SLICES) {
-      P v[8];
+      P v[8][CW];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) v[u] = partials[(size_t)(p + u * FINISH_SLICES) * n + col];
+      for (int u = 0; u < 8; ++u) load_pack<P, CW>(partials + (size_t)(p + u * FINISH_SLICES) * n + col, v[u]);
 #pragma unroll
-      for (int u = 0; u < 8; ++u) s += (double)v[u];
+      for (int u = 0; u < 8; ++u)
+#pragma unroll
+        for (int i = 0; i < CW; ++i) s[i] += (double)v[u][i];
     }
-    for (; p < rows; p += FINISH_SLICES) s += (double)partials[(size_t)p * n + col];
-  }
-  part[slice][c] = s;
-  __syncthreads();
-  if (slice == 0 && col < n) {
-    double t = 0.0;
+    for (; p < rows; p += FINISH_SLICES) {
+      P v[CW];
+      load_pack<P, CW>(partials + (size_t)p * n + col, v);
 #pragma unroll
-    for (int i = 0; i < FINISH_SLICES; ++i) t += part[i][c];
-    if (alpha != 0.0) t += alpha * (double)dg[col];
-    dg[col] = (T)t;
+      for (int i = 0; i < CW; ++i) s[i] += (double)v[i];
+    }
+  }
+#pragma unroll
+  for (int i = 0; i < CW; ++i) part[slice][c * CW + i] = s[i];
+  __syncthreads();
+  /* the first FINISH_LANES * CW threads finish one column each */
+  const int mine = threadIdx.x;
+  const size_t out = (size_t)blockIdx.x * FINISH_LANES * CW + mine;
+  if (mine < FINISH_LANES * CW && out < n) {
+    double t = 0.0;
+#pragma unroll 8
+    for (int i = 0; i < FINISH_SLICES; ++i) t += part[i][mine];
+    if (alpha != 0.0) t += alpha * (double)dg[out];
+    dg[out] = (T)t;
   }
 }
 
@@ -434,8 +448,16 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
     else rmsnorm_rev_stream<T, W, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
   }
   MP_CHECK_LAUNCH();
-  const unsigned fin = (unsigned)((n + FINISH_COLS - 1) / FINISH_COLS);
-  rmsnorm_dgain_finish<T><<<dim3(fin), dim3(FINISH_COLS * FINISH_SLICES), 0, stream>>>(partials, dg, alpha, (int)rows, n);
+  /* wide loads need 16-byte aligned partial rows: fp32 accumulators, n % 4 == 0, aligned scratch */
+  const bool wide = sizeof(P) == 4 && (n % 4) == 0 && aligned16(partials);
+  const dim3 fblock(FINISH_LANES * FINISH_SLICES);
+  if (wide) {
+    const unsigned fin = (unsigned)((n + FINISH_LANES * 4 - 1) / (FINISH_LANES * 4));
+    rmsnorm_dgain_finish<T, 4><<<dim3(fin), fblock, 0, stream>>>(partials, dg, alpha, (int)rows, n);
+  } else {
+    const unsigned fin = (unsigned)((n + FINISH_LANES - 1) / FINISH_LANES);
+    rmsnorm_dgain_finish<T, 1><<<dim3(fin), fblock, 0, stream>>>(partials, dg, alpha, (int)rows, n);
+  }
   MP_CHECK_LAUNCH();
 }
 

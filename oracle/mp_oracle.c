@@ -27,6 +27,8 @@
  *   oracle_reduce_ij_i       src/cuda/nvcc_src/reduce_ij_i.cu:20-32     dst_i = sum_j + alpha*dst_i
  *   oracle_reduce_ij_j       src/cuda/nvcc_src/reduce_ij_j.cu:10-44     dst_j = sum_i + alpha*dst_j (the intent; the
  *                                                                       reference body mis-indexes dst, :42-43)
+ *   oracle_broadcast_i_ij    src/cuda/nvcc_src/broadcast_i_ij.cu:35        dst_ij = src_i + alpha*dst_ij
+ *   oracle_broadcast_j_ij    src/cuda/nvcc_src/broadcast_j_ij.cu:30        dst_ij = src_j + alpha*dst_ij
  *   oracle_selu / _reverse   no reference kernel (only README.md:97); signature and the
  *                            accumulate-into-gradient convention follow relu.cu:11-12 and
  *                            relu_reverse.cu:12-14. Closed form stated below.
@@ -255,6 +257,24 @@ void oracle_reduce_ij_j(int key, const void* src, const void* dst_in, double* ds
     for (size_t i = 0; i < m; ++i) s += ld(key, src, i * n + j);
     dst[j] = s + (dst_in ? alpha * ld(key, dst_in, j) : 0.0);
   }
+}
+
+/* dst[i,j] = src[i] + alpha*dst_in[i,j]  (src/cuda/nvcc_src/broadcast_i_ij.cu:35) */
+void oracle_broadcast_i_ij(int key, const void* src, const void* dst_in, double* dst, double alpha,
+                           size_t m, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < m; ++i)
+    for (size_t j = 0; j < n; ++j)
+      dst[i * n + j] = ld(key, src, i) + (dst_in ? alpha * ld(key, dst_in, i * n + j) : 0.0);
+}
+
+/* dst[i,j] = src[j] + alpha*dst_in[i,j]  (src/cuda/nvcc_src/broadcast_j_ij.cu:30) */
+void oracle_broadcast_j_ij(int key, const void* src, const void* dst_in, double* dst, double alpha,
+                           size_t m, size_t n) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < m; ++i)
+    for (size_t j = 0; j < n; ++j)
+      dst[i * n + j] = ld(key, src, j) + (dst_in ? alpha * ld(key, dst_in, i * n + j) : 0.0);
 }
 
 /* ---- softmax over the last dim -------------------------------------------------------- */

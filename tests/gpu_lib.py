@@ -197,6 +197,11 @@ def fused_reverse(a, b, c, d, de, da, db, dc, dd, alpha=0.0):
           float(alpha), a.numel())
 
 
+def matrix_op(stem, src, dst, alpha, m, n):
+    """reduce_ij_i, reduce_ij_j, broadcast_i_ij, broadcast_j_ij: (src, dst, alpha, m, n)."""
+    _call(stem, src.dtype, src.data_ptr(), dst.data_ptr(), float(alpha), m, n)
+
+
 def softmax(x, y):
     m, n = x.shape
     _call("softmax_ij_j", x.dtype, x.data_ptr(), y.data_ptr(), m, n)

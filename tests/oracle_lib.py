@@ -49,6 +49,8 @@ _fused = _sig("oracle_fused_selu_hadamard_add_add", _it, _vp, _vp, _vp, _vp, _vp
 _fused_rev = _sig("oracle_fused_selu_hadamard_add_add_reverse", _it, *([_vp] * 13), _db, _sz)
 _reduce_i = _sig("oracle_reduce_ij_i", _it, _vp, _vp, _vp, _db, _sz, _sz)
 _reduce_j = _sig("oracle_reduce_ij_j", _it, _vp, _vp, _vp, _db, _sz, _sz)
+_bcast_i = _sig("oracle_broadcast_i_ij", _it, _vp, _vp, _vp, _db, _sz, _sz)
+_bcast_j = _sig("oracle_broadcast_j_ij", _it, _vp, _vp, _vp, _db, _sz, _sz)
 _softmax = _sig("oracle_softmax_ij_j", _it, _vp, _vp, _sz, _sz)
 _softmax_rev = _sig("oracle_softmax_ij_j_reverse", _it, _vp, _vp, _vp, _vp, _db, _sz, _sz)
 _rmsnorm = _sig("oracle_rmsnorm_ij_j", _it, _vp, _vp, _vp, _db, _sz, _sz)
@@ -237,6 +239,20 @@ def reduce_ij_j(src, dst_in=None, alpha=0.0):
     m, n = src.shape
     dst = _out((n,))
     _reduce_j(k, _p(src), _p(dst_in), _p(dst), float(alpha), m, n)
+    return dst
+
+
+def broadcast_i_ij(src, m, n, dst_in=None, alpha=0.0):
+    k, (src, dst_in) = _prep(src, dst_in)
+    dst = _out((m, n))
+    _bcast_i(k, _p(src), _p(dst_in), _p(dst), float(alpha), m, n)
+    return dst
+
+
+def broadcast_j_ij(src, m, n, dst_in=None, alpha=0.0):
+    k, (src, dst_in) = _prep(src, dst_in)
+    dst = _out((m, n))
+    _bcast_j(k, _p(src), _p(dst_in), _p(dst), float(alpha), m, n)
     return dst
 
 

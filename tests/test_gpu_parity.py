@@ -196,6 +196,51 @@ def test_fused_chain_forward_and_reverse(dtype, shift):
             g.check(f"fused n={n}")
 
 
+# ------------------------------------------------------------------ reduce / broadcast
+
+MATRIX_SHAPES = [(1, 1), (3, 2), (2, 2), (7, 5), (33, 64), (64, 1000), (5, 1027), (300, 4096), (2, 50257),
+                 (4100, 36), (2, 20000)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shift", [0, 1])
+def test_reduce_and_broadcast(dtype, shift):
+    r = rng(15)
+    for (m, n) in MATRIX_SHAPES:
+        for alpha in (0.0, 1.0):
+            G.say(f"reduce/broadcast dtype={dtype} shape=({m},{n}) alpha={alpha} shift={shift}")
+            src = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            hs = G.host(src.t)
+            for stem, ref_fn, k in (("reduce_ij_i", O.reduce_ij_i, m), ("reduce_ij_j", O.reduce_ij_j, n)):
+                dst = G.dev(r.normal(0, 1, k), dtype, shift)
+                before = G.host(dst.t).copy()
+                G.matrix_op(stem, src.t, dst.t, alpha, m, n)
+                ref = ref_fn(hs, before if alpha else None, alpha)
+                scale = np.abs(hs.astype(np.float64)).sum(axis=1 if stem == "reduce_ij_i" else 0)
+                G.compare(dst.t, ref, dtype, f"{stem} ({m},{n}) alpha {alpha}", rowwise=False, scale=scale)
+                dst.check(stem)
+            for stem, ref_fn, k in (("broadcast_i_ij", O.broadcast_i_ij, m), ("broadcast_j_ij", O.broadcast_j_ij, n)):
+                vec = G.dev(r.normal(0, 1, k), dtype, shift)
+                dst = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+                before = G.host(dst.t).copy()
+                G.matrix_op(stem, vec.t, dst.t, alpha, m, n)
+                ref = ref_fn(G.host(vec.t), m, n, before if alpha else None, alpha)
+                G.compare(dst.t, ref, dtype, f"{stem} ({m},{n}) alpha {alpha}")
+                dst.check(stem)
+
+
+def test_reference_example_reductions():
+    # src/examples/experimental.zig:19-34
+    f32 = torch.float32
+    x = G.dev(np.array([[1, 2], [3, 4], [5, 6]]), f32)
+    y = G.dev(np.array([[1, 2], [3, 4]]), f32)
+    yi, xj = G.Guarded((2,), f32), G.Guarded((2,), f32)
+    G.say("experimental example: reduce ij->i and ij->j")
+    G.matrix_op("reduce_ij_i", y.t, yi.t, 0.0, 2, 2)
+    G.matrix_op("reduce_ij_j", x.t, xj.t, 0.0, 3, 2)
+    assert yi.t.tolist() == [3.0, 7.0] and xj.t.tolist() == [9.0, 12.0]
+
+
 # ------------------------------------------------------------------ softmax
 
 SOFTMAX_SHAPES = [(1, 1), (3, 7), (5, 64), (4, 65), (9, 256), (7, 1000), (256, 1024), (6, 2048),

@@ -111,6 +111,23 @@ def test_reduce_blend_and_orientation():
     np.testing.assert_allclose(O.reduce_ij_j(src, d_j, -2.0), src.sum(0) - 2.0 * d_j, rtol=1e-14)
 
 
+def test_broadcasts_are_the_reverses_of_the_reductions():
+    m, n = 5, 9
+    src_i, src_j = RNG.normal(0, 1, m), RNG.normal(0, 1, n)
+    old = RNG.normal(0, 1, (m, n))
+    np.testing.assert_allclose(O.broadcast_i_ij(src_i, m, n), np.repeat(src_i[:, None], n, 1), rtol=0)
+    np.testing.assert_allclose(O.broadcast_j_ij(src_j, m, n), np.repeat(src_j[None, :], m, 0), rtol=0)
+    np.testing.assert_allclose(O.broadcast_i_ij(src_i, m, n, old, 1.0), src_i[:, None] + old, rtol=1e-15)
+    np.testing.assert_allclose(O.broadcast_j_ij(src_j, m, n, old, 0.5), src_j[None, :] + 0.5 * old, rtol=1e-15)
+    # autograd: d(sum_j x_ij)/dx = broadcast of the upstream gradient over j
+    xt = t64(old).requires_grad_(True)
+    xt.sum(dim=1).backward(t64(src_i))
+    np.testing.assert_allclose(O.broadcast_i_ij(src_i, m, n), xt.grad.numpy(), rtol=0)
+    xt = t64(old).requires_grad_(True)
+    xt.sum(dim=0).backward(t64(src_j))
+    np.testing.assert_allclose(O.broadcast_j_ij(src_j, m, n), xt.grad.numpy(), rtol=0)
+
+
 def test_selu_closed_form_and_library():
     x = np.concatenate([RNG.uniform(-20, 20, 4000), [0.0, -0.0, 1e-12, -1e-12, -745.0, 700.0]])
     got = O.selu(x)
