@@ -3,14 +3,18 @@
 // dst[i,j] = exp(src[i,j] - max_j src[i,:]) / sum_j exp(src[i,j] - max_j src[i,:]).
 // No reference kernel exists (NOTES.md:28); the (src, dst, m, n) shape follows the row
 // launchers (src/cuda/nvcc_src/reduce_ij_i.cu:35-42) and the "ij|j" name the parser stub of
-// src/ops/expression_parsing.zig:320-340. dst may be src.
+// src/ops/expression_parsing.zig:320-340. dst may be src. scratch is caller-owned workspace of
+// mpSoftmaxScratchBytes(dtype, m, n) bytes (0 for rows that fit one workgroup) that lets several
+// workgroups share a long row; the reference's own softmax call sites already pass a scratch
+// buffer (src/loss/loss.zig:204,226). With scratch == NULL long rows are read twice instead.
 extern "C" void launch_softmax_ij_j_Scalar(
   const void* src,
   void* dst,
+  void* scratch,
   len_t m,
   len_t n,
   StreamContext stream
 ) {
-  mp::softmax_forward<Scalar>(static_cast<const Scalar*>(src), static_cast<Scalar*>(dst), m, n,
+  mp::softmax_forward<Scalar>(static_cast<const Scalar*>(src), static_cast<Scalar*>(dst), scratch, m, n,
                               get_stream(stream));
 }

@@ -3,6 +3,7 @@
  * diagnostic row-regime override. Compiled once (no `Scalar` replication).
  */
 #include "row_rmsnorm.h"
+#include "row_softmax.h"
 
 // Bytes of caller-owned scratch that launch_rmsnorm_ij_j_reverse_<dtype> needs for an [m, n]
 // problem: one row of n accumulators (fp32 for r16/r32, fp64 for r64) per workgroup, at most
@@ -17,10 +18,33 @@ extern "C" len_t mpRmsnormReverseScratchBytes(len_t dtype, len_t m, len_t n) {
   }
 }
 
+// Bytes of caller-owned scratch that launch_softmax_ij_j_<dtype> can use for an [m, n] problem:
+// two accumulator words per workgroup of a row that is shared by several workgroups, 0 when a
+// row fits one workgroup. Passing NULL instead is allowed and costs a second read of long rows.
+extern "C" len_t mpSoftmaxScratchBytes(len_t dtype, len_t m, len_t n) {
+  switch (dtype) {
+    case MP_R16: return mp::softmax_scratch_bytes<r16>(m, n);
+    case MP_R32: return mp::softmax_scratch_bytes<r32>(m, n);
+    case MP_R64: return mp::softmax_scratch_bytes<r64>(m, n);
+    default: mp::require(false, "mpSoftmaxScratchBytes: dtype must be 0, 1 or 2"); return 0;
+  }
+}
+
 // Diagnostic: force the row regime of the softmax / RMSNorm launchers (0 auto; 1..5 = groups of
-// 64, 128, 256, 512, 1024 threads per row; 6 = streaming). A group that cannot hold a row falls
-// through to the next wider one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
+// 64, 128, 256, 512, 1024 threads per row; 6 = streaming; 7 = cluster path of the softmax
+// forward). A group that cannot hold a row falls through to the next wider one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
 extern "C" void mpSetRowRegime(len_t regime) {
-  mp::require(regime <= mp::REGIME_STREAM, "mpSetRowRegime: regime must be 0..6");
+  mp::require(regime <= mp::REGIME_CLUSTER, "mpSetRowRegime: regime must be 0..7");
   mp::row_regime_override() = (int)regime;
+}
+
+// Diagnostic: packs (16-byte units) of a row handled per workgroup on the cluster path of the
+// softmax forward (0 = default, one pack per thread less than the register tile; larger values
+// are clipped to the tile) and the number of polls a workgroup
+// waits for its partners before it folds the row itself. Tests set a tiny spin limit to drive
+// that second path. Process-wide, like mpSetRowRegime.
+extern "C" void mpSetClusterTuning(len_t packs_per_block, len_t spin_limit) {
+  mp::require(packs_per_block <= 0x7fffffffull, "mpSetClusterTuning: packs_per_block out of range");
+  mp::cluster_tuning().packs_per_block = (int)packs_per_block;
+  mp::cluster_tuning().spin_limit = (unsigned)spin_limit;
 }

@@ -22,9 +22,10 @@
 
 namespace mp {
 
-/* 0 = automatic; 1..5 force G = 64, 128, 256, 512, 1024; 6 forces the streaming kernels. */
+/* 0 = automatic; 1..5 force G = 64, 128, 256, 512, 1024; 6 forces the streaming kernels;
+ * 7 forces the cluster path of the softmax forward (the other launchers treat it as automatic). */
 enum RowRegime { REGIME_AUTO = 0, REGIME_G64 = 1, REGIME_G128 = 2, REGIME_G256 = 3, REGIME_G512 = 4,
-                 REGIME_G1024 = 5, REGIME_STREAM = 6 };
+                 REGIME_G1024 = 5, REGIME_STREAM = 6, REGIME_CLUSTER = 7 };
 
 /* Diagnostic override set through mpSetRowRegime; AUTO in normal use. */
 inline int& row_regime_override() {
@@ -50,7 +51,8 @@ struct RowPlan {
 /* nv_target: packs per thread the automatic plan aims for before it widens the group. */
 inline RowPlan plan_row(size_t packs, int max_nv, int nv_target) {
   static const int group_of[] = {0, 64, 128, 256, 512, 1024};
-  const int forced = row_regime_override();
+  int forced = row_regime_override();
+  if (forced == REGIME_CLUSTER) forced = REGIME_AUTO;
   if (forced == REGIME_STREAM) return RowPlan{0, 0};
   if (forced == REGIME_AUTO) {
     const int want = nv_target < max_nv ? nv_target : max_nv;

@@ -11,8 +11,11 @@
  *
  * Resident kernels read each row once, keep it in registers across both reductions and write
  * it once; the reverse folds dot(y, dy) and the gradient write into the same pass over
- * registers. Streaming kernels cover rows too long for registers with one online max/sum pass
- * (running maximum, running sum rescaled whenever the maximum moves) and one write pass.
+ * registers. Rows longer than one workgroup's registers are shared by a cluster of consecutive
+ * workgroups that exchange their (max, sum) through caller-owned scratch, still reading the row
+ * once. Streaming kernels cover what is left (no scratch given, or rows beyond a cluster) with
+ * one online max/sum pass (running maximum, running sum rescaled whenever the maximum moves)
+ * and one write pass that re-reads the row.
  */
 #ifndef MP_ROW_SOFTMAX_H
 #define MP_ROW_SOFTMAX_H
@@ -120,6 +123,51 @@ template <class P> __device__ __forceinline__ void online_rescale(P& run_max, P&
   }
 }
 
+/* One lane's share of a row folded online: running maximum and the sum of exp(x - maximum),
+ * rescaled whenever the maximum moves. G threads stride the packs, U loads in flight. */
+template <class T, int W, int G, int U>
+__device__ __forceinline__ void row_online_max_sum(const T* xr, const RowGeom<T, W>& g, int lane,
+                                                   typename precision<T>::type& run_max,
+                                                   typename precision<T>::type& run_sum) {
+  using P = typename precision<T>::type;
+  const T* body = xr + g.head;
+  run_max = neg_inf<P>();
+  run_sum = (P)0;
+  for (int p0 = lane; p0 < g.nvec; p0 += G * U) {
+    P buf[U][W];
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int p = p0 + u * G;
+      if (p < g.nvec) {
+        load_pack<T, W>(body + (size_t)p * W, buf[u]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) buf[u][i] = neg_inf<P>();
+      }
+    }
+    P cm = neg_inf<P>();
+#pragma unroll
+    for (int u = 0; u < U; ++u)
+#pragma unroll
+      for (int i = 0; i < W; ++i) cm = buf[u][i] > cm ? buf[u][i] : cm;
+    online_rescale(run_max, run_sum, cm);
+    if (run_max > neg_inf<P>()) {
+      const P sh = shift_of(run_max);
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < W; ++i) run_sum += exp_shifted(buf[u][i], sh);
+    }
+  }
+  if (W > 1) {
+    P e = neg_inf<P>();
+    if (lane < g.head) e = (P)xr[lane];
+    else if (lane - g.head < g.tail) e = (P)body[(size_t)g.nvec * W + (lane - g.head)];
+    online_rescale(run_max, run_sum, e);
+    if (e > neg_inf<P>()) run_sum += exp_shifted(e, shift_of(run_max));
+  }
+}
+
 template <class T, int W>
 __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
     const T* x, T* y, size_t m, size_t n) {
@@ -136,40 +184,8 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
     const T* body = xr + g.head;
 
     /* pass 1: online max / sum */
-    P run_max = neg_inf<P>(), run_sum = (P)0;
-    for (int p0 = lane; p0 < g.nvec; p0 += G * U) {
-      P buf[U][W];
-#pragma unroll
-      for (int u = 0; u < U; ++u) {
-        const int p = p0 + u * G;
-        if (p < g.nvec) {
-          load_pack<T, W>(body + (size_t)p * W, buf[u]);
-        } else {
-#pragma unroll
-          for (int i = 0; i < W; ++i) buf[u][i] = neg_inf<P>();
-        }
-      }
-      P cm = neg_inf<P>();
-#pragma unroll
-      for (int u = 0; u < U; ++u)
-#pragma unroll
-        for (int i = 0; i < W; ++i) cm = buf[u][i] > cm ? buf[u][i] : cm;
-      online_rescale(run_max, run_sum, cm);
-      if (run_max > neg_inf<P>()) {
-        const P sh = shift_of(run_max);
-#pragma unroll
-        for (int u = 0; u < U; ++u)
-#pragma unroll
-          for (int i = 0; i < W; ++i) run_sum += exp_shifted(buf[u][i], sh);
-      }
-    }
-    if (W > 1) {
-      P e = neg_inf<P>();
-      if (lane < g.head) e = (P)xr[lane];
-      else if (lane - g.head < g.tail) e = (P)body[(size_t)g.nvec * W + (lane - g.head)];
-      online_rescale(run_max, run_sum, e);
-      if (e > neg_inf<P>()) run_sum += exp_shifted(e, shift_of(run_max));
-    }
+    P run_max, run_sum;
+    row_online_max_sum<T, W, G, 4>(xr, g, lane, run_max, run_sum);
 
     const P mx = group_allreduce<MaxOP, G>(run_max, slots[parity][0], lane);
     const P sh = shift_of(mx);
@@ -204,6 +220,185 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
       }
     }
   }
+}
+
+/* ------------------------------------------------------------------ cluster forward */
+
+/* Rows too long for one workgroup's registers but short enough for a few: C consecutive
+ * workgroups share a row. Each keeps its chunk in registers, publishes its (max, sum) through
+ * two agent-scope atomic words in caller-owned scratch, waits for the other C-1, and writes its
+ * chunk: the row is still read once and written once.
+ *
+ * A published word is never zero (a maximum of +0 is stored as -0; the sum of a chunk without a
+ * finite entry is stored as 1 and ignored through its -inf maximum), so "non-zero" means
+ * "published" and the scratch only has to be zero when the kernel starts (cluster_zero_slots).
+ *
+ * Waiting is bounded. Workgroups of one row have consecutive indices and a workgroup publishes
+ * before it waits, so with in-order dispatch the wait is short; if spin_limit polls pass
+ * anyway, the workgroup stops waiting and folds the whole row itself (one extra read of the row),
+ * so every wave reaches the end whatever the scheduling. */
+constexpr int CLUSTER_THREADS = 1024, CLUSTER_MAX = WAVE;
+/* packs per thread: 24 registers of row data, so that two workgroups fit a CU (64 registers) */
+template <class T> constexpr int cluster_nv() {
+  return 24 / ((PACK_BYTES / (int)sizeof(T)) * (int)(sizeof(typename precision<T>::type) / 4));
+}
+
+template <class P> struct slot_word { using type = unsigned; };
+template <> struct slot_word<double> { using type = unsigned long long; };
+
+template <class T, int W>
+__global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
+    const T* x, T* y, typename slot_word<typename precision<T>::type>::type* slots,
+    size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
+  using P = typename precision<T>::type;
+  using Word = typename slot_word<P>::type;
+  constexpr int G = CLUSTER_THREADS, NV = cluster_nv<T>();
+  __shared__ P red[4][G / WAVE];
+  __shared__ P bc[3];
+  const int lane = threadIdx.x;
+  const size_t row = blockIdx.x / (unsigned)C;
+  const int rank = (int)(blockIdx.x % (unsigned)C);
+  const T* xr = x + row * n;
+  T* yr = y + row * n;
+  const RowGeom<T, W> g(xr, n, true);
+  const T* body = xr + g.head;
+  const int lo = rank * packs_per_block;
+  const int hi = lo + packs_per_block < g.nvec ? lo + packs_per_block : g.nvec;
+
+  /* this workgroup's chunk; rank 0 also holds the row's head / tail scalars */
+  P v[NV][W];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = lo + k * G + lane;
+    if (p < hi) {
+      load_pack_nt<T, W>(body + (size_t)p * W, v[k]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[k][i] = neg_inf<P>();
+    }
+  }
+  P edge = neg_inf<P>();
+  size_t edge_at = (size_t)-1;
+  if (W > 1 && rank == 0) {
+    if (lane < g.head) edge_at = (size_t)lane;
+    else if (lane - g.head < g.tail) edge_at = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
+    if (edge_at != (size_t)-1) edge = (P)xr[edge_at];
+  }
+
+  P mx = edge;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) mx = v[k][i] > mx ? v[k][i] : mx;
+  mx = group_allreduce<MaxOP, G>(mx, red[0], lane);
+  /* a chunk without a finite entry (fully masked) contributes exact zeros, not exp(-inf + inf) */
+  const P sh = shift_of(mx > neg_inf<P>() ? mx : (P)0);
+  P s = (P)0;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      v[k][i] = exp_shifted(v[k][i], sh);
+      s += v[k][i];
+    }
+  edge = exp_shifted(edge, sh);
+  s += edge;
+  s = group_allreduce<AddOP, G>(s, red[1], lane);
+
+  P M = mx, S = s;
+  if (C > 1) {
+    Word* mine = slots + ((size_t)row * C + rank) * 2;
+    if (lane == 0) {
+      const P pm = mx == (P)0 ? -(P)0 : mx;
+      const P ps = mx > neg_inf<P>() ? s : (P)1;
+      __hip_atomic_store(mine + 0, __builtin_bit_cast(Word, pm), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(mine + 1, __builtin_bit_cast(Word, ps), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (lane < WAVE) { /* wave 0: lane b waits for workgroup b of this row */
+      P om = neg_inf<P>(), os = (P)0;
+      bool ok = true;
+      if (lane < C) {
+        Word* theirs = slots + ((size_t)row * C + lane) * 2;
+        Word a = 0, b = 0;
+        for (unsigned spins = 0;; ++spins) {
+          a = __hip_atomic_load(theirs + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          b = __hip_atomic_load(theirs + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if ((a != 0 && b != 0) || spins >= spin_limit) break;
+          __builtin_amdgcn_s_sleep(4);
+        }
+        ok = a != 0 && b != 0;
+        om = __builtin_bit_cast(P, a);
+        os = __builtin_bit_cast(P, b);
+      }
+      const P all_ok = wave_allreduce<AddOP>(ok ? (P)0 : (P)1); /* every lane takes part */
+      const P gm = wave_allreduce<MaxOP>(ok ? om : neg_inf<P>());
+      const P part = (lane < C && ok && om > neg_inf<P>()) ? os * exp_shifted(om, shift_of(gm)) : (P)0;
+      const P gs = wave_allreduce<AddOP>(part);
+      if (lane == 0) {
+        bc[0] = gm;
+        bc[1] = gs;
+        bc[2] = all_ok;
+      }
+    }
+    __syncthreads();
+    M = bc[0];
+    S = bc[1];
+    if (bc[2] != (P)0) { /* gave up waiting: fold the whole row here */
+      P run_max, run_sum;
+      row_online_max_sum<T, W, G, 1>(xr, g, lane, run_max, run_sum); /* rare path: keep it lean */
+      M = group_allreduce<MaxOP, G>(run_max, red[2], lane);
+      const P scaled = run_max > neg_inf<P>() ? run_sum * exp_shifted(run_max, shift_of(M)) : (P)0;
+      S = group_allreduce<AddOP, G>(scaled, red[3], lane);
+    }
+  }
+
+  const P scale = exp_shifted(mx, shift_of(M)) / S;
+  T* ybody = yr + g.head;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = lo + k * G + lane;
+    if (p < hi) {
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[k][i] *= scale;
+      store_pack_nt<T, W>(ybody + (size_t)p * W, v[k]);
+    }
+  }
+  if (edge_at != (size_t)-1) yr[edge_at] = (T)(edge * scale);
+}
+
+template <class Word> __global__ __launch_bounds__(256) void cluster_zero_slots(Word* slots, size_t words) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < words) slots[i] = 0;
+}
+
+/* Diagnostic knobs of the cluster path (set through mpSetClusterTuning). */
+struct ClusterTuning {
+  int packs_per_block = 0; /* 0: one pack per thread less than the register tile holds */
+  unsigned spin_limit = 1u << 22;
+};
+inline ClusterTuning& cluster_tuning() {
+  static ClusterTuning t;
+  return t;
+}
+
+/* Workgroups per row on the cluster path; 0 when the row does not take it. */
+template <class T> inline int cluster_size(size_t packs) {
+  const int regime = row_regime_override();
+  if (regime != REGIME_AUTO && regime != REGIME_CLUSTER) return 0;
+  if (regime == REGIME_AUTO && packs <= (size_t)CLUSTER_THREADS * 2) return 0; /* one workgroup, two packs each */
+  constexpr size_t tile = (size_t)CLUSTER_THREADS * cluster_nv<T>();
+  size_t ppb = (size_t)cluster_tuning().packs_per_block;
+  if (ppb == 0) ppb = tile - CLUSTER_THREADS;
+  if (ppb > tile) ppb = tile;
+  const size_t c = (packs + ppb - 1) / ppb;
+  return c >= 1 && c <= (size_t)CLUSTER_MAX ? (int)c : 0;
+}
+
+template <class T> inline size_t softmax_scratch_bytes(size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  const int c = cluster_size<T>((n + W - 1) / W);
+  return c > 1 ? m * (size_t)c * 2 * sizeof(P) : 0;
 }
 
 /* ------------------------------------------------------------------ streaming reverse */
@@ -296,8 +491,9 @@ inline unsigned stream_grid(size_t m) {
 }
 
 template <class T>
-inline void softmax_forward(const T* x, T* y, size_t m, size_t n, hipStream_t stream) {
+inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n, hipStream_t stream) {
   if (m == 0 || n == 0) return;
+  using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "softmax: row length must not exceed 2^30");
   if (misalign16(x) != misalign16(y)) { /* rows of x and y peel differently: element-wise */
@@ -305,9 +501,28 @@ inline void softmax_forward(const T* x, T* y, size_t m, size_t n, hipStream_t st
     MP_CHECK_LAUNCH();
     return;
   }
+  const size_t packs = (n + W - 1) / W;
+  const int C = cluster_size<T>(packs);
+  /* in place, a workgroup that gives up waiting would re-read chunks its partners already
+   * overwrote: shared rows need distinct buffers */
+  const bool shareable = scratch != nullptr && static_cast<const void*>(x) != static_cast<const void*>(y);
+  if (C >= 1 && (C == 1 || shareable) && m * (size_t)C < 0x7fffffffull) {
+    using Word = typename slot_word<P>::type;
+    Word* slots = static_cast<Word*>(scratch);
+    const int ppb = (int)((packs + C - 1) / C);
+    require(ppb <= CLUSTER_THREADS * cluster_nv<T>(), "softmax: cluster chunk exceeds the register tile");
+    if (C > 1) {
+      const size_t words = m * (size_t)C * 2;
+      cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
+    }
+    softmax_fwd_cluster<T, W><<<dim3((unsigned)(m * C)), dim3(CLUSTER_THREADS), 0, stream>>>(
+        x, y, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+    MP_CHECK_LAUNCH();
+    return;
+  }
   const bool ragged = !(aligned16(x) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(64);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 2);
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2);
   const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m)), block(G);
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n);

@@ -490,7 +490,9 @@ Tensor softmax(Tensor x, const char* expr) {
   void* px = x.data_ptr();
   Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
   const size_t n = x.sizes().back(), m = x.len() / n;
-  kernels::softmax_ij_j(dkey(z), px, z.data_ptr(), (len_t)m, (len_t)n, z.context());
+  const len_t bytes = mpSoftmaxScratchBytes((len_t)dkey(z), (len_t)m, (len_t)n);
+  void* scratch = bytes ? z.stream()->get_scratch(bytes) : nullptr;
+  kernels::softmax_ij_j(dkey(z), px, z.data_ptr(), scratch, (len_t)m, (len_t)n, z.context());
   g->launches++;
   if (g->mode == Mode::train) attach_op(z, softmax_reverse, {x, z});
   return z;

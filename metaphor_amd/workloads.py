@@ -32,9 +32,17 @@ def _launch(stem, dtype, *args):
 
 # ------------------------------------------------------------------ launch wrappers
 
-def softmax_forward(x, y):
+def softmax_scratch(dtype, m, n):
+    """Workspace for launch_softmax_ij_j (None when the rows fit one workgroup)."""
+    kernels, _ = ffi.load()
+    nbytes = int(kernels.mpSoftmaxScratchBytes(KEY[dtype], m, n))
+    return torch.empty(nbytes, dtype=torch.uint8, device="cuda") if nbytes else None
+
+
+def softmax_forward(x, y, scratch=None):
     m, n = x.shape
-    _launch("softmax_ij_j", x.dtype, x.data_ptr(), y.data_ptr(), m, n)
+    _launch("softmax_ij_j", x.dtype, x.data_ptr(), y.data_ptr(),
+            scratch.data_ptr() if scratch is not None else None, m, n)
 
 
 def softmax_reverse(y, dy, dx, alpha=0.0):
@@ -209,12 +217,13 @@ class _Vocab(Workload):
         spike = torch.randint(0, n, (m,), generator=g, device="cuda")
         self.x[torch.arange(m, device="cuda"), spike] += 12.0
         self.y = torch.empty_like(self.x)
+        self.scratch = softmax_scratch(torch.float32, m, n)
         self.rows = m
         self.fwd_bytes = 2 * m * n * 4
         self.rev_bytes = 0
 
     def forward(self):
-        softmax_forward(self.x, self.y)
+        softmax_forward(self.x, self.y, self.scratch)
 
 
 class Cfg5a(_Vocab):

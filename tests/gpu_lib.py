@@ -202,9 +202,24 @@ def matrix_op(stem, src, dst, alpha, m, n):
     _call(stem, src.dtype, src.data_ptr(), dst.data_ptr(), float(alpha), m, n)
 
 
-def softmax(x, y):
+def softmax_scratch(dtype, m, n):
+    kernels, _ = lib()
+    nbytes = int(kernels.mpSoftmaxScratchBytes(KEY[dtype], m, n))
+    return (Guarded((nbytes,), torch.uint8) if nbytes else None), nbytes
+
+
+def softmax(x, y, scratch="auto"):
+    """scratch: "auto" sizes and passes the workspace the launcher asks for, None passes NULL."""
     m, n = x.shape
-    _call("softmax_ij_j", x.dtype, x.data_ptr(), y.data_ptr(), m, n)
+    guard = None
+    if isinstance(scratch, str):
+        guard, _ = softmax_scratch(x.dtype, m, n)
+        scratch = guard.t if guard is not None else None
+    _call("softmax_ij_j", x.dtype, x.data_ptr(), y.data_ptr(),
+          scratch.data_ptr() if scratch is not None else None, m, n)
+    if guard is not None:
+        torch.cuda.synchronize()
+        guard.check("softmax scratch")
 
 
 def softmax_reverse(y, dy, dx, alpha=0.0):
@@ -232,3 +247,8 @@ def rmsnorm_reverse(x, g, dy, dx, dg, scratch, eps, alpha=0.0):
 def set_regime(r):
     kernels, _ = lib()
     kernels.mpSetRowRegime(int(r))
+
+
+def set_cluster_tuning(packs_per_block=0, spin_limit=1 << 22):
+    kernels, _ = lib()
+    kernels.mpSetClusterTuning(int(packs_per_block), int(spin_limit))

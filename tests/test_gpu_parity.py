@@ -13,14 +13,16 @@ pytestmark = pytest.mark.gpu
 
 DTYPES = [torch.float16, torch.float32, torch.float64]
 IDS = ["r16", "r32", "r64"]
-REGIMES = [0, 1, 2, 3, 4, 5, 6]  # auto, G = 64/128/256/512/1024, stream
+REGIMES = [0, 1, 2, 3, 4, 5, 6, 7]  # auto, G = 64/128/256/512/1024, stream, cluster (softmax forward)
 
 
 @pytest.fixture(autouse=True)
 def _auto_regime():
     G.set_regime(0)
+    G.set_cluster_tuning()
     yield
     G.set_regime(0)
+    G.set_cluster_tuning()
     torch.cuda.synchronize()
 
 
@@ -295,6 +297,45 @@ def test_softmax_unaligned_bases_and_in_place(dtype, regime):
         G.softmax(x.t, x.t)
         G.compare(x.t, ref, dtype, f"softmax in place ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
         x.check("in place")
+
+
+CLUSTER = 7
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("packs,spin", [(0, 1 << 22), (64, 1 << 22), (3, 1 << 22), (64, 0), (1000, 2)],
+                         ids=["default", "64packs", "3packs", "64packs-nowait", "1000packs-2polls"])
+def test_softmax_forward_cluster_path(dtype, packs, spin):
+    """Several workgroups per row with the (max, sum) exchange through scratch. A spin limit of 0
+    or 2 polls makes most workgroups give up waiting and fold the whole row themselves: every
+    kernel still ends and the results stay within tolerance."""
+    r = rng(32)
+    G.set_regime(CLUSTER)
+    G.set_cluster_tuning(packs, spin)
+    for (m, n) in [(3, 7), (5, 64), (4, 1000), (6, 2048), (33, 5000), (2, 50257), (2, 151936), (130, 777)]:
+        for masked in (False, True):
+            for shift in (0, 1):
+                G.say(f"softmax cluster dtype={dtype} packs={packs} spin={spin} shape=({m},{n}) masked={masked} shift={shift}")
+                x = G.dev(_softmax_inputs(r, m, n, dtype, masked), dtype, shift)
+                y = G.Guarded((m, n), dtype, shift)
+                G.softmax(x.t, y.t)
+                ref = O.softmax_ij_j(G.host(x.t))
+                G.compare(y.t, ref, dtype, f"softmax cluster ({m},{n}) packs {packs} spin {spin}",
+                          atol=G.SOFTMAX_ATOL[dtype])
+                if masked:
+                    assert bool((y.t[torch.isinf(x.t)] == 0).all())
+                x.check("x")
+                y.check("y")
+
+
+def test_softmax_long_rows_without_scratch_take_the_two_pass_kernel():
+    r = rng(33)
+    for (m, n) in [(3, 151936), (4, 50257)]:
+        x = G.dev(r.normal(0, 3, (m, n)), torch.float32)
+        y = G.Guarded((m, n), torch.float32)
+        G.say(f"softmax NULL scratch ({m},{n})")
+        G.softmax(x.t, y.t, scratch=None)
+        G.compare(y.t, O.softmax_ij_j(G.host(x.t)), torch.float32, f"no scratch ({m},{n})", atol=1e-6)
 
 
 def test_softmax_vocabulary_spike_rows_r32():
