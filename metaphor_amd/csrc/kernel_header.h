@@ -236,22 +236,34 @@ template <class OP, class P> __device__ __forceinline__ P wave_allreduce(P v) {
   return fold_rows<OP>(v);
 }
 
+/* NW per-wave partials, one per lane with index lane % NW, folded so that every lane holds the
+ * result: a DPP butterfly over NW <= 16 neighbouring lanes. Every lane applies OP over the same
+ * tree with commuted operands, so all lanes agree bit for bit. */
+template <class OP, int NW, class P> __device__ __forceinline__ P fold_partials(P v) {
+  static_assert(NW >= 1 && NW <= 16 && (NW & (NW - 1)) == 0, "partials per group: a power of two up to 16");
+  if constexpr (NW >= 2) v = OP::apply(v, dpp_move<DPP_XOR1>(v));
+  if constexpr (NW >= 4) v = OP::apply(v, dpp_move<DPP_XOR2>(v));
+  if constexpr (NW >= 8) v = OP::apply(v, dpp_move<DPP_HALF_MIRROR>(v));
+  if constexpr (NW >= 16) v = OP::apply(v, dpp_move<DPP_MIRROR>(v));
+  return v;
+}
+
 /* Every thread of a G-thread group (G/64 consecutive waves of the workgroup) returns OP
  * folded over the group. `slots` points at the group's G/64 LDS words for THIS reduction;
  * two reductions in flight must use different slots, and a loop that reuses slots must
- * alternate between two sets, which makes the single barrier below sufficient. */
+ * alternate between two sets, which makes the single barrier below sufficient. After the
+ * barrier each lane reads ONE partial (a conflict-free multicast) and the partials are folded
+ * across lanes, instead of every lane reading and adding all of them. */
 template <class OP, int G, class P>
 __device__ __forceinline__ P group_allreduce(P v, P* slots, int lane_in_group) {
   v = wave_allreduce<OP>(v);
   if constexpr (G == WAVE) {
     return v;
   } else {
+    constexpr int NW = G / WAVE;
     if ((lane_in_group & (WAVE - 1)) == 0) slots[lane_in_group / WAVE] = v;
     __syncthreads();
-    P r = slots[0];
-#pragma unroll
-    for (int i = 1; i < G / WAVE; ++i) r = OP::apply(r, slots[i]);
-    return r;
+    return fold_partials<OP, NW>(slots[lane_in_group & (NW - 1)]);
   }
 }
 

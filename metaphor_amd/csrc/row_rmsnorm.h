@@ -37,13 +37,9 @@ __device__ __forceinline__ void group_allreduce_sum2(P& a, P& b, P* slots_a, P* 
       slots_b[lane / WAVE] = b;
     }
     __syncthreads();
-    a = slots_a[0];
-    b = slots_b[0];
-#pragma unroll
-    for (int i = 1; i < G / WAVE; ++i) {
-      a += slots_a[i];
-      b += slots_b[i];
-    }
+    constexpr int NW = G / WAVE;
+    a = fold_partials<AddOP, NW>(slots_a[lane & (NW - 1)]);
+    b = fold_partials<AddOP, NW>(slots_b[lane & (NW - 1)]);
   }
 }
 
