@@ -117,6 +117,11 @@ template <class P> __device__ __forceinline__ P selu_slope(P x) {
   return x > (P)0 ? lam : neg;
 }
 
+/* relu with the reference's convention: zero counts as positive (src/cuda/nvcc_src/relu.cu:12,
+ * relu_reverse.cu:14) */
+template <class P> __device__ __forceinline__ P relu_value(P x) { return x >= (P)0 ? x : (P)0; }
+template <class P> __device__ __forceinline__ P relu_slope(P x) { return x >= (P)0 ? (P)1 : (P)0; }
+
 /* ---------------------------------------------------------------------------------------
  * 128-bit packs
  * ------------------------------------------------------------------------------------- */

@@ -158,6 +158,44 @@ static int fused_chain(mp::Stream stream) {
   f.reverse(mp::ReverseCleanup::keep);
   dump("rep_da", a.native_grad<float>()); dump("rep_dc", c.native_grad<float>());
 
+  /* other entries of the generated chain table: one kernel forward, one kernel reverse each */
+  G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+  {
+    size_t l = G->launches;
+    mp::Tensor p = mp::ops::hadamard(mp::ops::add(a, b), mp::ops::add(c, d));
+    dump("chain_mul_add_add", p.native<float>());
+    CHECK(G->launches == l + 1);
+    l = G->launches;
+    p.reverse(mp::ReverseCleanup::free);
+    CHECK(G->launches == l + 2);
+    dump("chain_mul_add_add_da", a.native_grad<float>()); dump("chain_mul_add_add_dd", d.native_grad<float>());
+
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+    l = G->launches;
+    mp::Tensor q = mp::ops::selu(mp::ops::hadamard(mp::ops::sub(a, b), c));
+    dump("chain_selu_mul_sub", q.native<float>());
+    CHECK(G->launches == l + 1);
+    q.reverse(mp::ReverseCleanup::free);
+    dump("chain_selu_mul_sub_da", a.native_grad<float>()); dump("chain_selu_mul_sub_db", b.native_grad<float>());
+    dump("chain_selu_mul_sub_dc", c.native_grad<float>());
+
+    /* not in the table as a whole: relu is eager, its operand selu(add(a,b)) is a chain */
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+    l = G->launches;
+    mp::Tensor r2 = mp::ops::relu(mp::ops::selu(mp::ops::add(a, b)));
+    dump("chain_relu_selu_add", r2.native<float>());
+    CHECK(G->launches == l + 2);
+    r2.reverse(mp::ReverseCleanup::free);
+    dump("chain_relu_selu_add_da", a.native_grad<float>());
+
+    /* sub alone is not a chain: per-op kernel and the per-op reverse (gx += gz, gy -= gz) */
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+    mp::Tensor s2 = mp::ops::sub(a, b);
+    dump("plain_sub", s2.native<float>());
+    s2.reverse(mp::ReverseCleanup::free);
+    dump("plain_sub_da", a.native_grad<float>()); dump("plain_sub_db", b.native_grad<float>());
+  }
+
   /* eval mode attaches nothing and reverse is refused by construction: only forward here */
   mp::Graph* E = mp::Graph::init({stream, mp::Mode::eval});
   mp::Tensor ea = leaf(E, mp::TensorClass::inp, {n}, ha), eb = leaf(E, mp::TensorClass::inp, {n}, hb);

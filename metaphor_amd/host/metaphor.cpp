@@ -11,6 +11,7 @@
 #include <cstring>
 #include <mutex>
 
+#include "chains.hpp"
 #include "kernels.hpp"
 
 namespace mp {
@@ -292,9 +293,53 @@ Tensor defer(Graph* g, Pending op, Tensor x, Tensor y) {
 }
 
 static void addition_reverse(const std::vector<OpDatum>& a);
+static void subtraction_reverse(const std::vector<OpDatum>& a);
 static void hadamard_reverse(const std::vector<OpDatum>& a);
 static void selu_reverse(const std::vector<OpDatum>& a);
-static void fused_reverse(const std::vector<OpDatum>& a);
+static void chain_reverse(const std::vector<OpDatum>& a);
+
+static const char* pending_name(Pending op) {
+  switch (op) {
+    case Pending::add: return "add";
+    case Pending::sub: return "sub";
+    case Pending::hadamard: return "mul";
+    case Pending::selu: return "selu";
+    default: return "?";
+  }
+}
+
+/* The expression below t, as the chain table spells it: pending nodes of this graph become
+ * op(...), everything else a leaf numbered in order of first appearance (the same tensor keeps
+ * its number). Gives up (returns false) beyond eight leaves or 64 nodes. */
+static bool spell(Graph* g, Tensor t, std::string& out, std::vector<Tensor>& leaves, int& budget) {
+  if (--budget < 0) return false;
+  if (is_pending(t) && t.ptr == g) {
+    const Graph::Node& node = g->nodes_[t.idx];
+    out += pending_name(node.pending);
+    out += '(';
+    if (!spell(g, node.in0, out, leaves, budget)) return false;
+    if (node.pending != Pending::selu) {
+      out += ',';
+      if (!spell(g, node.in1, out, leaves, budget)) return false;
+    }
+    out += ')';
+    return true;
+  }
+  size_t k = 0;
+  while (k < leaves.size() && !leaves[k].same(t)) ++k;
+  if (k == leaves.size()) {
+    if (leaves.size() == 8) return false;
+    leaves.push_back(t);
+  }
+  out += std::to_string(k);
+  return true;
+}
+
+static const FusedChain* find_chain(const std::string& signature) {
+  for (const FusedChain& c : fused_chains)
+    if (signature == c.signature) return &c;
+  return nullptr;
+}
 
 void materialise(Tensor t) {
   if (!is_pending(t)) return;
@@ -313,31 +358,34 @@ void materialise(Tensor t) {
     return d.ptr;
   };
 
-  /* selu(hadamard(add(a,b), add(c,d))) with the three inner nodes still pending and owned by
-   * the same graph: one launch, and the inner nodes stay unmaterialised */
-  if (op == Pending::selu && is_pending(in0) && in0.ptr == g && g->nodes_[in0.idx].pending == Pending::hadamard) {
-    const Tensor u = g->nodes_[in0.idx].in0, v = g->nodes_[in0.idx].in1;
-    if (is_pending(u) && is_pending(v) && u.ptr == g && v.ptr == g && !u.same(v) &&
-        g->nodes_[u.idx].pending == Pending::add && g->nodes_[v.idx].pending == Pending::add) {
-      const Tensor a = g->nodes_[u.idx].in0, b = g->nodes_[u.idx].in1;
-      const Tensor c = g->nodes_[v.idx].in0, d = g->nodes_[v.idx].in1;
-      const bool distinct = !a.same(b) && !a.same(c) && !a.same(d) && !b.same(c) && !b.same(d) && !c.same(d);
-      if (distinct) {
-      void* pa = a.data_ptr();
-      void* pb = b.data_ptr();
-      void* pc = c.data_ptr();
-      void* pd = d.data_ptr();
-      void* pe = take_buffer();
-      kernels::fused_selu_hadamard_add_add(key, pa, pb, pc, pd, pe, (len_t)n, ctx);
+  /* the whole pending expression as one generated kernel, if the table has it; the inner
+   * pending nodes then stay unmaterialised */
+  {
+    std::string signature;
+    std::vector<Tensor> leaves;
+    int budget = 64;
+    const FusedChain* chain = spell(g, t, signature, leaves, budget) ? find_chain(signature) : nullptr;
+    if (chain) {
+      void* x[8];
+      for (size_t i = 0; i < leaves.size(); ++i) {
+        if (leaves[i].len() == 0) panic("materialise: an input of a pending node was freed");
+        x[i] = leaves[i].data_ptr();
+      }
+      void* out = take_buffer();
+      chain->forward(key, x, out, (len_t)n, ctx);
       g->launches++;
-      if (g->mode == Mode::train) attach_op(t, fused_reverse, {a, b, c, d, t});
+      if (g->mode == Mode::train) {
+        std::vector<OpDatum> args(leaves.begin(), leaves.end());
+        args.push_back(OpDatum((double)(chain - fused_chains)));
+        args.push_back(t);
+        attach_op(t, chain_reverse, std::move(args));
+      }
       return;
-      } /* a repeated input needs its contributions added up: per-op path below */
     }
   }
-  if (in0.len() == 0 || in1.len() == 0) panic("materialise: an input of a pending node was freed");
 
   /* anything else: one launch per op, as the reference's forward_impl does */
+  if (in0.len() == 0 || in1.len() == 0) panic("materialise: an input of a pending node was freed");
   void* p0 = in0.data_ptr();
   if (op == Pending::selu) {
     void* pz = take_buffer();
@@ -351,6 +399,9 @@ void materialise(Tensor t) {
   if (op == Pending::add) {
     kernels::addition(key, p0, p1, pz, (len_t)n, ctx);
     if (g->mode == Mode::train) attach_op(t, addition_reverse, {in0, in1, t});
+  } else if (op == Pending::sub) {
+    kernels::subtraction(key, p0, p1, pz, (len_t)n, ctx);
+    if (g->mode == Mode::train) attach_op(t, subtraction_reverse, {in0, in1, t});
   } else {
     kernels::hadamard(key, p0, p1, pz, (len_t)n, ctx);
     if (g->mode == Mode::train) attach_op(t, hadamard_reverse, {in0, in1, t});
@@ -380,6 +431,18 @@ static void addition_reverse(const std::vector<OpDatum>& a) {
   z.ptr->launches += 2;
 }
 
+/* src/ops/subtraction.zig:60-82 with the sign its second launch means: gx = gz + gx, gy = gy - gz
+ * (the reference passes (gz, gy) to the subtraction kernel, which yields gz - gy) */
+static void subtraction_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, y = a[1].t, z = a[2].t;
+  enable_gradient(x);
+  enable_gradient(y);
+  const size_t key = dkey(z);
+  kernels::addition(key, z.grad_ptr(), x.grad_ptr(), x.grad_ptr(), (len_t)x.len(), x.context());
+  kernels::subtraction(key, y.grad_ptr(), z.grad_ptr(), y.grad_ptr(), (len_t)y.len(), y.context());
+  z.ptr->launches += 2;
+}
+
 /* src/ops/hadamard.zig:58-80 */
 static void hadamard_reverse(const std::vector<OpDatum>& a) {
   const Tensor x = a[0].t, y = a[1].t, z = a[2].t;
@@ -406,23 +469,27 @@ static void relu_reverse(const std::vector<OpDatum>& a) {
   z.ptr->launches++;
 }
 
-/* One launch writes all four leaf gradients (the four inputs are distinct tensors: materialise
- * only fuses then). If none of them has a gradient yet the launch creates them (alpha = 0
- * overwrites); otherwise the missing ones are zero-filled and all four are blended (alpha = 1). */
-static void fused_reverse(const std::vector<OpDatum>& a) {
-  const Tensor ins[4] = {a[0].t, a[1].t, a[2].t, a[3].t};
-  const Tensor te = a[4].t;
-  Graph* g = te.ptr;
+/* One launch writes every leaf gradient of a generated chain. args = leaves..., chain index,
+ * output. If no leaf has a gradient yet the launch creates them (alpha = 0 overwrites);
+ * otherwise the missing ones are zero-filled and all are blended (alpha = 1). A tensor that
+ * appears more than once in the expression is one leaf whose contributions the kernel adds. */
+static void chain_reverse(const std::vector<OpDatum>& a) {
+  const size_t k = a.size() - 2;
+  const FusedChain& chain = fused_chains[(size_t)a[k].s];
+  const Tensor out = a[k + 1].t;
+  Graph* g = out.ptr;
   bool any = false;
-  for (const Tensor& t : ins) any = any || t.has_grad();
-  for (const Tensor& t : ins) {
+  for (size_t i = 0; i < k; ++i) any = any || a[i].t.has_grad();
+  void* x[8];
+  void* grads[8];
+  for (size_t i = 0; i < k; ++i) {
+    const Tensor t = a[i].t;
     if (any) enable_gradient(t);
     else t.ptr->grad_of(t) = t.ptr->allocator_.alloc(t.dtype(), t.len(), t.ptr->stream);
+    x[i] = t.data_ptr();
+    grads[i] = t.grad_ptr();
   }
-  kernels::fused_selu_hadamard_add_add_reverse(dkey(te), ins[0].data_ptr(), ins[1].data_ptr(), ins[2].data_ptr(),
-                                               ins[3].data_ptr(), te.grad_ptr(), ins[0].grad_ptr(),
-                                               ins[1].grad_ptr(), ins[2].grad_ptr(), ins[3].grad_ptr(),
-                                               any ? 1.0 : 0.0, (len_t)te.len(), te.context());
+  chain.reverse(dkey(out), x, out.grad_ptr(), grads, any ? 1.0 : 0.0, (len_t)out.len(), out.context());
   g->launches++;
 }
 
@@ -463,6 +530,11 @@ namespace ops {
 Tensor add(Tensor x, Tensor y) {
   check_pair(x, y, "add: operands must agree in dtype and sizes");
   return defer(x.ptr, Pending::add, x, y);
+}
+
+Tensor sub(Tensor x, Tensor y) {
+  check_pair(x, y, "sub: operands must agree in dtype and sizes");
+  return defer(x.ptr, Pending::sub, x, y);
 }
 
 Tensor hadamard(Tensor x, Tensor y) {

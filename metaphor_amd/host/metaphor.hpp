@@ -12,13 +12,15 @@
  * Errors follow the reference: an impossible request panics (prints and aborts), nothing returns
  * a status.
  *
- * What is new here is where the kernels come from. add / hadamard / selu do not launch: they
- * record a pending node. A pending node is materialised when something needs its bytes (a
- * non-elementwise op, data_ptr(), native(), reverse()), and at that point the recorded
- * expression selu(hadamard(add(a,b), add(c,d))) becomes ONE launch of
- * launch_fused_selu_hadamard_add_add and, in reverse, one launch of its _reverse twin; any other
- * expression falls back to one launch per op exactly as the reference does
- * (src/ops/addition.zig:27-58, src/ops/hadamard.zig:25-56).
+ * What is new here is where the kernels come from. add / sub / hadamard / selu do not launch:
+ * they record a pending node. A pending node is materialised when something needs its bytes (a
+ * non-elementwise op, data_ptr(), native(), reverse()). At that point the recorded expression is
+ * written out with its leaves numbered in order of first appearance and looked up in the table
+ * of generated fused chains (chains.hpp, from chains.json): selu(hadamard(add(a,b), add(c,d)))
+ * becomes ONE launch of launch_fused_selu_hadamard_add_add and, in reverse, one launch of its
+ * _reverse twin. An expression that is not in the table runs one launch per op exactly as the
+ * reference does (src/ops/addition.zig:27-58, src/ops/hadamard.zig:25-56), each of its operands
+ * getting the same chance first.
  */
 #ifndef MP_HOST_METAPHOR_HPP
 #define MP_HOST_METAPHOR_HPP
@@ -144,7 +146,7 @@ class TensorAllocator {
   std::unordered_map<size_t, std::vector<void*>> cache_;
 };
 
-enum class Pending : int { none = 0, add, hadamard, selu };
+enum class Pending : int { none = 0, add, sub, hadamard, selu };
 
 /* deferred elementwise nodes: record, query, compute */
 Tensor defer(Graph* g, Pending op, Tensor x, Tensor y);
@@ -208,6 +210,7 @@ void attach_op(Tensor t, void (*rev)(const std::vector<OpDatum>&), std::vector<O
 
 namespace ops {
 Tensor add(Tensor x, Tensor y);
+Tensor sub(Tensor x, Tensor y);
 Tensor hadamard(Tensor x, Tensor y);
 Tensor selu(Tensor x);
 Tensor relu(Tensor x);

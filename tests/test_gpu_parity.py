@@ -198,6 +198,46 @@ def test_fused_chain_forward_and_reverse(dtype, shift):
             g.check(f"fused n={n}")
 
 
+# ------------------------------------------------------------------ generated chains
+
+def _chain_cases():
+    from metaphor_amd import chaingen
+    return [(c["name"], c["expr"]) for c in chaingen.load_chains()]
+
+
+@pytest.mark.parametrize("name,expr", _chain_cases(), ids=[c[0] for c in _chain_cases()])
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_generated_chain_launchers(name, expr, dtype):
+    """Every chain of chains.json through the C-ABI against fp64 torch (forward and autograd) on
+    the same rounded inputs; alpha = 0 overwrites, alpha = 1 accumulates."""
+    from metaphor_amd import chaingen
+    from test_chaingen import _torch_eval
+    root, k = chaingen.parse(expr)
+    r = rng(16)
+    for n in [1, 7, 1000, 65539]:
+        G.say(f"chain {name} dtype={dtype} n={n}")
+        xs = [G.dev(r.uniform(-2, 2, n), dtype) for _ in range(k)]
+        up = G.dev(r.normal(0, 1, n), dtype)
+        ts = [torch.from_numpy(G.host(x.t).astype(np.float64)).requires_grad_(True) for x in xs]
+        ref = _torch_eval(root, ts)
+        ref.backward(torch.from_numpy(G.host(up.t).astype(np.float64)))
+        out = G.Guarded((n,), dtype)
+        G._call(name, dtype, *[x.t.data_ptr() for x in xs], out.t.data_ptr(), n)
+        G.compare(out.t, ref.detach().numpy(), dtype, f"{name} forward n={n}", rowwise=False)
+        for alpha in (0.0, 1.0):
+            gs = [G.dev(r.normal(0, 1, n), dtype) for _ in range(k)]
+            olds = [G.host(g.t).astype(np.float64) for g in gs]
+            G._call(name + "_reverse", dtype, *[x.t.data_ptr() for x in xs], up.t.data_ptr(),
+                    *[g.t.data_ptr() for g in gs], float(alpha), n)
+            for i in range(k):
+                want = ts[i].grad.numpy() + alpha * olds[i]
+                # terms of a sum may cancel (sub, repeated leaves): scale by their size
+                scale = np.abs(ts[i].grad.numpy()) + alpha * np.abs(olds[i])
+                G.compare(gs[i].t, want, dtype, f"{name} reverse g{i} alpha={alpha} n={n}", rowwise=False, scale=scale)
+                gs[i].check(name)
+        out.check(name)
+
+
 # ------------------------------------------------------------------ reduce / broadcast
 
 MATRIX_SHAPES = [(1, 1), (3, 2), (2, 2), (7, 5), (33, 64), (64, 1000), (5, 1027), (300, 4096), (2, 50257),

@@ -52,6 +52,29 @@ def test_host_library_end_to_end(tmp_path):
     _cmp(_load(d, "rep_da"), 2.0 * g * v, "host repeated-input da", rowwise=False, rtol=2e-5)
     _cmp(_load(d, "rep_dc"), g * u, "host repeated-input dc", rowwise=False, rtol=2e-5)
 
+    # other generated chains (fp64 compositions of the pinned oracle pieces; upstream gradient = 1)
+    a64, b64, c64, d64 = (z.astype(np.float64) for z in (a, b, c, dd))
+    u, v = a64 + b64, c64 + d64
+    _cmp(_load(d, "chain_mul_add_add"), u * v, "chain mul(add,add)", rowwise=False)
+    _cmp(_load(d, "chain_mul_add_add_da"), v, "chain mul(add,add) da", rowwise=False)
+    _cmp(_load(d, "chain_mul_add_add_dd"), u, "chain mul(add,add) dd", rowwise=False)
+    w = (a64 - b64) * c64
+    slope = O.selu_reverse(w, np.ones_like(w))
+    _cmp(_load(d, "chain_selu_mul_sub"), O.selu(w), "chain selu(mul(sub,c))", rowwise=False)
+    _cmp(_load(d, "chain_selu_mul_sub_da"), slope * c64, "chain selu(mul(sub,c)) da", rowwise=False)
+    _cmp(_load(d, "chain_selu_mul_sub_db"), -slope * c64, "chain selu(mul(sub,c)) db", rowwise=False)
+    _cmp(_load(d, "chain_selu_mul_sub_dc"), slope * (a64 - b64), "chain selu(mul(sub,c)) dc", rowwise=False,
+         scale=np.abs(slope) * (np.abs(a64) + np.abs(b64)))
+    sa = O.selu(a64 + b64)
+    _cmp(_load(d, "chain_relu_selu_add"), O.relu(sa), "relu(selu(add))", rowwise=False)
+    sa32 = _load(d, "chain_relu_selu_add")  # the eager relu saw the r32 selu output
+    _cmp(_load(d, "chain_relu_selu_add_da"),
+         O.selu_reverse(a64 + b64, np.ones_like(a64)) * (O.selu(a64 + b64) >= 0), "relu(selu(add)) da",
+         rowwise=False)
+    del sa32
+    _cmp(_load(d, "plain_sub"), a64 - b64, "sub", rowwise=False)
+    assert np.all(_load(d, "plain_sub_da") == 1.0) and np.all(_load(d, "plain_sub_db") == -1.0)
+
     m, n, eps = 37, 1000, 1e-6
     x, gain, dy = _load(d, "row_x", (m, n)), _load(d, "row_g"), _load(d, "row_dy", (m, n))
     _cmp(_load(d, "row_y", (m, n)), O.rmsnorm_ij_j(x, gain, eps), "host rmsnorm y")
