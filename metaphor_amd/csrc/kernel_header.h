@@ -206,39 +206,53 @@ template <int CTRL> __device__ __forceinline__ double dpp_move(double v) {
 
 typedef unsigned uint2_t __attribute__((ext_vector_type(2)));
 
-/* After the four DPP steps every lane of a 16-lane row holds that row's result; the two
- * swaps exchange odd/even rows and then the wave halves, returning both values to fold. */
-template <class OP> __device__ __forceinline__ float fold_rows(float v) {
-  /* the two results are copied to scalars before the bit cast: casting the vector element
-   * expression itself reads element 0 twice with this compiler */
-  uint2_t r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
-  unsigned kept = r[0], swapped = r[1];
-  v = OP::apply(__builtin_bit_cast(float, kept), __builtin_bit_cast(float, swapped));
-  r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
-  kept = r[0];
-  swapped = r[1];
+/* After the four DPP steps every lane of a 16-lane row holds that row's result. swap16 pairs
+ * odd and even rows (lanes 0-31 and 32-63 then agree), swap32 pairs the wave halves; each
+ * returns both values to fold. The two results are copied to scalars before the bit cast:
+ * casting the vector element expression itself reads element 0 twice with this compiler. */
+template <class OP> __device__ __forceinline__ float fold_swap16(float v) {
+  const uint2_t r = __builtin_amdgcn_permlane16_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+  const unsigned kept = r[0], swapped = r[1];
   return OP::apply(__builtin_bit_cast(float, kept), __builtin_bit_cast(float, swapped));
 }
-template <class OP> __device__ __forceinline__ double fold_rows(double v) {
-  unsigned long long b = __builtin_bit_cast(unsigned long long, v);
-  uint2_t lo = __builtin_amdgcn_permlane16_swap((unsigned)b, (unsigned)b, false, false);
-  uint2_t hi = __builtin_amdgcn_permlane16_swap((unsigned)(b >> 32), (unsigned)(b >> 32), false, false);
-  v = OP::apply(__builtin_bit_cast(double, ((unsigned long long)hi[0] << 32) | lo[0]),
-                __builtin_bit_cast(double, ((unsigned long long)hi[1] << 32) | lo[1]));
-  b = __builtin_bit_cast(unsigned long long, v);
-  lo = __builtin_amdgcn_permlane32_swap((unsigned)b, (unsigned)b, false, false);
-  hi = __builtin_amdgcn_permlane32_swap((unsigned)(b >> 32), (unsigned)(b >> 32), false, false);
-  return OP::apply(__builtin_bit_cast(double, ((unsigned long long)hi[0] << 32) | lo[0]),
-                   __builtin_bit_cast(double, ((unsigned long long)hi[1] << 32) | lo[1]));
+template <class OP> __device__ __forceinline__ float fold_swap32(float v) {
+  const uint2_t r = __builtin_amdgcn_permlane32_swap(__builtin_bit_cast(unsigned, v), __builtin_bit_cast(unsigned, v), false, false);
+  const unsigned kept = r[0], swapped = r[1];
+  return OP::apply(__builtin_bit_cast(float, kept), __builtin_bit_cast(float, swapped));
+}
+template <class OP> __device__ __forceinline__ double fold_swap16(double v) {
+  const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+  const uint2_t lo = __builtin_amdgcn_permlane16_swap((unsigned)b, (unsigned)b, false, false);
+  const uint2_t hi = __builtin_amdgcn_permlane16_swap((unsigned)(b >> 32), (unsigned)(b >> 32), false, false);
+  const unsigned lo0 = lo[0], lo1 = lo[1], hi0 = hi[0], hi1 = hi[1];
+  return OP::apply(__builtin_bit_cast(double, ((unsigned long long)hi0 << 32) | lo0),
+                   __builtin_bit_cast(double, ((unsigned long long)hi1 << 32) | lo1));
+}
+template <class OP> __device__ __forceinline__ double fold_swap32(double v) {
+  const unsigned long long b = __builtin_bit_cast(unsigned long long, v);
+  const uint2_t lo = __builtin_amdgcn_permlane32_swap((unsigned)b, (unsigned)b, false, false);
+  const uint2_t hi = __builtin_amdgcn_permlane32_swap((unsigned)(b >> 32), (unsigned)(b >> 32), false, false);
+  const unsigned lo0 = lo[0], lo1 = lo[1], hi0 = hi[0], hi1 = hi[1];
+  return OP::apply(__builtin_bit_cast(double, ((unsigned long long)hi0 << 32) | lo0),
+                   __builtin_bit_cast(double, ((unsigned long long)hi1 << 32) | lo1));
 }
 
-/* Every lane of the wave returns OP folded over all 64 lanes. */
-template <class OP, class P> __device__ __forceinline__ P wave_allreduce(P v) {
+/* OP folded over the S = 16, 32 or 64 lanes of an aligned sub-group of the wave; every lane of
+ * the sub-group returns the result. All 64 lanes must execute it. */
+template <class OP, int S, class P> __device__ __forceinline__ P lanes_allreduce(P v) {
+  static_assert(S == 16 || S == 32 || S == 64, "sub-groups of 16, 32 or 64 lanes");
   v = OP::apply(v, dpp_move<DPP_XOR1>(v));
   v = OP::apply(v, dpp_move<DPP_XOR2>(v));
   v = OP::apply(v, dpp_move<DPP_HALF_MIRROR>(v));
   v = OP::apply(v, dpp_move<DPP_MIRROR>(v));
-  return fold_rows<OP>(v);
+  if constexpr (S >= 32) v = fold_swap16<OP>(v);
+  if constexpr (S >= 64) v = fold_swap32<OP>(v);
+  return v;
+}
+
+/* Every lane of the wave returns OP folded over all 64 lanes. */
+template <class OP, class P> __device__ __forceinline__ P wave_allreduce(P v) {
+  return lanes_allreduce<OP, WAVE>(v);
 }
 
 /* NW per-wave partials, one per lane with index lane % NW, folded so that every lane holds the
@@ -261,10 +275,10 @@ template <class OP, int NW, class P> __device__ __forceinline__ P fold_partials(
  * across lanes, instead of every lane reading and adding all of them. */
 template <class OP, int G, class P>
 __device__ __forceinline__ P group_allreduce(P v, P* slots, int lane_in_group) {
-  v = wave_allreduce<OP>(v);
-  if constexpr (G == WAVE) {
-    return v;
+  if constexpr (G <= WAVE) { /* a wave or an aligned part of one: cross-lane only */
+    return lanes_allreduce<OP, G>(v);
   } else {
+    v = wave_allreduce<OP>(v);
     constexpr int NW = G / WAVE;
     if ((lane_in_group & (WAVE - 1)) == 0) slots[lane_in_group / WAVE] = v;
     __syncthreads();

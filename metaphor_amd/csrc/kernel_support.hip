@@ -32,9 +32,9 @@ extern "C" len_t mpSoftmaxScratchBytes(len_t dtype, len_t m, len_t n) {
 
 // Diagnostic: force the row regime of the softmax / RMSNorm launchers (0 auto; 1..5 = groups of
 // 64, 128, 256, 512, 1024 threads per row; 6 = streaming; 7 = cluster path of the softmax
-// forward). A group that cannot hold a row falls through to the next wider one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
+// forward; 8, 9 = sub-wave groups of 16 and 32 lanes of the softmax kernels). A group that cannot hold a row falls through to the next wider one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
 extern "C" void mpSetRowRegime(len_t regime) {
-  mp::require(regime <= mp::REGIME_CLUSTER, "mpSetRowRegime: regime must be 0..7");
+  mp::require(regime <= mp::REGIME_G32, "mpSetRowRegime: regime must be 0..9");
   mp::row_regime_override() = (int)regime;
 }
 

@@ -6,6 +6,8 @@
  * HBM once. HBM streams fastest here with many small waves each moving one or two packs, so
  * the plan takes the narrowest group that covers the row at a target NV (2 for softmax, 1 for
  * RMSNorm) and only lets NV grow once the group is 1024 threads wide:
+ *   G = 16, 32         (softmax) several short rows per wavefront, DPP reductions inside 16- or
+ *                      32-lane parts of the wave, so rows of a few hundred bytes keep all lanes busy;
  *   G = 64             one wavefront per row, cross-lane (DPP / permlane-swap) reductions only;
  *   G = 128 ... 1024   per-wave partials combined through LDS with one barrier per reduction;
  *   stream             rows too long for registers: an online first pass and a second pass that
@@ -23,9 +25,10 @@
 namespace mp {
 
 /* 0 = automatic; 1..5 force G = 64, 128, 256, 512, 1024; 6 forces the streaming kernels;
- * 7 forces the cluster path of the softmax forward (the other launchers treat it as automatic). */
+ * 7 forces the cluster path of the softmax forward; 8 and 9 force sub-wave groups of 16 and 32
+ * lanes (softmax only). A launcher without the forced path treats the value as automatic. */
 enum RowRegime { REGIME_AUTO = 0, REGIME_G64 = 1, REGIME_G128 = 2, REGIME_G256 = 3, REGIME_G512 = 4,
-                 REGIME_G1024 = 5, REGIME_STREAM = 6, REGIME_CLUSTER = 7 };
+                 REGIME_G1024 = 5, REGIME_STREAM = 6, REGIME_CLUSTER = 7, REGIME_G16 = 8, REGIME_G32 = 9 };
 
 /* Diagnostic override set through mpSetRowRegime; AUTO in normal use. */
 inline int& row_regime_override() {
@@ -48,37 +51,46 @@ struct RowPlan {
   int NV;  /* packs per thread */
 };
 
-/* nv_target: packs per thread the automatic plan aims for before it widens the group. */
-inline RowPlan plan_row(size_t packs, int max_nv, int nv_target) {
-  static const int group_of[] = {0, 64, 128, 256, 512, 1024};
+/* nv_target: packs per thread the automatic plan aims for before it widens the group.
+ * subwave: the kernel also comes in groups of 16 and 32 lanes (several rows per wavefront), which
+ * keeps every lane busy on rows shorter than a wavefront's worth of packs. */
+inline RowPlan plan_row(size_t packs, int max_nv, int nv_target, bool subwave = false) {
+  static const int ladder[] = {16, 32, 64, 128, 256, 512, 1024};
+  constexpr int RUNGS = 7;
   int forced = row_regime_override();
-  if (forced == REGIME_CLUSTER) forced = REGIME_AUTO;
+  if (forced == REGIME_CLUSTER || (!subwave && (forced == REGIME_G16 || forced == REGIME_G32))) forced = REGIME_AUTO;
   if (forced == REGIME_STREAM) return RowPlan{0, 0};
+  const int first_rung = subwave ? 0 : 2;
   if (forced == REGIME_AUTO) {
     const int want = nv_target < max_nv ? nv_target : max_nv;
-    for (int r = REGIME_G64; r <= REGIME_G1024; ++r) {
-      const int nv = packs_per_thread(packs, group_of[r], want);
-      if (nv) return RowPlan{group_of[r], nv};
+    for (int r = first_rung; r < RUNGS; ++r) {
+      const int nv = packs_per_thread(packs, ladder[r], want);
+      if (nv) return RowPlan{ladder[r], nv};
     }
     const int nv = packs_per_thread(packs, 1024, max_nv);
     return nv ? RowPlan{1024, nv} : RowPlan{0, 0};
   }
   /* a forced group that cannot hold the row moves on to the next wider one */
-  for (int r = forced; r <= REGIME_G1024; ++r) {
-    const int nv = packs_per_thread(packs, group_of[r], max_nv);
-    if (nv) return RowPlan{group_of[r], nv};
+  const int start = forced == REGIME_G16 ? 0 : forced == REGIME_G32 ? 1 : forced + 1;
+  for (int r = start; r < RUNGS; ++r) {
+    const int nv = packs_per_thread(packs, ladder[r], max_nv);
+    if (nv) return RowPlan{ladder[r], nv};
   }
   return RowPlan{0, 0};
 }
 
 /* Calls f.template operator()<G, NV>() for the plan; returns false for the streaming plan. */
-template <int MAXNV, class F> inline bool for_row_plan(const RowPlan& plan, F&& f) {
+template <int MAXNV, bool SUBWAVE = false, class F> inline bool for_row_plan(const RowPlan& plan, F&& f) {
 #define MP_PLAN_CASE(G_, NV_) \
   if constexpr (NV_ <= MAXNV) { \
     if (plan.G == G_ && plan.NV == NV_) { f.template operator()<G_, NV_>(); return true; } \
   }
 #define MP_PLAN_GROUP(G_) \
   MP_PLAN_CASE(G_, 1) MP_PLAN_CASE(G_, 2) MP_PLAN_CASE(G_, 4) MP_PLAN_CASE(G_, 8) MP_PLAN_CASE(G_, 16)
+  if constexpr (SUBWAVE) {
+    MP_PLAN_GROUP(16)
+    MP_PLAN_GROUP(32)
+  }
   MP_PLAN_GROUP(64)
   MP_PLAN_GROUP(128)
   MP_PLAN_GROUP(256)
@@ -91,9 +103,12 @@ template <int MAXNV, class F> inline bool for_row_plan(const RowPlan& plan, F&& 
 
 constexpr int STREAM_THREADS = 1024;
 
-inline unsigned row_grid(size_t m) {
-  require(m < 0x7fffffffull, "row launch: too many rows for one grid");
-  return (unsigned)m;
+/* workgroups for m rows when a workgroup of max(G, 64) threads holds max(1, 64 / G) rows */
+inline unsigned row_grid(size_t m, int G) {
+  const size_t rows_per_block = G < WAVE ? WAVE / G : 1;
+  const size_t blocks = (m + rows_per_block - 1) / rows_per_block;
+  require(blocks < 0x7fffffffull, "row launch: too many rows for one grid");
+  return (unsigned)blocks;
 }
 
 }  // namespace mp

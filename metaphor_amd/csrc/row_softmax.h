@@ -29,13 +29,16 @@ namespace mp {
 /* ------------------------------------------------------------------ resident forward */
 
 template <class T, int W, int G, int NV, bool RAGGED>
-__global__ __launch_bounds__(G) void softmax_fwd_resident(
+__global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_fwd_resident(
     const T* x, T* y, size_t m, size_t n) {
   using P = typename precision<T>::type;
-  __shared__ P slots[2][G / WAVE];
+  constexpr int RPB = G < WAVE ? WAVE / G : 1; /* rows per workgroup: several only below a wave */
+  __shared__ P slots[2][G < WAVE ? 1 : G / WAVE];
 
-  const int lane = threadIdx.x; /* one row per workgroup of G threads */
-  const size_t row = blockIdx.x;
+  const int lane = threadIdx.x % G;
+  const size_t row_at = (size_t)blockIdx.x * RPB + threadIdx.x / G;
+  const bool live = row_at < m;            /* a dead part of a wave still runs the cross-lane steps */
+  const size_t row = live ? row_at : m - 1;
 
   const T* xr = x + row * n;
   const RowGeom<T, W> g(xr, n, RAGGED);
@@ -53,19 +56,22 @@ __global__ __launch_bounds__(G) void softmax_fwd_resident(
 
   const P inv = (P)1 / s;
   t.each([&](P& e) { e *= inv; });
-  t.store(y + row * n, g, lane);
+  if (live) t.store(y + row * n, g, lane);
 }
 
 /* ------------------------------------------------------------------ resident reverse */
 
 template <class T, int W, int G, int NV, bool RAGGED, bool BLEND>
-__global__ __launch_bounds__(G) void softmax_rev_resident(
+__global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_rev_resident(
     const T* y, const T* dy, T* dx, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
-  __shared__ P slots[G / WAVE];
+  constexpr int RPB = G < WAVE ? WAVE / G : 1;
+  __shared__ P slots[G < WAVE ? 1 : G / WAVE];
 
-  const int lane = threadIdx.x;
-  const size_t row = blockIdx.x;
+  const int lane = threadIdx.x % G;
+  const size_t row_at = (size_t)blockIdx.x * RPB + threadIdx.x / G;
+  const bool live = row_at < m;
+  const size_t row = live ? row_at : m - 1;
 
   const T* yr = y + row * n;
   const T* gr = dy + row * n;
@@ -82,6 +88,7 @@ __global__ __launch_bounds__(G) void softmax_rev_resident(
     for (int i = 0; i < W; ++i) dot += ty.v[k][i] * tg.v[k][i];
   if constexpr (RAGGED) dot += ty.edge * tg.edge;
   dot = group_allreduce<AddOP, G>(dot, slots, lane);
+  if (!live) return; /* nothing below crosses lanes */
 
   T* body = dr + g.head;
 #pragma unroll
@@ -522,9 +529,9 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   }
   const bool ragged = !(aligned16(x) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(64);
-  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2);
-  const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
-    const dim3 grid(row_grid(m)), block(G);
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, true);
+  const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
+    const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n);
     else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n);
   });
@@ -551,9 +558,9 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, double alpha, size_t
   }
   const bool ragged = !(aligned16(y) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 2);
-  const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
-    const dim3 grid(row_grid(m)), block(G);
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 2, true);
+  const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
+    const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) {
       if (blend) softmax_rev_resident<T, W, G, NV, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
       else softmax_rev_resident<T, W, G, NV, true, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);

@@ -13,7 +13,7 @@ pytestmark = pytest.mark.gpu
 
 DTYPES = [torch.float16, torch.float32, torch.float64]
 IDS = ["r16", "r32", "r64"]
-REGIMES = [0, 1, 2, 3, 4, 5, 6, 7]  # auto, G = 64/128/256/512/1024, stream, cluster (softmax forward)
+REGIMES = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9]  # auto, G = 64..1024, stream, cluster (softmax fwd), G = 16, 32 (softmax)
 
 
 @pytest.fixture(autouse=True)
@@ -285,7 +285,7 @@ def test_reference_example_reductions():
 
 # ------------------------------------------------------------------ softmax
 
-SOFTMAX_SHAPES = [(1, 1), (3, 7), (5, 64), (4, 65), (9, 256), (7, 1000), (256, 1024), (6, 2048),
+SOFTMAX_SHAPES = [(1, 1), (3, 7), (5, 64), (4, 65), (1031, 16), (9, 256), (7, 1000), (256, 1024), (6, 2048),
                   (3, 5000), (5, 8192), (2, 20000), (2, 50257), (1, 151936), (1030, 33)]
 
 
