@@ -6,7 +6,7 @@
  * HBM once. HBM streams fastest here with many small waves each moving one or two packs, so
  * the plan takes the narrowest group that covers the row at a target NV (2 for softmax, 1 for
  * RMSNorm) and only lets NV grow once the group is 1024 threads wide:
- *   G = 16, 32         (softmax) several short rows per wavefront, DPP reductions inside 16- or
+ *   G = 16, 32         several short rows per wavefront, DPP reductions inside 16- or
  *                      32-lane parts of the wave, so rows of a few hundred bytes keep all lanes busy;
  *   G = 64             one wavefront per row, cross-lane (DPP / permlane-swap) reductions only;
  *   G = 128 ... 1024   per-wave partials combined through LDS with one barrier per reduction;
@@ -26,7 +26,7 @@ namespace mp {
 
 /* 0 = automatic; 1..5 force G = 64, 128, 256, 512, 1024; 6 forces the streaming kernels;
  * 7 forces the cluster path of the softmax forward; 8 and 9 force sub-wave groups of 16 and 32
- * lanes (softmax only). A launcher without the forced path treats the value as automatic. */
+ * lanes. A launcher without the forced path treats the value as automatic. */
 enum RowRegime { REGIME_AUTO = 0, REGIME_G64 = 1, REGIME_G128 = 2, REGIME_G256 = 3, REGIME_G512 = 4,
                  REGIME_G1024 = 5, REGIME_STREAM = 6, REGIME_CLUSTER = 7, REGIME_G16 = 8, REGIME_G32 = 9 };
 

@@ -29,8 +29,8 @@ constexpr int NORM_BLOCK = 1024;
 /* Both values folded over a G-thread group with a single barrier. */
 template <int G, class P>
 __device__ __forceinline__ void group_allreduce_sum2(P& a, P& b, P* slots_a, P* slots_b, int lane) {
-  a = wave_allreduce<AddOP>(a);
-  b = wave_allreduce<AddOP>(b);
+  a = lanes_allreduce<AddOP, (G < WAVE ? G : WAVE)>(a);
+  b = lanes_allreduce<AddOP, (G < WAVE ? G : WAVE)>(b);
   if constexpr (G > WAVE) {
     if ((lane & (WAVE - 1)) == 0) {
       slots_a[lane / WAVE] = a;
@@ -50,7 +50,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_fwd_resident(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
   using P = typename precision<T>::type;
   constexpr int RPB = NORM_BLOCK / G;
-  __shared__ P slots[2][RPB][G / WAVE];
+  __shared__ P slots[2][G < WAVE ? 1 : RPB][G < WAVE ? 1 : G / WAVE];
 
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
 
@@ -80,7 +80,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_fwd_resident(
 
     P ss = (P)0;
     t.each([&](P& e) { ss += e * e; });
-    ss = group_allreduce<AddOP, G>(ss, slots[parity][sub], lane);
+    ss = group_allreduce<AddOP, G>(ss, slots[parity][G < WAVE ? 0 : sub], lane);
     const P r = rsqrt_of(ss / (P)n + eps);
 
     if (live) {
@@ -173,7 +173,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
   constexpr int RPB = NORM_BLOCK / G;
-  __shared__ P slots[2][2][RPB][G / WAVE];
+  __shared__ P slots[2][2][G < WAVE ? 1 : RPB][G < WAVE ? 1 : G / WAVE];
   __shared__ P comb[RPB > 1 ? G * NV * W : 1];
 
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
@@ -215,7 +215,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
         ss += xv[k][i] * xv[k][i];
         c += dv[k][i] * gv[k][i] * xv[k][i];
       }
-    group_allreduce_sum2<G>(ss, c, slots[parity][0][sub], slots[parity][1][sub], lane);
+    group_allreduce_sum2<G>(ss, c, slots[parity][0][G < WAVE ? 0 : sub], slots[parity][1][G < WAVE ? 0 : sub], lane);
     const P r = rsqrt_of(ss / (P)n + eps);
     const P cc = c / (P)n * r * r;
 
@@ -404,8 +404,8 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, double eps, size_t 
   }
   const bool ragged = !(aligned16(x) && aligned16(gain) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 1);
-  const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 1, true);
+  const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
     if (ragged) rmsnorm_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
@@ -429,8 +429,8 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
   /* four register arrays per thread (x, dy, gain, dg sums): 16 registers each when packed,
    * 8 elements each on the element-wise path */
   constexpr int MAXNV = W == 1 ? 8 : max_nv_for<T>(16);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 1);
-  const bool resident = for_row_plan<MAXNV>(plan, [&]<int G, int NV>() {
+  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 1, true);
+  const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     rows = (unsigned)(need < max_rows ? need : max_rows);
     const dim3 grid(rows), block(NORM_BLOCK);

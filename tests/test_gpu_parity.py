@@ -444,7 +444,7 @@ def test_softmax_reverse_unaligned(dtype):
 
 # ------------------------------------------------------------------ RMSNorm
 
-NORM_SHAPES = [(1, 1), (3, 7), (17, 64), (33, 256), (64, 4096), (5, 1000), (300, 1024), (3, 50257),
+NORM_SHAPES = [(1, 1), (3, 7), (17, 64), (1031, 16), (259, 128), (33, 256), (64, 4096), (5, 1000), (300, 1024), (3, 50257),
                (2, 70001), (1025, 128), (40, 8192)]
 
 
