@@ -272,40 +272,64 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
 
 /* ------------------------------------------------------------------ streaming reverse */
 
-/* Rows too long for registers. Same alignment rule as the resident reverse. Each workgroup
- * owns one partial row and adds every row it processes into it (first row: overwrite). */
-template <class T, int W, bool BLEND>
+/* Rows too long to keep x and dy in registers: they are read twice (the second read mostly from
+ * cache). Same alignment rule as the resident reverse. NA > 0: a thread still keeps the dg sums
+ * of its NA packs of columns in registers and the workgroup writes one partial row at the end.
+ * NA == 0 (rows beyond 1024 * NA packs): each workgroup adds every row it processes into its
+ * partial row in memory (first row: overwrite). */
+template <class T> constexpr int stream_acc_packs() {
+  using P = typename precision<T>::type;
+  return 64 / ((PACK_BYTES / (int)sizeof(T)) * (int)(sizeof(P) / 4)); /* 64 registers of sums */
+}
+
+template <class T, int W, int NA, bool BLEND>
 __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
-  constexpr int G = STREAM_THREADS;
+  constexpr int G = STREAM_THREADS, U = 2;
   __shared__ P slots[2][2][G / WAVE];
   const int lane = threadIdx.x;
   const int nvec = (int)(n / W);
   P* mine = partials + (size_t)blockIdx.x * n;
   int parity = 0;
   bool first = true;
+  P acc[NA > 0 ? NA : 1][W];
+#pragma unroll
+  for (int k = 0; k < (NA > 0 ? NA : 1); ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) acc[k][i] = (P)0;
 
   for (size_t row = blockIdx.x; row < m; row += gridDim.x, parity ^= 1, first = false) {
     const size_t off = row * n;
     P ss = (P)0, c = (P)0;
-    for (int p = lane; p < nvec; p += G) {
-      P xv[W], dv[W], gv[W];
-      load_pack<T, W>(x + off + (size_t)p * W, xv);
-      load_pack<T, W>(dy + off + (size_t)p * W, dv);
-      load_pack<T, W>(gain + (size_t)p * W, gv);
+    for (int p0 = lane; p0 < nvec; p0 += G * U) {
+      P xv[U][W], dv[U][W], gv[U][W];
 #pragma unroll
-      for (int i = 0; i < W; ++i) {
-        ss += xv[i] * xv[i];
-        c += dv[i] * gv[i] * xv[i];
+      for (int u = 0; u < U; ++u) {
+        const int p = p0 + u * G;
+        if (p < nvec) {
+          load_pack<T, W>(x + off + (size_t)p * W, xv[u]);
+          load_pack<T, W>(dy + off + (size_t)p * W, dv[u]);
+          load_pack<T, W>(gain + (size_t)p * W, gv[u]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < W; ++i) xv[u][i] = dv[u][i] = gv[u][i] = (P)0;
+        }
       }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+          ss += xv[u][i] * xv[u][i];
+          c += dv[u][i] * gv[u][i] * xv[u][i];
+        }
     }
     group_allreduce_sum2<G>(ss, c, slots[parity][0], slots[parity][1], lane);
     const P r = rsqrt_of(ss / (P)n + eps);
     const P cc = c / (P)n * r * r;
 
-    for (int p = lane; p < nvec; p += G) {
+    auto finish_pack = [&](int p, P (&sum)[W], bool in_registers) {
       P xv[W], dv[W], gv[W], out[W];
       load_pack_nt<T, W>(x + off + (size_t)p * W, xv);
       load_pack_nt<T, W>(dy + off + (size_t)p * W, dv);
@@ -314,8 +338,12 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
       for (int i = 0; i < W; ++i) {
         out[i] = r * (dv[i] * gv[i] - xv[i] * cc);
         const P t = dv[i] * xv[i] * r;
-        P* slot = mine + (size_t)p * W + i;
-        *slot = first ? t : *slot + t;
+        if (in_registers) {
+          sum[i] += t;
+        } else {
+          P* slot = mine + (size_t)p * W + i;
+          *slot = first ? t : *slot + t;
+        }
       }
       if constexpr (BLEND) {
         P old[W];
@@ -324,6 +352,26 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
         for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
       }
       store_pack_nt<T, W>(dx + off + (size_t)p * W, out);
+    };
+    if constexpr (NA > 0) {
+#pragma unroll
+      for (int k = 0; k < NA; ++k) {
+        const int p = k * G + lane;
+        if (p < nvec) finish_pack(p, acc[k], true);
+      }
+    } else {
+      for (int p = lane; p < nvec; p += G) finish_pack(p, acc[0], false);
+    }
+  }
+
+  if constexpr (NA > 0) {
+#pragma unroll
+    for (int k = 0; k < NA; ++k) {
+      const int p = k * G + lane;
+      if (p < nvec) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) mine[(size_t)p * W + i] = acc[k][i];
+      }
     }
   }
 }
@@ -440,8 +488,15 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
   if (!resident) {
     rows = (unsigned)max_rows;
     const dim3 grid(rows), block(STREAM_THREADS);
-    if (blend) rmsnorm_rev_stream<T, W, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
-    else rmsnorm_rev_stream<T, W, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+    constexpr int NA = W == 1 ? 16 : stream_acc_packs<T>();
+    const bool sums_fit = (n + W - 1) / W <= (size_t)STREAM_THREADS * NA;
+    if (sums_fit) {
+      if (blend) rmsnorm_rev_stream<T, W, NA, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+      else rmsnorm_rev_stream<T, W, NA, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+    } else {
+      if (blend) rmsnorm_rev_stream<T, W, 0, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+      else rmsnorm_rev_stream<T, W, 0, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+    }
   }
   MP_CHECK_LAUNCH();
   /* wide loads need 16-byte aligned partial rows: fp32 accumulators, n % 4 == 0, aligned scratch */

@@ -445,7 +445,7 @@ def test_softmax_reverse_unaligned(dtype):
 # ------------------------------------------------------------------ RMSNorm
 
 NORM_SHAPES = [(1, 1), (3, 7), (17, 64), (1031, 16), (259, 128), (33, 256), (64, 4096), (5, 1000), (300, 1024), (3, 50257),
-               (2, 70001), (1025, 128), (40, 8192)]
+               (2, 70001), (1025, 128), (40, 8192), (3, 32768), (2, 300000)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
