@@ -22,7 +22,8 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0
-SETS = {"cfg1": 16, "cfg2": 4, "cfg3": 2, "cfg4": 2, "cfg5a": 3, "cfg5b": 3, "copy": 2}
+SETS = {"cfg1": 16, "cfg2": 4, "cfg3": 2, "cfg4": 2, "cfg5a": 3, "cfg5b": 3, "copy": 2, "permutate": 2, "gemm": 2}
+MFMA_PEAK_TFLOPS = {"gemm": 2500.0}  # dense fp16 matrix rate of the MI355X
 
 
 PROFILE_OF = {"cfg1": "cfg1_softmax", "cfg2": "cfg2_rmsnorm", "cfg3": "cfg3_softmax_r16",
@@ -128,6 +129,10 @@ def rates(w, fwd_ms, rev_ms):
         out["rev_GBps"] = round(w.rev_bytes / (_median(rev_ms) * 1e-3) / 1e9, 1)
         out["rev_frac"] = round(out["rev_GBps"] / HBM_PEAK_GBPS, 4)
         out["rev_rows_per_s"] = round(w.rows / (_median(rev_ms) * 1e-3), 1)
+    if hasattr(w, "fwd_flops"):
+        out["fwd_TFLOPs"] = round(w.fwd_flops / (_median(fwd_ms) * 1e-3) / 1e12, 1)
+        if rev_ms:
+            out["rev_TFLOPs"] = round(w.rev_flops / (_median(rev_ms) * 1e-3) / 1e12, 1)
     return out
 
 
@@ -211,7 +216,7 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": {"cfg3": "f16"}.get(name, "f32"),
+        "dtype": {"cfg3": "f16", "gemm": "f16"}.get(name, "f32"),
         "data": "synthetic",
         "config": {"workload": f"{name}: {W.DESCRIPTION[name]}", "buffer_sets": len(sets),
                    "bytes_per_step": step_bytes},
@@ -224,6 +229,11 @@ def main():
         name: rates(w, fwd_ms, rev_ms),
     }
 
+    if name in MFMA_PEAK_TFLOPS:  # the matrix product is priced in flops against the matrix cores
+        tf = w.rev_flops / (avg_ms * 1e-3) / 1e12
+        line["roofline"].update({"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS[name],
+                                 "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
+                                 "flops_per_launch": w.rev_flops})
     if not args.no_cpu and name == "cfg2":
         line["cpu_baseline"], line["parity"] = cpu_baseline_cfg2(w)
     del sets, w

@@ -33,10 +33,16 @@ EXTERN_C void mpMemFree(void* dptr, StreamContext);
 EXTERN_C void mpDeviceSynchronize();
 /* device_utils.cu:25-28 */
 EXTERN_C void mpStreamSynchronize(StreamContext);
-/* device_utils.cu:70-88 — create a stream (default priority); blas_handle is NULL. */
+/* device_utils.cu:70-88 — create a stream (default priority) and a rocBLAS handle bound to it. */
 EXTERN_C StreamContext mpInitStream();
 /* device_utils.cu:90-99 */
 EXTERN_C void mpDeinitStream(StreamContext);
+/* No counterpart in the reference: for callers that bring their own stream (a framework's).
+ * Returns a context for `hip_stream` (NULL = the default stream) with a new rocBLAS handle bound
+ * to it, which the matrix-product launchers need; mpReleaseStream destroys that handle and
+ * leaves the stream alone. */
+EXTERN_C StreamContext mpAdoptStream(void* hip_stream);
+EXTERN_C void mpReleaseStream(StreamContext);
 /* device_utils.cu:55-62 — device sync, then print (not exit on) the last error. */
 EXTERN_C void mpCheckLastError();
 /* device_utils.cu:64-68 */

@@ -1,10 +1,10 @@
 /*
- * Device utilities on the HIP runtime: the eleven mp* exports of the boundary
+ * Device utilities on the HIP runtime: the mp* exports of the boundary
  * (include/device_utils.h), replacing the CUDA driver-API bodies of the reference's
  * src/cuda/device_utils.cu:4-99. Built as libdev_utils.so, as the reference does
  * (build.zig:23-45).
  */
-#include "kernel_header.h"
+#include "gemm_dispatch.h"
 #include "device_utils.h"
 
 extern "C" void* mpMemAlloc(len_t N, StreamContext stream) {
@@ -63,10 +63,30 @@ extern "C" StreamContext mpInitStream() {
   HIP_ASSERT(hipStreamCreate(&hip_stream));
   StreamContext context;
   context.hip_stream.ptr = reinterpret_cast<void*>(hip_stream);
-  context.blas_handle.ptr = nullptr;
+  /* the matrix-product launchers find their library handle here, bound to this stream
+   * (device_utils.cu:72-86 does the same with cuBLAS) */
+  rocblas_handle blas = nullptr;
+  ROCBLAS_ASSERT(rocblas_create_handle(&blas));
+  ROCBLAS_ASSERT(rocblas_set_stream(blas, hip_stream));
+  context.blas_handle.ptr = reinterpret_cast<void*>(blas);
   return context;
 }
 
+extern "C" StreamContext mpAdoptStream(void* hip_stream) {
+  rocblas_handle blas = nullptr;
+  ROCBLAS_ASSERT(rocblas_create_handle(&blas));
+  ROCBLAS_ASSERT(rocblas_set_stream(blas, static_cast<hipStream_t>(hip_stream)));
+  StreamContext context;
+  context.hip_stream.ptr = hip_stream;
+  context.blas_handle.ptr = reinterpret_cast<void*>(blas);
+  return context;
+}
+
+extern "C" void mpReleaseStream(StreamContext stream) {
+  if (get_handle(stream) != nullptr) ROCBLAS_ASSERT(rocblas_destroy_handle(get_handle(stream)));
+}
+
 extern "C" void mpDeinitStream(StreamContext stream) {
+  if (get_handle(stream) != nullptr) ROCBLAS_ASSERT(rocblas_destroy_handle(get_handle(stream)));
   HIP_ASSERT(hipStreamDestroy(get_stream(stream)));
 }

@@ -12,6 +12,9 @@ Workloads (N(mu, s) = mean mu, standard deviation s; seed 0 unless a set index i
   cfg4  fused e = selu((a+b)*(c+d)) forward + reverse, r32, flat 2^28, inputs U(-2,2), de ~ N(0,1)
   cfg5a softmax forward, r32, [512, 151936], N(0,3) + 12 on one random column per row
   cfg5b softmax forward, r32, [2048, 50257], same distribution
+  permutate  transpose, r32, [16384, 16384] ~ N(0,1); reverse = the accumulating transpose (alpha 1)
+  gemm       c = a.b, r16 with fp32 accumulation, [8192, 8192] x [8192, 8192], inputs N(0, 0.25);
+             reverse = the two products of its gradient (G.T(b) and T(a).G)
 """
 import torch
 
@@ -30,7 +33,31 @@ def _launch(stem, dtype, *args):
     ffi.invoke(getattr(kernels, stem), KEY[dtype], *args, _ctx())
 
 
+_blas_contexts = {}
+
+
+def blas_ctx():
+    """Context of torch's current stream carrying a rocBLAS handle (made once per stream)."""
+    _, utils = ffi.load()
+    handle = torch.cuda.current_stream().cuda_stream
+    if handle not in _blas_contexts:
+        _blas_contexts[handle] = utils.mpAdoptStream(handle or None)
+    return _blas_contexts[handle]
+
+
 # ------------------------------------------------------------------ launch wrappers
+
+def permutate(src, dst, alpha=0.0):
+    rows, cols = src.shape
+    _launch("permutate_ij_ji", src.dtype, src.data_ptr(), dst.data_ptr(), float(alpha), rows, cols)
+
+
+def inner_product(form, a, b, alpha, c, beta, m, n, k):
+    """form "ij_jk_ik", "ij_kj_ik" or "ji_jk_ik": c[m,k] = alpha * op(a).op(b) + beta * c over n."""
+    kernels, _ = ffi.load()
+    ffi.invoke(getattr(kernels, "inner_product_" + form), KEY[a.dtype], a.data_ptr(), b.data_ptr(),
+               float(alpha), c.data_ptr(), float(beta), m, n, k, blas_ctx())
+
 
 def softmax_scratch(dtype, m, n):
     """Workspace for launch_softmax_ij_j (None when the rows fit one workgroup)."""
@@ -254,7 +281,60 @@ class Copy(Workload):
         _launch("copy", self.x.dtype, self.x.data_ptr(), self.y.data_ptr(), self.n)
 
 
-WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b, Copy)}
+class Permutate(Workload):
+    name, dtype = "permutate", torch.float32
+    shape = (16384, 16384)
+
+    def __init__(self, seed=0, shape=None, dtype=None):
+        self.shape = shape or self.shape
+        self.dtype = dtype or self.dtype
+        rows, cols = self.shape
+        self.x = torch.randn(self.shape, generator=_gen(seed), device="cuda", dtype=torch.float32).to(self.dtype)
+        self.y = torch.empty((cols, rows), dtype=self.dtype, device="cuda")
+        self.gx = torch.zeros_like(self.x)
+        self.rows = rows * cols
+        self.fwd_bytes = 2 * self.x.numel() * self.x.element_size()
+        self.rev_bytes = 3 * self.x.numel() * self.x.element_size()
+
+    def forward(self):
+        permutate(self.x, self.y)
+
+    def reverse(self):  # src/ops/permutate.zig:58-69: the gradient comes back transposed and accumulates
+        permutate(self.y, self.gx, 1.0)
+
+
+class Gemm(Workload):
+    name, dtype = "gemm", torch.float16
+    mnk = (8192, 8192, 8192)
+
+    def __init__(self, seed=0, mnk=None, dtype=None):
+        self.mnk = mnk or self.mnk
+        self.dtype = dtype or self.dtype
+        m, n, k = self.mnk
+        g = _gen(seed)
+        self.a = (0.25 * torch.randn((m, n), generator=g, device="cuda")).to(self.dtype)
+        self.b = (0.25 * torch.randn((n, k), generator=g, device="cuda")).to(self.dtype)
+        self.gc = (0.25 * torch.randn((m, k), generator=g, device="cuda")).to(self.dtype)
+        self.c = torch.empty((m, k), dtype=self.dtype, device="cuda")
+        self.ga, self.gb = torch.zeros_like(self.a), torch.zeros_like(self.b)
+        es = self.a.element_size()
+        self.rows = m
+        self.fwd_flops = 2 * m * n * k
+        self.rev_flops = 4 * m * n * k
+        self.fwd_bytes = (m * n + n * k + m * k) * es
+        self.rev_bytes = (2 * m * k + 2 * n * k + 2 * m * n + m * n + n * k) * es
+
+    def forward(self):
+        m, n, k = self.mnk
+        inner_product("ij_jk_ik", self.a, self.b, 1.0, self.c, 0.0, m, n, k)
+
+    def reverse(self):  # src/ops/inner_product.zig:305-326 without the scratch transposes
+        m, n, k = self.mnk
+        inner_product("ij_kj_ik", self.gc, self.b, 1.0, self.ga, 1.0, m, k, n)
+        inner_product("ji_jk_ik", self.a, self.gc, 1.0, self.gb, 1.0, n, m, k)
+
+
+WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b, Copy, Permutate, Gemm)}
 
 DESCRIPTION = {
     "cfg1": "softmax fwd r32 [256,1024]",
@@ -264,4 +344,6 @@ DESCRIPTION = {
     "cfg5a": "vocabulary softmax fwd r32 [512,151936]",
     "cfg5b": "vocabulary softmax fwd r32 [2048,50257]",
     "copy": "plain copy r32 flat 2^28 (calibration)",
+    "permutate": "transpose r32 [16384,16384], reverse = accumulating transpose",
+    "gemm": "matrix product r16 (fp32 accumulate) 8192^3 on rocBLAS, reverse = its two gradient products",
 }

@@ -29,6 +29,11 @@
  *                                                                       reference body mis-indexes dst, :42-43)
  *   oracle_broadcast_i_ij    src/cuda/nvcc_src/broadcast_i_ij.cu:35        dst_ij = src_i + alpha*dst_ij
  *   oracle_broadcast_j_ij    src/cuda/nvcc_src/broadcast_j_ij.cu:30        dst_ij = src_j + alpha*dst_ij
+ *   oracle_permutate_ij_ji   src/cuda/nvcc_src/permutate_ij_ji.cu:20-44    dst_ji = src_ij + alpha*dst_ji
+ *   oracle_inner_product     src/cuda/nvcc_src/inner_product_ij_jk_ik.cu:12-26 with the operand forms of
+ *                            src/ops/inner_product.zig:286-383: c_ik = alpha * sum_j op(a)_ij op(b)_jk + beta*c_ik
+ *                            (the arithmetic itself is cuBLAS in the reference, src/cuda/gemm_dispatch.cuh:24-110:
+ *                            a closed-source library, restated here as the textbook triple loop)
  *   oracle_selu / _reverse   no reference kernel (only README.md:97); signature and the
  *                            accumulate-into-gradient convention follow relu.cu:11-12 and
  *                            relu_reverse.cu:12-14. Closed form stated below.
@@ -278,6 +283,40 @@ void oracle_broadcast_j_ij(int key, const void* src, const void* dst_in, double*
 }
 
 /* ---- softmax over the last dim -------------------------------------------------------- */
+
+/* ---- transpose and matrix product ------------------------------------------------------- */
+
+void oracle_permutate_ij_ji(int key, const void* src, const void* dst_in, double* dst, double alpha,
+                            size_t rows, size_t cols) {
+#pragma omp parallel for schedule(static)
+  for (size_t j = 0; j < cols; ++j)
+    for (size_t i = 0; i < rows; ++i)
+      dst[j * rows + i] = ld(key, src, i * cols + j) + (dst_in ? alpha * ld(key, dst_in, j * rows + i) : 0.0);
+}
+
+/* a is [m,n] (stored [n,m] when ta), b is [n,k] (stored [k,n] when tb), c is [m,k]. `scale`, when
+ * given, receives |alpha| * sum_j |op(a)_ij op(b)_jk| + |beta c_ik|: the size of the terms that a
+ * finite-precision sum of the same products can lose to rounding. */
+void oracle_inner_product(int key, int ta, int tb, const void* a, const void* b, double alpha,
+                          const void* c_in, double beta, double* c, double* scale,
+                          size_t m, size_t n, size_t k) {
+#pragma omp parallel for schedule(static)
+  for (size_t i = 0; i < m; ++i) {
+    for (size_t l = 0; l < k; ++l) {
+      double s = 0.0, mag = 0.0;
+      for (size_t j = 0; j < n; ++j) {
+        const double x = ta ? ld(key, a, j * m + i) : ld(key, a, i * n + j);
+        const double y = tb ? ld(key, b, l * n + j) : ld(key, b, j * k + l);
+        s += x * y;
+        mag += fabs(x * y);
+      }
+      const double old = (c_in && beta != 0.0) ? beta * ld(key, c_in, i * k + l) : 0.0;
+      c[i * k + l] = alpha * s + old;
+      if (scale) scale[i * k + l] = fabs(alpha) * mag + fabs(old);
+    }
+  }
+}
+
 
 /* y_ij = exp(x_ij - max_j x_ij) / sum_j exp(x_ij - max_j x_ij); -inf entries give exactly 0.
  * A row with no finite entry (all -inf) yields NaN, as the closed form does. */

@@ -252,3 +252,34 @@ def set_regime(r):
 def set_cluster_tuning(packs_per_block=0, spin_limit=1 << 22):
     kernels, _ = lib()
     kernels.mpSetClusterTuning(int(packs_per_block), int(spin_limit))
+
+
+def permutate(src, dst, alpha=0.0):
+    rows, cols = src.shape
+    _call("permutate_ij_ji", src.dtype, src.data_ptr(), dst.data_ptr(), float(alpha), rows, cols)
+
+
+class BlasStream:
+    """A stream context from mpInitStream: the only kind that carries the BLAS handle the
+    matrix-product launchers need. Work on it is fenced against torch's stream by full
+    device synchronisation on entry and a stream synchronisation after each call."""
+
+    def __enter__(self):
+        _, utils = lib()
+        torch.cuda.synchronize()
+        self.sc = utils.mpInitStream()
+        assert self.sc.blas_handle.ptr
+        return self
+
+    def __exit__(self, *exc):
+        _, utils = lib()
+        utils.mpStreamSynchronize(self.sc)
+        utils.mpDeinitStream(self.sc)
+
+    def inner_product(self, form, a, b, alpha, c, beta, m, n, k):
+        """form: "ij_jk_ik", "ij_kj_ik" or "ji_jk_ik"."""
+        kernels, utils = lib()
+        torch.cuda.synchronize()
+        getattr(kernels, "inner_product_" + form)[KEY[a.dtype]](
+            a.data_ptr(), b.data_ptr(), float(alpha), c.data_ptr(), float(beta), m, n, k, self.sc)
+        utils.mpStreamSynchronize(self.sc)

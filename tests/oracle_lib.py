@@ -68,6 +68,8 @@ _translate = _sig("oracle_translate", _it, _vp, _db, _vp, _sz)
 _fill = _sig("oracle_fill", _it, _db, _vp, _sz)
 _sequence = _sig("oracle_sequence", _it, _db, _db, _vp, _sz)
 _copy = _sig("oracle_copy", _it, _vp, _vp, _sz)
+_permutate = _sig("oracle_permutate_ij_ji", _it, _vp, _vp, _vp, _db, _sz, _sz)
+_inner = _sig("oracle_inner_product", _it, _it, _it, _vp, _vp, _db, _vp, _db, _vp, _vp, _sz, _sz, _sz)
 
 
 def threads():
@@ -254,6 +256,26 @@ def broadcast_j_ij(src, m, n, dst_in=None, alpha=0.0):
     dst = _out((m, n))
     _bcast_j(k, _p(src), _p(dst_in), _p(dst), float(alpha), m, n)
     return dst
+
+
+def permutate_ij_ji(src, dst_in=None, alpha=0.0):
+    k, (src, dst_in) = _prep(src, dst_in)
+    rows, cols = src.shape
+    dst = _out((cols, rows))
+    _permutate(k, _p(src), _p(dst_in), _p(dst), float(alpha), rows, cols)
+    return dst
+
+
+def inner_product(a, b, alpha=1.0, c_in=None, beta=0.0, ta=False, tb=False, with_scale=False):
+    """c[m,k] = alpha * op(a) . op(b) + beta * c_in; a is stored [n,m] when ta, b [k,n] when tb."""
+    key, (a, b, c_in) = _prep(a, b, c_in)
+    m, n = (a.shape[1], a.shape[0]) if ta else a.shape
+    k = b.shape[0] if tb else b.shape[1]
+    assert (b.shape[1] if tb else b.shape[0]) == n
+    c = _out((m, k))
+    scale = _out((m, k))
+    _inner(key, int(ta), int(tb), _p(a), _p(b), float(alpha), _p(c_in), float(beta), _p(c), _p(scale), m, n, k)
+    return (c, scale) if with_scale else c
 
 
 def softmax_ij_j(x):

@@ -1,0 +1,139 @@
+"""GPU parity of the transpose and the matrix products, through the C-ABI, against the fp64
+oracle. The products are compared with a tolerance relative to the size of the summed terms
+(|alpha| * sum_j |a_ij b_jk| + |beta c_ik|): r32 1e-5, r16 2e-3, r64 1e-12 of that."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_lib as G
+import oracle_lib as O
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float16, torch.float32, torch.float64]
+IDS = ["r16", "r32", "r64"]
+
+
+def rng(seed):
+    return np.random.default_rng(seed)
+
+
+# rows x cols: single element, vectors, tiles exactly, one past a tile, ragged both ways,
+# odd sizes that force the scalar paths on one side or both
+TRANSPOSE_SHAPES = [(1, 1), (1, 7), (7, 1), (3, 2), (64, 64), (128, 128), (65, 64), (64, 65), (129, 257),
+                    (32, 1000), (1000, 32), (8, 4096), (50257, 3), (100, 104), (104, 100), (1027, 513)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("shift", [0, 1])
+def test_permutate_forward_and_blend(dtype, shift):
+    r = rng(31)
+    for (rows, cols) in TRANSPOSE_SHAPES:
+        for alpha in (0.0, 1.0, -0.5):
+            G.say(f"permutate dtype={dtype} shape=({rows},{cols}) alpha={alpha} shift={shift}")
+            src = G.dev(r.normal(0, 1, (rows, cols)), dtype, shift)
+            dst = G.dev(r.normal(0, 1, (cols, rows)), dtype, shift)
+            before = G.host(dst.t).copy()
+            G.permutate(src.t, dst.t, alpha)
+            ref = O.permutate_ij_ji(G.host(src.t), before if alpha else None, alpha)
+            if alpha == 0.0:
+                assert np.array_equal(G.host(dst.t).astype(np.float64), ref), "transpose must move bits unchanged"
+            else:
+                G.compare(dst.t, ref, dtype, f"permutate ({rows},{cols}) alpha {alpha}", rowwise=False,
+                          scale=np.abs(G.host(src.t).T.astype(np.float64)) + abs(alpha) * np.abs(before.astype(np.float64)))
+            dst.check("permutate dst")
+            src.check("permutate src")
+
+
+def test_permutate_mixed_alignment_and_empty():
+    f32 = torch.float32
+    r = rng(32)
+    for (s_shift, d_shift) in ((0, 1), (1, 0), (3, 2)):
+        G.say(f"permutate r32 (96,200) shifts {s_shift},{d_shift}")
+        src = G.dev(r.normal(0, 1, (96, 200)), f32, s_shift)
+        dst = G.Guarded((200, 96), f32, d_shift)
+        G.permutate(src.t, dst.t)
+        assert torch.equal(dst.t, src.t.t())
+        dst.check("permutate")
+    G.say("permutate with an empty dimension")
+    src, dst = G.Guarded((0, 5), f32), G.Guarded((5, 0), f32)
+    G.permutate(src.t, dst.t)
+    torch.cuda.synchronize()
+    dst.check("empty permutate")
+
+
+def test_permutate_involution_at_size():
+    # a large ragged matrix: transposing twice returns every bit (size-independent property)
+    G.say("permutate r16 (8191, 4104) twice")
+    x = torch.randn(8191, 4104, device="cuda").to(torch.float16)
+    y = torch.empty(4104, 8191, dtype=torch.float16, device="cuda")
+    z = torch.empty_like(x)
+    G.permutate(x, y)
+    G.permutate(y, z)
+    assert torch.equal(y, x.t())
+    assert torch.equal(z, x)
+
+
+GEMM_SHAPES = [(1, 1, 1), (3, 2, 2), (2, 3, 4), (5, 7, 3), (1, 64, 9), (9, 64, 1), (33, 1, 17), (64, 64, 64),
+               (129, 255, 65), (256, 1024, 96), (7, 4099, 5)]
+FORMS = [("ij_jk_ik", False, False), ("ij_kj_ik", False, True), ("ji_jk_ik", True, False)]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_inner_product_every_operand_form(dtype):
+    r = rng(33)
+    with G.BlasStream() as bs:
+        for (m, n, k) in GEMM_SHAPES:
+            for form, ta, tb in FORMS:
+                for alpha, beta in ((1.0, 0.0), (0.5, 1.0), (-2.0, -0.25)):
+                    G.say(f"inner_product_{form} dtype={dtype} m,n,k=({m},{n},{k}) alpha={alpha} beta={beta}")
+                    a = G.dev(r.normal(0, 1, (n, m) if ta else (m, n)), dtype)
+                    b = G.dev(r.normal(0, 1, (k, n) if tb else (n, k)), dtype)
+                    c = G.dev(r.normal(0, 1, (m, k)), dtype)
+                    before = G.host(c.t).copy()
+                    bs.inner_product(form, a.t, b.t, alpha, c.t, beta, m, n, k)
+                    ref, scale = O.inner_product(G.host(a.t), G.host(b.t), alpha, before if beta else None, beta,
+                                                 ta=ta, tb=tb, with_scale=True)
+                    G.compare(c.t, ref, dtype, f"inner_product_{form} ({m},{n},{k}) {alpha},{beta}", rowwise=False,
+                              scale=scale)
+                    c.check("inner product c")
+
+
+def test_inner_product_reference_example():
+    # src/examples/experimental.zig:19-34,51-62: z = x.y, then the reverse with a seed of ones
+    f32 = torch.float32
+    x = G.dev(np.array([[1, 2], [3, 4], [5, 6]]), f32)
+    y = G.dev(np.array([[1, 2], [3, 4]]), f32)
+    z, gz = G.Guarded((3, 2), f32), G.dev(np.ones((3, 2)), f32)
+    gx, gy = G.dev(np.zeros((3, 2)), f32), G.dev(np.zeros((2, 2)), f32)
+    with G.BlasStream() as bs:
+        G.say("experimental example: ij,jk->ik and its two reverse products")
+        bs.inner_product("ij_jk_ik", x.t, y.t, 1.0, z.t, 0.0, 3, 2, 2)
+        bs.inner_product("ij_kj_ik", gz.t, y.t, 1.0, gx.t, 1.0, 3, 2, 2)   # dx = G(z).T(y)
+        bs.inner_product("ji_jk_ik", x.t, gz.t, 1.0, gy.t, 1.0, 2, 3, 2)   # dy = T(x).G(z)
+    assert z.t.tolist() == [[7, 10], [15, 22], [23, 34]]
+    assert gx.t.tolist() == [[3, 7]] * 3
+    assert gy.t.tolist() == [[9, 9], [12, 12]]
+
+
+def test_inner_product_at_size_is_linear_in_its_operands():
+    # 4096^3 in r16: (A1 + A2).B against A1.B + A2.B accumulated with beta = 1; both sides come
+    # from the launcher, the tolerance is r16 output rounding on sums of 4096 products
+    n = 4096
+    G.say("inner_product r16 4096^3 linearity")
+    a1 = (torch.randn(n, n, device="cuda") * 0.25).to(torch.float16)
+    a2 = (torch.randn(n, n, device="cuda") * 0.25).to(torch.float16)
+    s = (a1.float() + a2.float())
+    exact = s.to(torch.float16).float() == s            # rows of A1 + A2 that r16 holds exactly
+    a2 = torch.where(exact, a2, torch.zeros_like(a2))   # keep the sum exact everywhere
+    asum = (a1.float() + a2.float()).to(torch.float16)
+    b = (torch.randn(n, n, device="cuda") * 0.25).to(torch.float16)
+    c_sum = torch.empty(n, n, dtype=torch.float16, device="cuda")
+    c_acc = torch.empty_like(c_sum)
+    with G.BlasStream() as bs:
+        bs.inner_product("ij_jk_ik", asum, b, 1.0, c_sum, 0.0, n, n, n)
+        bs.inner_product("ij_jk_ik", a1, b, 1.0, c_acc, 0.0, n, n, n)
+        bs.inner_product("ij_jk_ik", a2, b, 1.0, c_acc, 1.0, n, n, n)
+    scale = float((a1.float().abs().mean() + a2.float().abs().mean()) * b.float().abs().mean() * n)
+    err = (c_sum.float() - c_acc.float()).abs().max().item()
+    assert err <= 4e-3 * scale, (err, scale)

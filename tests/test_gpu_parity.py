@@ -557,7 +557,7 @@ def test_rmsnorm_reverse_is_deterministic():
 def test_launchers_follow_the_stream_of_the_context():
     kernels, utils = G.lib()
     sc = utils.mpInitStream()
-    assert sc.blas_handle.ptr is None and sc.hip_stream.ptr
+    assert sc.blas_handle.ptr and sc.hip_stream.ptr  # the stream and its BLAS handle
     r = rng(70)
     n = 1 << 20
     a, b = G.dev(r.normal(0, 1, n), torch.float32), G.dev(r.normal(0, 1, n), torch.float32)

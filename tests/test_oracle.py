@@ -111,6 +111,56 @@ def test_reduce_blend_and_orientation():
     np.testing.assert_allclose(O.reduce_ij_j(src, d_j, -2.0), src.sum(0) - 2.0 * d_j, rtol=1e-14)
 
 
+def test_permutate_is_numpy_transpose_with_blend():
+    src = RNG.normal(0, 1, (7, 13)).astype(np.float32)
+    old = RNG.normal(0, 1, (13, 7)).astype(np.float32)
+    assert np.array_equal(O.permutate_ij_ji(src), src.T.astype(np.float64))
+    assert np.array_equal(O.permutate_ij_ji(O.permutate_ij_ji(src).astype(np.float32)), src.astype(np.float64))
+    np.testing.assert_allclose(O.permutate_ij_ji(src, old, 1.0), src.T.astype(np.float64) + old, rtol=1e-15)
+    np.testing.assert_allclose(O.permutate_ij_ji(src, old, -0.5), src.T.astype(np.float64) - 0.5 * old, rtol=1e-15)
+    # a non-square index slip (cols used as the output stride) would move this single entry
+    e = np.zeros((3, 5), dtype=np.float64)
+    e[2, 1] = 1.0
+    out = O.permutate_ij_ji(e)
+    assert out.shape == (5, 3) and out[1, 2] == 1.0 and out.sum() == 1.0
+
+
+def test_inner_product_known_answers_and_operand_forms():
+    # src/examples/experimental.zig:19-34,51-62 — x = [[1,2],[3,4],[5,6]], y = [[1,2],[3,4]]:
+    # z = x.y by hand; with a seed of ones the reverse gives dx = ones.T(y) (rows [3,7]) and
+    # dy = T(x).ones (rows [9,9],[12,12]), the values the example prints as bn and dn.
+    x = np.array([[1, 2], [3, 4], [5, 6]], dtype=np.float32)
+    y = np.array([[1, 2], [3, 4]], dtype=np.float32)
+    assert np.array_equal(O.inner_product(x, y), [[7, 10], [15, 22], [23, 34]])
+    ones = np.ones((3, 2), dtype=np.float32)
+    assert np.array_equal(O.inner_product(ones, y, tb=True), [[3, 7]] * 3)       # ij,kj->ik
+    assert np.array_equal(O.inner_product(x, ones, ta=True), [[9, 9], [12, 12]])  # ji,jk->ik
+    # library routine in fp64, every operand form, non-square everywhere
+    m, n, k = 5, 7, 3
+    a, b = RNG.normal(0, 1, (m, n)), RNG.normal(0, 1, (n, k))
+    c0 = RNG.normal(0, 1, (m, k))
+    ref = a @ b
+    np.testing.assert_allclose(O.inner_product(a, b), ref, rtol=1e-13, atol=1e-14)
+    np.testing.assert_allclose(O.inner_product(a, np.ascontiguousarray(b.T), tb=True), ref, rtol=1e-13, atol=1e-14)
+    np.testing.assert_allclose(O.inner_product(np.ascontiguousarray(a.T), b, ta=True), ref, rtol=1e-13, atol=1e-14)
+    np.testing.assert_allclose(O.inner_product(a, b, 0.5, c0, -2.0), 0.5 * ref - 2.0 * c0, rtol=1e-13, atol=1e-14)
+    # identity and (A.B)^T = B^T.A^T
+    np.testing.assert_allclose(O.inner_product(a, np.eye(n)), a, rtol=0)
+    np.testing.assert_allclose(O.inner_product(np.ascontiguousarray(b.T), np.ascontiguousarray(a.T)), ref.T, rtol=1e-13, atol=1e-14)
+    # the scale output is the same product over absolute values
+    _, scale = O.inner_product(a, b, 0.5, c0, -2.0, with_scale=True)
+    np.testing.assert_allclose(scale, 0.5 * (np.abs(a) @ np.abs(b)) + 2.0 * np.abs(c0), rtol=1e-13)
+    # autograd of z = scale * x.y gives the reverse operand forms used by src/ops/inner_product.zig:305-326
+    at, bt = t64(a).requires_grad_(True), t64(b).requires_grad_(True)
+    gz = RNG.normal(0, 1, (m, k))
+    (1.5 * at @ bt).backward(t64(gz))
+    np.testing.assert_allclose(O.inner_product(gz, b, 1.5, tb=True), at.grad.numpy(), rtol=1e-13, atol=1e-14)
+    np.testing.assert_allclose(O.inner_product(a, gz, 1.5, ta=True), bt.grad.numpy(), rtol=1e-13, atol=1e-14)
+    # half inputs are read exactly
+    ah, bh = a.astype(np.float16), b.astype(np.float16)
+    np.testing.assert_allclose(O.inner_product(ah, bh), ah.astype(np.float64) @ bh.astype(np.float64), rtol=1e-13, atol=1e-14)
+
+
 def test_broadcasts_are_the_reverses_of_the_reductions():
     m, n = 5, 9
     src_i, src_j = RNG.normal(0, 1, m), RNG.normal(0, 1, n)
