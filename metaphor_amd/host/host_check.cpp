@@ -9,6 +9,8 @@
  * reverse are one kernel each, and writes inputs, outputs and gradients as raw little-endian
  * files for the Python test to compare with the CPU oracle; the same for softmax and RMSNorm
  * through the graph, and for an expression that must NOT fuse (a repeated input).
+ * Part 3 is the matrix side: the reference's src/examples/experimental.zig, every inner-product
+ * expression, permutate, reduce / broadcast, and checkpoint files.
  */
 #include <cmath>
 #include <cstdio>
@@ -236,6 +238,111 @@ static int row_ops(mp::Stream stream) {
   return 0;
 }
 
+/* Part 3: the matrix side of the surface. First the reference's own example with its hand-computable
+ * answers (src/examples/experimental.zig:19-62), then every inner-product expression, permutate,
+ * reduce / broadcast, dilate and translate on random operands, dumped for the oracle check, and a
+ * checkpoint round trip in the reference's file format. */
+static int matrix_ops(mp::Stream stream) {
+  mp::Graph* G = mp::Graph::init({stream, mp::Mode::train});
+  {
+    mp::Tensor x = G->tensor(mp::TensorClass::wgt, mp::Tag::r32, {3, 2});
+    mp::Tensor y = G->tensor(mp::TensorClass::wgt, mp::Tag::r32, {2, 2});
+    mp::algo::sequence(x, 1.0, 1.0);
+    mp::algo::sequence(y, 1.0, 1.0);
+    mp::Tensor z = mp::ops::inner_product(x, y, "ij,jk->ik");
+    mp::Tensor a = mp::ops::reduce(y, "ij->i");
+    mp::Tensor b = mp::ops::broadcast(a, x.sizes(), "j->ij");
+    mp::Tensor c = mp::ops::reduce(x, "ij->j");
+    mp::Tensor d = mp::ops::broadcast(c, y.sizes(), "i->ij");
+    CHECK((z.native<float>() == std::vector<float>{7, 10, 15, 22, 23, 34}));
+    CHECK((b.native<float>() == std::vector<float>{3, 7, 3, 7, 3, 7}));
+    CHECK((d.native<float>() == std::vector<float>{9, 9, 12, 12}));
+    z.reverse(mp::ReverseCleanup::keep);
+    CHECK(x.native_grad<float>() == b.native<float>()); /* reverse mode agrees with the forward-mode check */
+    CHECK(y.native_grad<float>() == d.native<float>());
+    G->reset(mp::Graph::ResetGroup::node, mp::Graph::ResetComponent::all);
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+  }
+  Rng r{99};
+  const size_t m = 37, n = 53, k = 29;
+  const auto ha = r.normal(m * n, 0, 1), hb = r.normal(n * k, 0, 1), hbt = r.normal(k * n, 0, 1);
+  const auto hat = r.normal(n * m, 0, 1), hv = r.normal(n, 0, 1), hu = r.normal(m, 0, 1);
+  const auto hg = r.normal(m * k, 0, 1), hgi = r.normal(m, 0, 1), hgn = r.normal(n, 0, 1), hgmn = r.normal(m * n, 0, 1);
+  dump("mx_a", ha); dump("mx_b", hb); dump("mx_bt", hbt); dump("mx_at", hat); dump("mx_v", hv); dump("mx_u", hu);
+  dump("mx_g", hg); dump("mx_gi", hgi); dump("mx_gn", hgn); dump("mx_gmn", hgmn);
+  mp::Tensor a = leaf(G, mp::TensorClass::wgt, {m, n}, ha);
+  mp::Tensor b = leaf(G, mp::TensorClass::wgt, {n, k}, hb);
+  mp::Tensor bt = leaf(G, mp::TensorClass::wgt, {k, n}, hbt);
+  mp::Tensor at = leaf(G, mp::TensorClass::wgt, {n, m}, hat);
+  mp::Tensor v = leaf(G, mp::TensorClass::wgt, {n}, hv);
+  mp::Tensor u = leaf(G, mp::TensorClass::wgt, {m}, hu);
+  struct Case { const char* name; const char* expr; mp::Tensor x, y; const std::vector<float>* seed; double scale; };
+  const Case cases[] = {
+      {"nn", "ij,jk->ik", a, b, &hg, 1.0},   {"nt", "ij,kj->ik", a, bt, &hg, 0.5}, {"tn", "ji,jk->ik", at, b, &hg, -2.0},
+      {"mv", "ij,j->i", a, v, &hgi, 1.0},    {"vm", "i,ij->j", u, a, &hgn, 1.5},
+  };
+  for (const Case& c : cases) {
+    const size_t before = G->launches;
+    mp::Tensor z = mp::ops::inner_product_scaled(c.x, c.y, c.scale, c.expr);
+    CHECK(G->launches == before + 1); /* transposed operands cost no extra kernel */
+    dump(std::string("mx_") + c.name + "_z", z.native<float>());
+    set_grad(z, *c.seed);
+    const size_t mid = G->launches;
+    z.reverse(mp::ReverseCleanup::keep);
+    CHECK(G->launches == mid + 2); /* one product per operand gradient, no zero fills, no transposes */
+    dump(std::string("mx_") + c.name + "_dx", c.x.native_grad<float>());
+    dump(std::string("mx_") + c.name + "_dy", c.y.native_grad<float>());
+    G->reset(mp::Graph::ResetGroup::node, mp::Graph::ResetComponent::all);
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+  }
+  { /* a gradient that already exists is accumulated into: the same product twice */
+    mp::Tensor z1 = mp::ops::inner_product(a, b, "ij,jk->ik"), z2 = mp::ops::inner_product(a, b, "ij,jk->ik");
+    set_grad(z1, hg); set_grad(z2, hg);
+    z1.reverse(mp::ReverseCleanup::keep);
+    z2.reverse(mp::ReverseCleanup::keep);
+    dump("mx_nn_dx2", a.native_grad<float>());
+    G->reset(mp::Graph::ResetGroup::node, mp::Graph::ResetComponent::all);
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+  }
+  { /* t = permutate(dilate(translate(a, 0.25), 3.0)) with an upstream gradient */
+    mp::Tensor t = mp::ops::permutate(mp::ops::dilate(mp::ops::translate(a, 0.25), 3.0), "ij->ji");
+    CHECK((t.sizes() == std::vector<size_t>{n, m}));
+    dump("mx_perm", t.native<float>());
+    set_grad(t, hat); /* any [n, m] values */
+    t.reverse(mp::ReverseCleanup::keep);
+    dump("mx_perm_da", a.native_grad<float>());
+    G->reset(mp::Graph::ResetGroup::node, mp::Graph::ResetComponent::all);
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+  }
+  { /* reduce and broadcast with upstream gradients */
+    mp::Tensor ri = mp::ops::reduce(a, "ij->i");
+    set_grad(ri, hgi);
+    ri.reverse(mp::ReverseCleanup::keep);
+    dump("mx_reduce_i", ri.native<float>()); dump("mx_reduce_i_da", a.native_grad<float>());
+    G->reset(mp::Graph::ResetGroup::node, mp::Graph::ResetComponent::all);
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+    mp::Tensor bj = mp::ops::broadcast(v, {m, n}, "j->ij");
+    set_grad(bj, hgmn);
+    bj.reverse(mp::ReverseCleanup::keep);
+    dump("mx_bcast_j", bj.native<float>()); dump("mx_bcast_j_dv", v.native_grad<float>());
+    G->reset(mp::Graph::ResetGroup::node, mp::Graph::ResetComponent::all);
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+  }
+  { /* checkpoint round trip: every weight of the graph -> ckpt_0, ckpt_1, ..., overwrite, load, compare */
+    G->save(out_dir, "ckpt");
+    mp::io::save_tensor(out_dir, "single_a", a);
+    for (mp::Tensor t : {a, b, bt, at, v, u}) mp::algo::fill(t, -1.0);
+    G->load(out_dir, "ckpt");
+    CHECK(a.native<float>() == ha && b.native<float>() == hb && bt.native<float>() == hbt);
+    CHECK(at.native<float>() == hat && v.native<float>() == hv && u.native<float>() == hu);
+    mp::algo::fill(a, 0.0);
+    mp::io::load_tensor(out_dir, "single_a", a);
+    CHECK(a.native<float>() == ha);
+  }
+  G->deinit();
+  return 0;
+}
+
 int main(int argc, char** argv) {
   if (argc != 2) {
     fprintf(stderr, "usage: host_check <output directory>\n");
@@ -255,6 +362,8 @@ int main(int argc, char** argv) {
   printf("host_check: fused chain ok (one kernel forward, one kernel reverse)\n");
   if (row_ops(stream)) return 1;
   printf("host_check: softmax / rmsnorm through the graph ok\n");
+  if (matrix_ops(stream)) return 1;
+  printf("host_check: inner products, permutate, reduce / broadcast, checkpoint files ok\n");
 
   mp::stream::sync(stream);
   mp::stream::deinit(stream);

@@ -10,6 +10,7 @@
 #include <cstdlib>
 #include <cstring>
 #include <mutex>
+#include <string>
 
 #include "chains.hpp"
 #include "kernels.hpp"
@@ -525,6 +526,119 @@ static void rmsnorm_reverse(const std::vector<OpDatum>& a) {
   z.ptr->launches += 2;
 }
 
+/* Gradient storage on first touch. Returns the blend factor for the launcher that writes it:
+ * 0 for storage just allocated (the first write overwrites, nothing is zero-filled or read
+ * back), 1 for a gradient that already holds a sum. */
+static double first_touch(Tensor t) {
+  if (t.has_grad()) return 1.0;
+  t.ptr->grad_of(t) = t.ptr->allocator_.alloc(t.dtype(), t.len(), t.ptr->stream);
+  return 0.0;
+}
+
+/* src/ops/translate.zig: gx = gz + gx */
+static void translate_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, z = a[2].t;
+  if (first_touch(x) == 0.0) kernels::copy(dkey(z), z.grad_ptr(), x.grad_ptr(), (len_t)x.len(), x.context());
+  else kernels::addition(dkey(z), z.grad_ptr(), x.grad_ptr(), x.grad_ptr(), (len_t)x.len(), x.context());
+  z.ptr->launches++;
+}
+
+/* src/ops/dilate.zig:46-58: gx += gz * value */
+static void dilate_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, z = a[2].t;
+  const double value = a[1].s;
+  if (first_touch(x) == 0.0) kernels::dilate(dkey(z), z.grad_ptr(), value, x.grad_ptr(), (len_t)x.len(), x.context());
+  else kernels::dilate_reverse(dkey(z), z.grad_ptr(), value, x.grad_ptr(), (len_t)x.len(), x.context());
+  z.ptr->launches++;
+}
+
+/* src/ops/reduce.zig:104-121,148-165: the reverse of a sum is a broadcast of its gradient */
+static void reduce_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, y = a[2].t;
+  const double beta = first_touch(x);
+  const len_t m = (len_t)x.sizes()[0], n = (len_t)x.sizes()[1];
+  if (a[1].e == "ij->i") kernels::broadcast_i_ij(dkey(y), y.grad_ptr(), x.grad_ptr(), beta, m, n, x.context());
+  else kernels::broadcast_j_ij(dkey(y), y.grad_ptr(), x.grad_ptr(), beta, m, n, x.context());
+  y.ptr->launches++;
+}
+
+/* src/ops/broadcast.zig:109-125,153-169 with the sizes of the broadcast OUTPUT (the reference
+ * reads them from the rank-1 input and would trip its own rank assertion) */
+static void broadcast_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, y = a[2].t;
+  const double beta = first_touch(x);
+  const len_t m = (len_t)y.sizes()[0], n = (len_t)y.sizes()[1];
+  if (a[1].e == "i->ij") kernels::reduce_ij_i(dkey(y), y.grad_ptr(), x.grad_ptr(), beta, m, n, x.context());
+  else kernels::reduce_ij_j(dkey(y), y.grad_ptr(), x.grad_ptr(), beta, m, n, x.context());
+  y.ptr->launches++;
+}
+
+/* src/ops/permutate.zig:58-69: the gradient comes back transposed and accumulates */
+static void permutate_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, y = a[2].t;
+  const double beta = first_touch(x);
+  kernels::permutate_ij_ji(dkey(y), y.grad_ptr(), x.grad_ptr(), beta, (len_t)y.sizes()[0], (len_t)y.sizes()[1],
+                           x.context());
+  y.ptr->launches++;
+}
+
+/* The three operand forms of the matrix product, c[m,k] = alpha * op(a) . op(b) + beta * c over n. */
+enum class Product { ij_jk, ij_kj, ji_jk };
+
+static void product(Graph* g, size_t key, Product form, const void* a, const void* b, double alpha, void* c,
+                    double beta, size_t m, size_t n, size_t k) {
+  const StreamContext ctx = g->stream->context;
+  switch (form) {
+    case Product::ij_jk: kernels::inner_product_ij_jk_ik(key, a, b, alpha, c, beta, (len_t)m, (len_t)n, (len_t)k, ctx); break;
+    case Product::ij_kj: kernels::inner_product_ij_kj_ik(key, a, b, alpha, c, beta, (len_t)m, (len_t)n, (len_t)k, ctx); break;
+    case Product::ji_jk: kernels::inner_product_ji_jk_ik(key, a, b, alpha, c, beta, (len_t)m, (len_t)n, (len_t)k, ctx); break;
+  }
+  g->launches++;
+}
+
+struct ProductPlan {
+  Product form;
+  size_t m, n, k;            /* output rows, contraction, output columns */
+  std::vector<size_t> sizes; /* of the output tensor */
+};
+
+/* src/ops/inner_product.zig:124-133 (the expression map) and :150-260 (vectors as matrices with
+ * one unit dimension). */
+static ProductPlan plan_product(Tensor x, Tensor y, const std::string& expr) {
+  const std::vector<size_t>&xs = x.sizes(), &ys = y.sizes();
+  auto need = [](bool ok) { if (!ok) panic("inner_product: operand sizes do not fit the expression"); };
+  if (expr == "ij,jk->ik") { need(xs.size() == 2 && ys.size() == 2 && xs[1] == ys[0]); return {Product::ij_jk, xs[0], xs[1], ys[1], {xs[0], ys[1]}}; }
+  if (expr == "ij,kj->ik") { need(xs.size() == 2 && ys.size() == 2 && xs[1] == ys[1]); return {Product::ij_kj, xs[0], xs[1], ys[0], {xs[0], ys[0]}}; }
+  if (expr == "ji,jk->ik") { need(xs.size() == 2 && ys.size() == 2 && xs[0] == ys[0]); return {Product::ji_jk, xs[1], xs[0], ys[1], {xs[1], ys[1]}}; }
+  if (expr == "ij,j->i") { need(xs.size() == 2 && ys.size() == 1 && xs[1] == ys[0]); return {Product::ij_jk, xs[0], xs[1], 1, {xs[0]}}; }
+  if (expr == "i,ij->j") { need(xs.size() == 1 && ys.size() == 2 && xs[0] == ys[0]); return {Product::ij_jk, 1, xs[0], ys[1], {ys[1]}}; }
+  panic("Invalid expression for inner product.");
+}
+
+/* The reverse products of src/ops/inner_product.zig:200-421, one launch each: with G = grad(z),
+ *   z = x.y     : gx += s G.T(y)   gy += s T(x).G
+ *   z = x.T(y)  : gx += s G.y      gy += s T(G).x
+ *   z = T(x).y  : gx += s y.T(G)   gy += s x.G                                              */
+static void inner_product_reverse(const std::vector<OpDatum>& a) {
+  const Tensor x = a[0].t, y = a[1].t, z = a[4].t;
+  const double s = a[2].s;
+  const ProductPlan p = plan_product(x, y, a[3].e);
+  Graph* g = z.ptr;
+  const size_t key = dkey(z);
+  const double bx = first_touch(x);
+  switch (p.form) {
+    case Product::ij_jk: product(g, key, Product::ij_kj, z.grad_ptr(), y.data_ptr(), s, x.grad_ptr(), bx, p.m, p.k, p.n); break;
+    case Product::ij_kj: product(g, key, Product::ij_jk, z.grad_ptr(), y.data_ptr(), s, x.grad_ptr(), bx, p.m, p.k, p.n); break;
+    case Product::ji_jk: product(g, key, Product::ij_kj, y.data_ptr(), z.grad_ptr(), s, x.grad_ptr(), bx, p.n, p.k, p.m); break;
+  }
+  const double by = first_touch(y); /* after x: when x and y are one tensor the second product accumulates */
+  switch (p.form) {
+    case Product::ij_jk: product(g, key, Product::ji_jk, x.data_ptr(), z.grad_ptr(), s, y.grad_ptr(), by, p.n, p.m, p.k); break;
+    case Product::ij_kj: product(g, key, Product::ji_jk, z.grad_ptr(), x.data_ptr(), s, y.grad_ptr(), by, p.k, p.m, p.n); break;
+    case Product::ji_jk: product(g, key, Product::ij_jk, x.data_ptr(), z.grad_ptr(), s, y.grad_ptr(), by, p.n, p.m, p.k); break;
+  }
+}
+
 namespace ops {
 
 Tensor add(Tensor x, Tensor y) {
@@ -584,6 +698,82 @@ Tensor rmsnorm(Tensor x, Tensor gain, double eps) {
   return z;
 }
 
+Tensor translate(Tensor x, double value) {
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
+  kernels::translate(dkey(z), px, value, z.data_ptr(), (len_t)z.len(), z.context());
+  g->launches++;
+  if (g->mode == Mode::train) attach_op(z, translate_reverse, {x, value, z});
+  return z;
+}
+
+Tensor dilate(Tensor x, double value) {
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
+  kernels::dilate(dkey(z), px, value, z.data_ptr(), (len_t)z.len(), z.context());
+  g->launches++;
+  if (g->mode == Mode::train) attach_op(z, dilate_reverse, {x, value, z});
+  return z;
+}
+
+Tensor reduce(Tensor x, const char* expr) {
+  const std::string e = expr;
+  if (e != "ij->i" && e != "ij->j") panic("Invalid expression for reduction.");
+  if (x.rank() != 2) panic("reduce: tensor must have rank 2");
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  const len_t m = (len_t)x.sizes()[0], n = (len_t)x.sizes()[1];
+  Tensor y = g->tensor(TensorClass::hid, x.dtype(), {e == "ij->i" ? (size_t)m : (size_t)n});
+  if (e == "ij->i") kernels::reduce_ij_i(dkey(y), px, y.data_ptr(), 0.0, m, n, y.context());
+  else kernels::reduce_ij_j(dkey(y), px, y.data_ptr(), 0.0, m, n, y.context());
+  g->launches++;
+  if (g->mode == Mode::train) attach_op(y, reduce_reverse, {x, e, y});
+  return y;
+}
+
+Tensor broadcast(Tensor x, const std::vector<size_t>& sizes, const char* expr) {
+  const std::string e = expr;
+  if (e != "i->ij" && e != "j->ij") panic("Invalid expression for broadcast.");
+  if (x.rank() != 1 || sizes.size() != 2) panic("broadcast: a rank-1 tensor broadcasts to rank 2");
+  if (x.len() != (e == "i->ij" ? sizes[0] : sizes[1])) panic("broadcast: sizes do not fit the expression");
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  Tensor y = g->tensor(TensorClass::hid, x.dtype(), sizes);
+  if (e == "i->ij") kernels::broadcast_i_ij(dkey(y), px, y.data_ptr(), 0.0, (len_t)sizes[0], (len_t)sizes[1], y.context());
+  else kernels::broadcast_j_ij(dkey(y), px, y.data_ptr(), 0.0, (len_t)sizes[0], (len_t)sizes[1], y.context());
+  g->launches++;
+  if (g->mode == Mode::train) attach_op(y, broadcast_reverse, {x, e, y});
+  return y;
+}
+
+Tensor permutate(Tensor x, const char* expr) {
+  if (std::strcmp(expr, "ij->ji") != 0) panic("Invalid expression for permutate.");
+  if (x.rank() != 2) panic("permutate: tensor must have rank 2");
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  Tensor y = g->tensor(TensorClass::hid, x.dtype(), {x.sizes()[1], x.sizes()[0]});
+  kernels::permutate_ij_ji(dkey(y), px, y.data_ptr(), 0.0, (len_t)x.sizes()[0], (len_t)x.sizes()[1], y.context());
+  g->launches++;
+  if (g->mode == Mode::train) attach_op(y, permutate_reverse, {x, std::string(expr), y});
+  return y;
+}
+
+Tensor inner_product_scaled(Tensor x, Tensor y, double scale, const char* expr) {
+  if (x.dtype() != y.dtype()) panic("inner_product: operands must agree in dtype");
+  const ProductPlan p = plan_product(x, y, expr);
+  Graph* g = x.ptr;
+  void* px = x.data_ptr();
+  void* py = y.data_ptr();
+  Tensor z = g->tensor(TensorClass::hid, x.dtype(), p.sizes);
+  product(g, dkey(z), p.form, px, py, scale, z.data_ptr(), 0.0, p.m, p.n, p.k);
+  if (g->mode == Mode::train) attach_op(z, inner_product_reverse, {x, y, scale, std::string(expr), z});
+  return z;
+}
+
+Tensor inner_product(Tensor x, Tensor y, const char* expr) { return inner_product_scaled(x, y, 1.0, expr); }
+
 }  // namespace ops
 
 namespace algo {
@@ -608,6 +798,73 @@ void sequence(Tensor t, double init, double step) {
 }
 
 }  // namespace algo
+
+/* ------------------------------------------------------------------ tensor files */
+
+static std::string join_path(const std::string& dir, const std::string& name) {
+  if (dir.empty()) return name;
+  return dir.back() == '/' ? dir + name : dir + "/" + name;
+}
+
+static void write_bytes(const std::string& path, const void* dev, size_t bytes, Stream s) {
+  std::vector<unsigned char> host(bytes);
+  mpMemcpyDtoH(host.data(), dev, bytes, s->context); /* returns with the bytes landed */
+  FILE* f = std::fopen(path.c_str(), "wb");
+  if (!f) panic("Failed to create save file");
+  const size_t done = std::fwrite(host.data(), 1, bytes, f);
+  if (std::fclose(f) != 0 || done != bytes) panic("Failed to write to save file");
+}
+
+static void read_bytes(const std::string& path, void* dev, size_t bytes, Stream s) {
+  FILE* f = std::fopen(path.c_str(), "rb");
+  if (!f) panic("Failed to open load file.");
+  std::vector<unsigned char> host(bytes + 1);
+  const size_t got = std::fread(host.data(), 1, bytes + 1, f); /* one more byte than fits shows a longer file */
+  std::fclose(f);
+  if (got != bytes) panic("Byte count loaded does not match provided tensor size.");
+  mpMemcpyHtoD(dev, host.data(), bytes, s->context);
+  mpStreamSynchronize(s->context);
+}
+
+namespace io {
+
+void save_tensor(const std::string& dir, const std::string& filename, Tensor x) {
+  const size_t bytes = x.len() * tag_size(x.dtype());
+  if (bytes == 0) panic("save_tensor: tensor holds no bytes");
+  write_bytes(join_path(dir, filename), x.data_ptr(), bytes, x.stream());
+}
+
+void load_tensor(const std::string& dir, const std::string& filename, Tensor x) {
+  const size_t bytes = x.len() * tag_size(x.dtype());
+  if (bytes == 0) panic("load_tensor: tensor holds no bytes");
+  x.ptr->flush(); /* pending nodes may still read the bytes about to be replaced */
+  read_bytes(join_path(dir, filename), x.data_ptr(), bytes, x.stream());
+}
+
+}  // namespace io
+
+void Graph::save(const std::string& dir, const std::string& prefix) {
+  size_t wgt_idx = 0;
+  for (const Leaf& leaf : leaves_) {
+    if (leaf.cls != TensorClass::wgt) continue;
+    const size_t bytes = leaf.data.len * tag_size(leaf.data.dtype);
+    if (bytes == 0) panic("Graph.save: a weight has no storage");
+    write_bytes(join_path(dir, prefix + "_" + std::to_string(wgt_idx)), leaf.data.ptr, bytes, stream);
+    ++wgt_idx;
+  }
+}
+
+void Graph::load(const std::string& dir, const std::string& prefix) {
+  flush();
+  size_t wgt_idx = 0;
+  for (const Leaf& leaf : leaves_) {
+    if (leaf.cls != TensorClass::wgt) continue;
+    const size_t bytes = leaf.data.len * tag_size(leaf.data.dtype);
+    if (bytes == 0) panic("Graph.load: a weight has no storage");
+    read_bytes(join_path(dir, prefix + "_" + std::to_string(wgt_idx)), leaf.data.ptr, bytes, stream);
+    ++wgt_idx;
+  }
+}
 
 namespace util {
 

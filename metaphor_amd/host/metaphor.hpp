@@ -7,7 +7,10 @@
  *   mp::device::{init, sync, check, total_memory}       src/metaphor.zig:13-18
  *   mp::stream::{init, deinit, sync}, 16 slots          src/core/utils.zig:39-111
  *   mp::Graph / mp::Tensor / GraphConfig / TensorClass  src/core/graph.zig:28-121, 256-363, 500-631
- *   mp::ops::{add, hadamard, selu, relu, softmax, rmsnorm}   src/ops/{addition,hadamard,relu}.zig
+ *   mp::ops::{add, sub, hadamard, translate, dilate, relu, reduce, broadcast, inner_product,
+ *             inner_product_scaled, permutate}           src/metaphor.zig:44-56, src/ops/*.zig
+ *   mp::ops::{selu, softmax, rmsnorm}                   new ops in the same shape
+ *   mp::io::{save_tensor, load_tensor}, Graph::{save, load}   src/core/tensor_file.zig
  *   mp::algo::{fill, copy, sequence}, mp::util::{to_device, from_device}
  * Errors follow the reference: an impossible request panics (prints and aborts), nothing returns
  * a status.
@@ -114,12 +117,16 @@ struct Tensor {
   }
 };
 
+/* src/core/graph.zig:776-829: a tensor, a scalar or an index expression such as "ij,jk->ik" */
 struct OpDatum {
-  enum Kind { tensor, scalar } kind = tensor;
+  enum Kind { tensor, scalar, expr } kind = tensor;
   Tensor t{};
   double s = 0.0;
+  std::string e;
   OpDatum(Tensor x) : kind(tensor), t(x) {}
   OpDatum(double v) : kind(scalar), s(v) {}
+  OpDatum(const char* x) : kind(expr), e(x) {}
+  OpDatum(const std::string& x) : kind(expr), e(x) {}
 };
 
 /* src/core/graph.zig:776-829: reverse through a table of functions, arguments stored by value */
@@ -174,6 +181,12 @@ class Graph {
   /* materialise every pending node; called before anything mutates tensor bytes in place */
   void flush();
 
+  /* Checkpoints in the reference's format (src/core/tensor_file.zig:25-86 and the save / load
+   * walk of src/core/graph.zig:633-702): the raw bytes of every weight leaf, one file per
+   * weight named <prefix>_<n> with n counting the weights in creation order. */
+  void save(const std::string& dir, const std::string& prefix);
+  void load(const std::string& dir, const std::string& prefix);
+
   /* core internals, public to the op modules as src/core/root.zig exports them */
   struct Leaf {
     TensorData data, grad;
@@ -214,6 +227,18 @@ Tensor sub(Tensor x, Tensor y);
 Tensor hadamard(Tensor x, Tensor y);
 Tensor selu(Tensor x);
 Tensor relu(Tensor x);
+Tensor translate(Tensor x, double value); /* src/ops/translate.zig */
+Tensor dilate(Tensor x, double value);    /* src/ops/dilate.zig */
+/* src/ops/reduce.zig: "ij->i", "ij->j"; src/ops/broadcast.zig: "i->ij", "j->ij" */
+Tensor reduce(Tensor x, const char* expr);
+Tensor broadcast(Tensor x, const std::vector<size_t>& sizes, const char* expr);
+/* src/ops/permutate.zig: "ij->ji" */
+Tensor permutate(Tensor x, const char* expr);
+/* src/ops/inner_product.zig: "ij,jk->ik", "ij,kj->ik", "ji,jk->ik", "ij,j->i", "i,ij->j".
+ * Transposed operands go to the matrix-product launchers as flags: nothing is transposed into
+ * scratch first, forward or reverse. */
+Tensor inner_product(Tensor x, Tensor y, const char* expr);
+Tensor inner_product_scaled(Tensor x, Tensor y, double scale, const char* expr);
 /* expr names the axis in the reference's notation; "ij|j" (rows over the last dim) is supported */
 Tensor softmax(Tensor x, const char* expr = "ij|j");
 Tensor rmsnorm(Tensor x, Tensor gain, double eps);
@@ -224,6 +249,12 @@ void fill(Tensor t, double value);
 void copy(Tensor src, Tensor dst);
 void sequence(Tensor t, double init, double step);
 }  // namespace algo
+
+/* src/core/tensor_file.zig:88-149: one tensor to / from a named file of raw bytes */
+namespace io {
+void save_tensor(const std::string& dir, const std::string& filename, Tensor x);
+void load_tensor(const std::string& dir, const std::string& filename, Tensor x);
+}  // namespace io
 
 namespace util {
 void to_device(const void* src, Tensor dst, size_t bytes);

@@ -90,3 +90,45 @@ def test_host_library_end_to_end(tmp_path):
     dz = O.softmax_ij_j_reverse(p, dp)
     _cmp(_load(d, "row_ds", (m, n)), 2.0 * dz, "host d softmax(s+s) / ds",
          scale=2.0 * G.softmax_reverse_scale(p, dp))
+
+    # ---- matrix side: every inner-product expression with its two gradients
+    assert "inner products, permutate, reduce / broadcast, checkpoint files ok" in res.stdout
+    m, n, k = 37, 53, 29
+    a, b, bt, at = _load(d, "mx_a", (m, n)), _load(d, "mx_b", (n, k)), _load(d, "mx_bt", (k, n)), _load(d, "mx_at", (n, m))
+    v, u = _load(d, "mx_v"), _load(d, "mx_u")
+    g, gi, gn = _load(d, "mx_g", (m, k)), _load(d, "mx_gi", (m, 1)), _load(d, "mx_gn", (1, n))
+
+    def prod(x, y, alpha, ta=False, tb=False):
+        return O.inner_product(x, y, alpha, ta=ta, tb=tb, with_scale=True)
+
+    def check(name, z, dx, dy):
+        for suffix, (ref, scale) in (("z", z), ("dx", dx), ("dy", dy)):
+            got = _load(d, f"mx_{name}_{suffix}")
+            _cmp(got.reshape(ref.shape), ref, f"host inner product {name} {suffix}", rowwise=False, scale=scale)
+
+    check("nn", prod(a, b, 1.0), prod(g, b, 1.0, tb=True), prod(a, g, 1.0, ta=True))
+    check("nt", prod(a, bt, 0.5, tb=True), prod(g, bt, 0.5), prod(g, a, 0.5, ta=True))
+    check("tn", prod(at, b, -2.0, ta=True), prod(b, g, -2.0, tb=True), prod(at, g, -2.0))
+    vcol, urow = v.reshape(n, 1), u.reshape(1, m)
+    check("mv", prod(a, vcol, 1.0), prod(gi, vcol, 1.0, tb=True), prod(a, gi, 1.0, ta=True))
+    check("vm", prod(urow, a, 1.5), prod(gn, a, 1.5, tb=True), prod(urow, gn, 1.5, ta=True))
+    ref, scale = prod(g, b, 1.0, tb=True)
+    _cmp(_load(d, "mx_nn_dx2", (m, n)), 2.0 * ref, "host inner product gradient accumulated twice", rowwise=False,
+         scale=2.0 * scale)
+    # the saved checkpoint files are the raw bytes of the weights, in creation order after the example's two
+    assert np.array_equal(np.fromfile(os.path.join(d, "single_a"), dtype=np.float32), a.ravel())
+    assert np.array_equal(np.fromfile(os.path.join(d, "ckpt_0"), dtype=np.float32), [1, 2, 3, 4, 5, 6])
+    assert np.array_equal(np.fromfile(os.path.join(d, "ckpt_2"), dtype=np.float32), a.ravel())
+    assert np.array_equal(np.fromfile(os.path.join(d, "ckpt_7"), dtype=np.float32), u)
+    # permutate(dilate(translate(a, 0.25), 3)) and its gradient
+    t = O.dilate(O.translate(a, 0.25).astype(np.float32), 3.0)
+    _cmp(_load(d, "mx_perm", (n, m)), O.permutate_ij_ji(t.astype(np.float32)), "host permutate chain", rowwise=False)
+    _cmp(_load(d, "mx_perm_da", (m, n)), 3.0 * O.permutate_ij_ji(at), "host permutate chain da", rowwise=False)
+    # reduce / broadcast and their reverses
+    _cmp(_load(d, "mx_reduce_i"), O.reduce_ij_i(a), "host reduce ij->i", rowwise=False,
+         scale=np.abs(a.astype(np.float64)).sum(1))
+    _cmp(_load(d, "mx_reduce_i_da", (m, n)), O.broadcast_i_ij(gi.ravel(), m, n), "host reduce reverse", rowwise=False)
+    gmn = _load(d, "mx_gmn", (m, n))
+    _cmp(_load(d, "mx_bcast_j", (m, n)), O.broadcast_j_ij(v, m, n), "host broadcast j->ij", rowwise=False)
+    _cmp(_load(d, "mx_bcast_j_dv"), O.reduce_ij_j(gmn), "host broadcast reverse", rowwise=False,
+         scale=np.abs(gmn.astype(np.float64)).sum(0))
