@@ -27,7 +27,8 @@ MFMA_PEAK_TFLOPS = {"gemm": 2500.0}  # dense fp16 matrix rate of the MI355X
 
 
 PROFILE_OF = {"cfg1": "cfg1_softmax", "cfg2": "cfg2_rmsnorm", "cfg3": "cfg3_softmax_r16",
-              "cfg4": "cfg4_fused_chain", "cfg5a": "cfg5a_softmax_vocab", "cfg5b": "cfg5b_softmax_vocab"}
+              "cfg4": "cfg4_fused_chain", "cfg5a": "cfg5a_softmax_vocab", "cfg5b": "cfg5b_softmax_vocab",
+              "permutate": "permutate_transpose", "gemm": "gemm_rocblas_r16"}
 
 
 def traffic_from_profile(name):
