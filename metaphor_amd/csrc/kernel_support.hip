@@ -30,9 +30,19 @@ extern "C" len_t mpSoftmaxScratchBytes(len_t dtype, len_t m, len_t n) {
   }
 }
 
+// The same for launch_softmax_ij_j_reverse_<dtype>: one word per workgroup of a shared row.
+extern "C" len_t mpSoftmaxReverseScratchBytes(len_t dtype, len_t m, len_t n) {
+  switch (dtype) {
+    case MP_R16: return mp::softmax_reverse_scratch_bytes<r16>(m, n);
+    case MP_R32: return mp::softmax_reverse_scratch_bytes<r32>(m, n);
+    case MP_R64: return mp::softmax_reverse_scratch_bytes<r64>(m, n);
+    default: mp::require(false, "mpSoftmaxReverseScratchBytes: dtype must be 0, 1 or 2"); return 0;
+  }
+}
+
 // Diagnostic: force the row regime of the softmax / RMSNorm launchers (0 auto; 1..5 = groups of
-// 64, 128, 256, 512, 1024 threads per row; 6 = streaming; 7 = cluster path of the softmax
-// forward; 8, 9 = sub-wave groups of 16 and 32 lanes of the softmax kernels). A group that cannot hold a row falls through to the next wider one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
+// 64, 128, 256, 512, 1024 threads per row; 6 = streaming; 7 = shared rows (cluster path) of the
+// softmax launchers; 8, 9 = sub-wave groups of 16 and 32 lanes of the softmax kernels). A group that cannot hold a row falls through to the next wider one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
 extern "C" void mpSetRowRegime(len_t regime) {
   mp::require(regime <= mp::REGIME_G32, "mpSetRowRegime: regime must be 0..9");
   mp::row_regime_override() = (int)regime;

@@ -21,6 +21,7 @@
 #define MP_ROW_SOFTMAX_H
 
 #include "row_dispatch.h"
+#include <type_traits>
 
 #if defined(__cplusplus) && defined(__HIPCC__)
 
@@ -247,7 +248,19 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
 constexpr int CLUSTER_THREADS = 1024, CLUSTER_MAX = WAVE;
 /* packs per thread: 24 registers of row data, so that two workgroups fit a CU (64 registers) */
 template <class T> constexpr int cluster_nv() {
+  /* r16 chunks stay in their storage type (four registers a pack) and are widened where they are
+   * used, at the price of a second exponential per element: 6 packs per thread like r32 */
+  if (sizeof(T) == 2) return 24 / 4;
   return 24 / ((PACK_BYTES / (int)sizeof(T)) * (int)(sizeof(typename precision<T>::type) / 4));
+}
+
+/* Makes the compiler forget what it knows about a register-held pack, so that widened copies
+ * of a whole chunk are not kept alive from one phase of a kernel to the next. */
+template <class V> __device__ __forceinline__ void forget(V& v) {
+  typedef unsigned words_t __attribute__((ext_vector_type(sizeof(V) / 4)));
+  words_t w = __builtin_bit_cast(words_t, v);
+  asm volatile("" : "+v"(w));
+  v = __builtin_bit_cast(V, w);
 }
 
 template <class P> struct slot_word { using type = unsigned; };
@@ -273,15 +286,19 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
   const int hi = lo + packs_per_block < g.nvec ? lo + packs_per_block : g.nvec;
 
   /* this workgroup's chunk; rank 0 also holds the row's head / tail scalars */
-  P v[NV][W];
+  constexpr bool RAW = sizeof(T) == 2; /* chunk kept in the storage type, exponentials taken twice */
+  using V = typename vec_of<T, W>::type;
+  using Held = typename std::conditional<RAW, V, P[W]>::type;
+  Held v[NV];
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int p = lo + k * G + lane;
     if (p < hi) {
-      load_pack_nt<T, W>(body + (size_t)p * W, v[k]);
+      if constexpr (RAW) v[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(body + (size_t)p * W));
+      else load_pack_nt<T, W>(body + (size_t)p * W, v[k]);
     } else {
 #pragma unroll
-      for (int i = 0; i < W; ++i) v[k][i] = neg_inf<P>();
+      for (int i = 0; i < W; ++i) v[k][i] = RAW ? (T)neg_inf<P>() : neg_inf<P>();
     }
   }
   P edge = neg_inf<P>();
@@ -293,11 +310,23 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
   }
 
   P mx = edge;
+  if constexpr (RAW) { /* packed half maxima (two elements an instruction), widened once at the end */
+    V vm = v[0];
 #pragma unroll
-  for (int k = 0; k < NV; ++k)
+    for (int k = 1; k < NV; ++k) vm = __builtin_elementwise_max(vm, v[k]);
 #pragma unroll
-    for (int i = 0; i < W; ++i) mx = v[k][i] > mx ? v[k][i] : mx;
+    for (int i = 0; i < W; ++i) mx = (P)vm[i] > mx ? (P)vm[i] : mx;
+  } else {
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int i = 0; i < W; ++i) mx = (P)v[k][i] > mx ? (P)v[k][i] : mx;
+  }
   mx = group_allreduce<MaxOP, G>(mx, red[0], lane);
+  if constexpr (RAW) {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) forget(v[k]);
+  }
   /* a chunk without a finite entry (fully masked) contributes exact zeros, not exp(-inf + inf) */
   const P sh = shift_of(mx > neg_inf<P>() ? mx : (P)0);
   P s = (P)0;
@@ -305,9 +334,15 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
   for (int k = 0; k < NV; ++k)
 #pragma unroll
     for (int i = 0; i < W; ++i) {
-      v[k][i] = exp_shifted(v[k][i], sh);
-      s += v[k][i];
+      const P e = exp_shifted((P)v[k][i], sh);
+      if constexpr (!RAW) v[k][i] = e;
+      s += e;
     }
+  if constexpr (RAW) {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) forget(v[k]);
+  }
+  const P edge_x = edge;
   edge = exp_shifted(edge, sh);
   s += edge;
   s = group_allreduce<AddOP, G>(s, red[1], lane);
@@ -361,16 +396,31 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
 
   const P scale = exp_shifted(mx, shift_of(M)) / S;
   T* ybody = yr + g.head;
+  if constexpr (RAW) {
+    const P shM = shift_of(M), inv = (P)1 / S;
 #pragma unroll
-  for (int k = 0; k < NV; ++k) {
-    const int p = lo + k * G + lane;
-    if (p < hi) {
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * G + lane;
+      if (p < hi) {
+        P out[W];
 #pragma unroll
-      for (int i = 0; i < W; ++i) v[k][i] *= scale;
-      store_pack_nt<T, W>(ybody + (size_t)p * W, v[k]);
+        for (int i = 0; i < W; ++i) out[i] = exp_shifted((P)v[k][i], shM) * inv;
+        store_pack_nt<T, W>(ybody + (size_t)p * W, out);
+      }
     }
+    if (edge_at != (size_t)-1) yr[edge_at] = (T)(exp_shifted(edge_x, shM) * inv);
+  } else {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * G + lane;
+      if (p < hi) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) v[k][i] *= scale;
+        store_pack_nt<T, W>(ybody + (size_t)p * W, v[k]);
+      }
+    }
+    if (edge_at != (size_t)-1) yr[edge_at] = (T)(edge * scale);
   }
-  if (edge_at != (size_t)-1) yr[edge_at] = (T)(edge * scale);
 }
 
 template <class Word> __global__ __launch_bounds__(256) void cluster_zero_slots(Word* slots, size_t words) {
@@ -490,6 +540,150 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_rev_stream(
   }
 }
 
+/* ------------------------------------------------------------------ cluster reverse */
+
+/* The reverse of a long row, shared like the forward: each of C consecutive workgroups keeps its
+ * chunk of y and dy in registers, publishes its part of dot(y, dy) as one agent-scope atomic word
+ * (a part of exactly +0 is stored as -0, so a published word is never zero), waits for the
+ * others with the same bounded poll, and writes its chunk of dx: y and dy are read once. A
+ * workgroup that stops waiting reads the whole row again for the dot product, which is why the
+ * shared path is not taken when dx overwrites y or dy. */
+/* packs of y and of dy per thread: kept in their storage type (four registers a pack whatever T
+ * is) and widened where they are used, so a workgroup holds the same 48 KiB of each for r16, r32
+ * and r64 within 64 registers a thread */
+constexpr int CLUSTER_REV_NV = 3;
+
+template <class T, int W, bool BLEND>
+__global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_rev_cluster(
+    const T* y, const T* dy, T* dx, typename precision<T>::type alpha,
+    typename slot_word<typename precision<T>::type>::type* slots,
+    size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
+  using P = typename precision<T>::type;
+  using Word = typename slot_word<P>::type;
+  constexpr int G = CLUSTER_THREADS, NV = CLUSTER_REV_NV;
+  using V = typename vec_of<T, W>::type;
+  __shared__ P red[2][G / WAVE];
+  __shared__ P bc[2];
+  const int lane = threadIdx.x;
+  const size_t row = blockIdx.x / (unsigned)C;
+  const int rank = (int)(blockIdx.x % (unsigned)C);
+  const T* yr = y + row * n;
+  const T* gr = dy + row * n;
+  T* dr = dx + row * n;
+  const RowGeom<T, W> g(yr, n, true);
+  const T* ybody = yr + g.head;
+  const T* gbody = gr + g.head;
+  T* dbody = dr + g.head;
+  const int lo = rank * packs_per_block;
+  const int hi = lo + packs_per_block < g.nvec ? lo + packs_per_block : g.nvec;
+
+  V a[NV], b[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = lo + k * G + lane;
+    if (p < hi) {
+      a[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(ybody + (size_t)p * W));
+      b[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(gbody + (size_t)p * W));
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i) a[k][i] = b[k][i] = (T)0;
+    }
+  }
+  P ey = (P)0, eg = (P)0; /* rank 0 also holds the row's head / tail scalars */
+  size_t edge_at = (size_t)-1;
+  if (W > 1 && rank == 0) {
+    if (lane < g.head) edge_at = (size_t)lane;
+    else if (lane - g.head < g.tail) edge_at = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
+    if (edge_at != (size_t)-1) {
+      ey = (P)yr[edge_at];
+      eg = (P)gr[edge_at];
+    }
+  }
+
+  P dot = ey * eg;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    if constexpr (sizeof(T) == 2) {
+      /* v_dot2_f32_f16: two exact half products added to an fp32 sum, no widening of the chunk
+       * (which would not fit the registers of two workgroups a CU) */
+      typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+#pragma unroll
+      for (int i = 0; i < W; i += 2)
+        dot = __builtin_amdgcn_fdot2(half2_t{a[k][i], a[k][i + 1]}, half2_t{b[k][i], b[k][i + 1]}, dot, false);
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i) dot += (P)a[k][i] * (P)b[k][i];
+    }
+  }
+  dot = group_allreduce<AddOP, G>(dot, red[0], lane);
+
+  if (C > 1) {
+    if (lane == 0) {
+      const P part = dot == (P)0 ? -(P)0 : dot;
+      __hip_atomic_store(slots + (size_t)row * C + rank, __builtin_bit_cast(Word, part), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+    if (lane < WAVE) { /* wave 0: lane r waits for workgroup r of this row */
+      Word w = 1;
+      if (lane < C) {
+        Word* theirs = slots + (size_t)row * C + lane;
+        for (unsigned spins = 0;; ++spins) {
+          w = __hip_atomic_load(theirs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          if (w != 0 || spins >= spin_limit) break;
+          __builtin_amdgcn_s_sleep(4);
+        }
+      }
+      const P missing = wave_allreduce<AddOP>(w != 0 ? (P)0 : (P)1); /* every lane takes part */
+      const P total = wave_allreduce<AddOP>(lane < C && w != 0 ? __builtin_bit_cast(P, w) : (P)0);
+      if (lane == 0) {
+        bc[0] = total;
+        bc[1] = missing;
+      }
+    }
+    __syncthreads();
+    dot = bc[0];
+    if (bc[1] != (P)0) { /* gave up waiting: the whole row's dot product here */
+      P d = (P)0;
+      for (int p = lane; p < g.nvec; p += G) {
+        P u[W], v[W];
+        load_pack<T, W>(ybody + (size_t)p * W, u);
+        load_pack<T, W>(gbody + (size_t)p * W, v);
+#pragma unroll
+        for (int i = 0; i < W; ++i) d += u[i] * v[i];
+      }
+      if (W > 1) {
+        size_t e = (size_t)-1;
+        if (lane < g.head) e = (size_t)lane;
+        else if (lane - g.head < g.tail) e = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
+        if (e != (size_t)-1) d += (P)yr[e] * (P)gr[e];
+      }
+      dot = group_allreduce<AddOP, G>(d, red[1], lane);
+    }
+  }
+
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = lo + k * G + lane;
+    if (p < hi) {
+      P out[W];
+#pragma unroll
+      for (int i = 0; i < W; ++i) out[i] = (P)a[k][i] * ((P)b[k][i] - dot);
+      if constexpr (BLEND) {
+        P old[W];
+        load_pack<T, W>(dbody + (size_t)p * W, old);
+#pragma unroll
+        for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+      }
+      store_pack_nt<T, W>(dbody + (size_t)p * W, out);
+    }
+  }
+  if (edge_at != (size_t)-1) {
+    P out = ey * (eg - dot);
+    if constexpr (BLEND) out += alpha * (P)dr[edge_at];
+    dr[edge_at] = (T)out;
+  }
+}
+
 /* ------------------------------------------------------------------ host dispatch */
 
 inline unsigned stream_grid(size_t m) {
@@ -540,8 +734,27 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   MP_CHECK_LAUNCH();
 }
 
+/* Workgroups per row when the reverse shares rows; 0 when it does not. */
+template <class T> inline int cluster_rev_size(size_t packs) {
+  const int regime = row_regime_override();
+  if (regime != REGIME_AUTO && regime != REGIME_CLUSTER) return 0;
+  if (regime == REGIME_AUTO && packs <= (size_t)CLUSTER_THREADS * 2) return 0; /* one workgroup, two packs each */
+  constexpr size_t tile = (size_t)CLUSTER_THREADS * CLUSTER_REV_NV;
+  size_t ppb = (size_t)cluster_tuning().packs_per_block;
+  if (ppb == 0 || ppb > tile) ppb = tile;
+  const size_t c = (packs + ppb - 1) / ppb;
+  return c >= 1 && c <= (size_t)CLUSTER_MAX ? (int)c : 0;
+}
+
+template <class T> inline size_t softmax_reverse_scratch_bytes(size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  const int c = cluster_rev_size<T>((n + W - 1) / W);
+  return c > 1 ? m * (size_t)c * sizeof(P) : 0;
+}
+
 template <class T>
-inline void softmax_reverse(const T* y, const T* dy, T* dx, double alpha, size_t m, size_t n,
+inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, double alpha, size_t m, size_t n,
                             hipStream_t stream) {
   if (m == 0 || n == 0) return;
   using P = typename precision<T>::type;
@@ -556,9 +769,28 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, double alpha, size_t
     MP_CHECK_LAUNCH();
     return;
   }
+  const size_t packs = (n + W - 1) / W;
+  const int C = cluster_rev_size<T>(packs);
+  const bool distinct = static_cast<const void*>(dx) != static_cast<const void*>(y) &&
+                        static_cast<const void*>(dx) != static_cast<const void*>(dy);
+  if (C >= 1 && (C == 1 || (scratch != nullptr && distinct)) && m * (size_t)C < 0x7fffffffull) {
+    using Word = typename slot_word<P>::type;
+    Word* slots = static_cast<Word*>(scratch);
+    const int ppb = (int)((packs + C - 1) / C);
+    require(ppb <= CLUSTER_THREADS * CLUSTER_REV_NV, "softmax reverse: cluster chunk exceeds the register tile");
+    if (C > 1) {
+      const size_t words = m * (size_t)C;
+      cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
+    }
+    const dim3 grid((unsigned)(m * C)), block(CLUSTER_THREADS);
+    if (blend) softmax_rev_cluster<T, W, true><<<grid, block, 0, stream>>>(y, dy, dx, al, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+    else softmax_rev_cluster<T, W, false><<<grid, block, 0, stream>>>(y, dy, dx, al, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+    MP_CHECK_LAUNCH();
+    return;
+  }
   const bool ragged = !(aligned16(y) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 2, true);
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, true);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) {

@@ -502,7 +502,9 @@ static void softmax_reverse(const std::vector<OpDatum>& a) {
     grd = x.ptr->allocator_.alloc(x.dtype(), x.len(), x.ptr->stream);
   }
   const size_t n = z.sizes().back(), m = z.len() / n;
-  kernels::softmax_ij_j_reverse(dkey(z), z.data_ptr(), z.grad_ptr(), x.grad_ptr(), fresh ? 0.0 : 1.0,
+  const len_t bytes = mpSoftmaxReverseScratchBytes((len_t)dkey(z), (len_t)m, (len_t)n);
+  void* scratch = bytes ? z.stream()->get_scratch(bytes) : nullptr;
+  kernels::softmax_ij_j_reverse(dkey(z), z.data_ptr(), z.grad_ptr(), x.grad_ptr(), scratch, fresh ? 0.0 : 1.0,
                                 (len_t)m, (len_t)n, z.context());
   z.ptr->launches++;
 }

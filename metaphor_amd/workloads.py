@@ -72,9 +72,17 @@ def softmax_forward(x, y, scratch=None):
             scratch.data_ptr() if scratch is not None else None, m, n)
 
 
-def softmax_reverse(y, dy, dx, alpha=0.0):
+def softmax_reverse_scratch(dtype, m, n):
+    """Workspace for launch_softmax_ij_j_reverse (None when the rows fit one workgroup)."""
+    kernels, _ = ffi.load()
+    nbytes = int(kernels.mpSoftmaxReverseScratchBytes(KEY[dtype], m, n))
+    return torch.empty(nbytes, dtype=torch.uint8, device="cuda") if nbytes else None
+
+
+def softmax_reverse(y, dy, dx, alpha=0.0, scratch=None):
     m, n = y.shape
-    _launch("softmax_ij_j_reverse", y.dtype, y.data_ptr(), dy.data_ptr(), dx.data_ptr(), float(alpha), m, n)
+    _launch("softmax_ij_j_reverse", y.dtype, y.data_ptr(), dy.data_ptr(), dx.data_ptr(),
+            scratch.data_ptr() if scratch is not None else None, float(alpha), m, n)
 
 
 def rmsnorm_forward(x, gain, y, eps):
@@ -234,7 +242,7 @@ class Cfg4(Workload):
 
 
 class _Vocab(Workload):
-    dtype, has_reverse = torch.float32, False
+    dtype, has_reverse = torch.float32, True  # the configs name the forward; the reverse is measured beside it
 
     def __init__(self, seed=0, shape=None):
         self.shape = shape or self.shape
@@ -244,13 +252,19 @@ class _Vocab(Workload):
         spike = torch.randint(0, n, (m,), generator=g, device="cuda")
         self.x[torch.arange(m, device="cuda"), spike] += 12.0
         self.y = torch.empty_like(self.x)
+        self.dy = torch.randn(self.shape, generator=g, device="cuda", dtype=torch.float32)
+        self.dx = torch.empty_like(self.x)
         self.scratch = softmax_scratch(torch.float32, m, n)
+        self.rev_scratch = softmax_reverse_scratch(torch.float32, m, n)
         self.rows = m
         self.fwd_bytes = 2 * m * n * 4
-        self.rev_bytes = 0
+        self.rev_bytes = 3 * m * n * 4
 
     def forward(self):
         softmax_forward(self.x, self.y, self.scratch)
+
+    def reverse(self):
+        softmax_reverse(self.y, self.dy, self.dx, 0.0, self.rev_scratch)
 
 
 class Cfg5a(_Vocab):
@@ -341,8 +355,8 @@ DESCRIPTION = {
     "cfg2": "RMSNorm fwd+rev r32 [8192,4096], gain [4096], eps 1e-6",
     "cfg3": "causal attention-score softmax fwd+rev r16 [524288,2048]",
     "cfg4": "fused selu((a+b)*(c+d)) fwd+rev r32 flat 2^28",
-    "cfg5a": "vocabulary softmax fwd r32 [512,151936]",
-    "cfg5b": "vocabulary softmax fwd r32 [2048,50257]",
+    "cfg5a": "vocabulary softmax fwd (+rev) r32 [512,151936]",
+    "cfg5b": "vocabulary softmax fwd (+rev) r32 [2048,50257]",
     "copy": "plain copy r32 flat 2^28 (calibration)",
     "permutate": "transpose r32 [16384,16384], reverse = accumulating transpose",
     "gemm": "matrix product r16 (fp32 accumulate) 8192^3 on rocBLAS, reverse = its two gradient products",

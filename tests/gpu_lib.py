@@ -222,9 +222,20 @@ def softmax(x, y, scratch="auto"):
         guard.check("softmax scratch")
 
 
-def softmax_reverse(y, dy, dx, alpha=0.0):
+def softmax_reverse(y, dy, dx, alpha=0.0, scratch="auto"):
+    """scratch: "auto" sizes and passes the workspace the launcher asks for, None passes NULL."""
     m, n = y.shape
-    _call("softmax_ij_j_reverse", y.dtype, y.data_ptr(), dy.data_ptr(), dx.data_ptr(), float(alpha), m, n)
+    guard = None
+    if isinstance(scratch, str):
+        kernels, _ = lib()
+        nbytes = int(kernels.mpSoftmaxReverseScratchBytes(KEY[y.dtype], m, n))
+        guard = Guarded((nbytes,), torch.uint8) if nbytes else None
+        scratch = guard.t if guard is not None else None
+    _call("softmax_ij_j_reverse", y.dtype, y.data_ptr(), dy.data_ptr(), dx.data_ptr(),
+          scratch.data_ptr() if scratch is not None else None, float(alpha), m, n)
+    if guard is not None:
+        torch.cuda.synchronize()
+        guard.check("softmax reverse scratch")
 
 
 def rmsnorm(x, g, y, eps):

@@ -427,6 +427,50 @@ def test_softmax_reverse_all_regimes(dtype, regime):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("packs,spin", [(0, 1 << 22), (64, 1 << 22), (3, 1 << 22), (64, 0), (1000, 2)],
+                         ids=["default", "64packs", "3packs", "64packs-nowait", "1000packs-2polls"])
+def test_softmax_reverse_cluster_path(dtype, packs, spin):
+    """Several workgroups per row exchanging their parts of dot(y, dy) through scratch; with a
+    poll limit of 0 or 2 most workgroups give up waiting and read the whole row themselves."""
+    r = rng(44)
+    G.set_regime(CLUSTER)
+    G.set_cluster_tuning(packs, spin)
+    for (m, n) in [(3, 7), (5, 64), (4, 1000), (6, 2048), (33, 5000), (2, 50257), (2, 151936), (130, 777)]:
+        for alpha in (0.0, 1.0):
+            for shift in (0, 1):
+                G.say(f"softmax rev cluster dtype={dtype} packs={packs} spin={spin} shape=({m},{n}) alpha={alpha} shift={shift}")
+                y = G.dev(O.softmax_ij_j(_softmax_inputs(r, m, n, dtype, masked=(m % 2 == 0))), dtype, shift)
+                dy = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+                dx = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+                before = G.host(dx.t).copy()
+                G.softmax_reverse(y.t, dy.t, dx.t, alpha)
+                ref = O.softmax_ij_j_reverse(G.host(y.t), G.host(dy.t), before if alpha else None, alpha)
+                scale = G.softmax_reverse_scale(G.host(y.t), G.host(dy.t), before if alpha else None, alpha)
+                G.compare(dx.t, ref, dtype, f"softmax rev cluster ({m},{n}) packs {packs} spin {spin}", scale=scale)
+                for g in (y, dy, dx):
+                    g.check("softmax rev cluster")
+
+
+def test_softmax_reverse_long_rows_in_place_and_without_scratch():
+    # dx written over dy, and a NULL workspace: both must leave the shared-row path
+    r = rng(45)
+    f32 = torch.float32
+    for (m, n) in [(3, 151936), (4, 50257)]:
+        y = G.dev(O.softmax_ij_j(r.normal(0, 3, (m, n))), f32)
+        dy = G.dev(r.normal(0, 1, (m, n)), f32)
+        ref = O.softmax_ij_j_reverse(G.host(y.t), G.host(dy.t))
+        scale = G.softmax_reverse_scale(G.host(y.t), G.host(dy.t))
+        dx = G.Guarded((m, n), f32)
+        G.say(f"softmax rev NULL scratch ({m},{n})")
+        G.softmax_reverse(y.t, dy.t, dx.t, 0.0, scratch=None)
+        G.compare(dx.t, ref, f32, f"softmax rev no scratch ({m},{n})", scale=scale)
+        G.say(f"softmax rev in place ({m},{n})")
+        G.softmax_reverse(y.t, dy.t, dy.t, 0.0)
+        G.compare(dy.t, ref, f32, f"softmax rev in place ({m},{n})", scale=scale)
+        dy.check("in place")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 def test_softmax_reverse_unaligned(dtype):
     r = rng(41)
     for (m, n) in [(5, 100), (3, 1027), (2, 50257)]:
