@@ -11,6 +11,6 @@ extern "C" void launch_reduce_ij_j_Scalar(
   len_t n,
   StreamContext stream
 ) {
-  mp::reduce_cols<Scalar>(static_cast<const Scalar*>(src), static_cast<Scalar*>(dst), alpha, m, n,
+  mp::reduce_cols<Scalar>(static_cast<const Scalar*>(src), static_cast<Scalar*>(dst), nullptr, alpha, m, n,
                           get_stream(stream));
 }

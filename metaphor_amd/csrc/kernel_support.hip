@@ -2,7 +2,7 @@
  * Exports of the kernel library that are not per-dtype launchers: workspace sizing and the
  * diagnostic row-regime override. Compiled once (no `Scalar` replication).
  */
-#include "row_rmsnorm.h"
+#include "row_reduce.h"
 #include "row_softmax.h"
 
 // Bytes of caller-owned scratch that launch_rmsnorm_ij_j_reverse_<dtype> needs for an [m, n]
@@ -37,6 +37,17 @@ extern "C" len_t mpSoftmaxReverseScratchBytes(len_t dtype, len_t m, len_t n) {
     case MP_R32: return mp::softmax_reverse_scratch_bytes<r32>(m, n);
     case MP_R64: return mp::softmax_reverse_scratch_bytes<r64>(m, n);
     default: mp::require(false, "mpSoftmaxReverseScratchBytes: dtype must be 0, 1 or 2"); return 0;
+  }
+}
+
+// Bytes of caller-owned scratch that launch_reduce_ij_j_scratch_<dtype> can use for an [m, n]
+// problem: one partial row of accumulators per row chunk, 0 when the column strips alone fill the GPU.
+extern "C" len_t mpReduceScratchBytes(len_t dtype, len_t m, len_t n) {
+  switch (dtype) {
+    case MP_R16: return mp::reduce_cols_scratch_bytes<r16>(m, n);
+    case MP_R32: return mp::reduce_cols_scratch_bytes<r32>(m, n);
+    case MP_R64: return mp::reduce_cols_scratch_bytes<r64>(m, n);
+    default: mp::require(false, "mpReduceScratchBytes: dtype must be 0, 1 or 2"); return 0;
   }
 }
 

@@ -14,7 +14,7 @@
 #ifndef MP_ROW_REDUCE_H
 #define MP_ROW_REDUCE_H
 
-#include "row_dispatch.h"
+#include "row_rmsnorm.h" /* sum_partial_rows */
 
 #if defined(__cplusplus) && defined(__HIPCC__)
 
@@ -22,16 +22,18 @@ namespace mp {
 
 /* ------------------------------------------------------------------ row sums */
 
-/* One group of G threads per row (256/G rows per workgroup when G == 64). */
+/* One group of G threads per row; groups of 16, 32 or 64 lanes share a 256-thread workgroup
+ * (several rows per wavefront below 64), wider groups own one row per workgroup. */
 template <class T, int W, int G>
 __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
     const T* src, T* dst, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
   constexpr int BLOCK = G < 256 ? 256 : G, RPB = BLOCK / G, U = 4;
-  __shared__ P slots[G / WAVE];
+  __shared__ P slots[G < WAVE ? 1 : G / WAVE];
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
-  const size_t row = (size_t)blockIdx.x * RPB + sub;
-  if (row >= m) return; /* whole waves; wider groups own one row per workgroup */
+  const size_t want = (size_t)blockIdx.x * RPB + sub;
+  const bool live = want < m; /* a dead group of a live wavefront walks the last row and stores nothing */
+  const size_t row = live ? want : m - 1;
 
   const T* r = src + row * n;
   const RowGeom<T, W> g(r, n, true);
@@ -59,7 +61,7 @@ __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
     else if (lane - g.head < g.tail) s += (P)body[(size_t)g.nvec * W + (lane - g.head)];
   }
   s = group_allreduce<AddOP, G>(s, slots, lane);
-  if (lane == 0) dst[row] = (T)(alpha != (P)0 ? s + alpha * (P)dst[row] : s);
+  if (live && lane == 0) dst[row] = (T)(alpha != (P)0 ? s + alpha * (P)dst[row] : s);
 }
 
 template <class T>
@@ -70,33 +72,40 @@ inline void reduce_rows(const T* src, T* dst, double alpha, size_t m, size_t n, 
   require(n <= 0x40000000ull, "reduce_ij_i: row length must not exceed 2^30");
   require(m < 0x7fffffffull, "reduce_ij_i: too many rows for one grid");
   const size_t packs = (n + W - 1) / W;
-  if (packs <= 256) {
-    reduce_rows_kernel<T, W, 64><<<dim3((unsigned)((m + 3) / 4)), dim3(256), 0, stream>>>(src, dst, (P)alpha, m, n);
-  } else if (packs <= 4096) {
-    reduce_rows_kernel<T, W, 256><<<dim3((unsigned)m), dim3(256), 0, stream>>>(src, dst, (P)alpha, m, n);
-  } else {
-    reduce_rows_kernel<T, W, 1024><<<dim3((unsigned)m), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n);
-  }
+#define MP_ROWS_LAUNCH(G_) \
+  reduce_rows_kernel<T, W, G_><<<dim3((unsigned)((m + (G_ < 256 ? 256 / G_ : 1) - 1) / (G_ < 256 ? 256 / G_ : 1))), \
+                              dim3(G_ < 256 ? 256 : G_), 0, stream>>>(src, dst, (P)alpha, m, n)
+  if (packs <= 16) MP_ROWS_LAUNCH(16);
+  else if (packs <= 32) MP_ROWS_LAUNCH(32);
+  else if (packs <= 256) MP_ROWS_LAUNCH(64);
+  else if (packs <= 4096) MP_ROWS_LAUNCH(256);
+  else MP_ROWS_LAUNCH(1024);
+#undef MP_ROWS_LAUNCH
   MP_CHECK_LAUNCH();
 }
 
 /* ------------------------------------------------------------------ column sums */
 
-/* A workgroup owns LANES*CW columns; its SLICES slices take every SLICES-th row and are folded
- * through LDS in slice order, so the result does not depend on scheduling. */
-template <class T, int CW, int LANES, int SLICES>
+/* A workgroup owns LANES*CW columns of the rows [blockIdx.y * chunk, (blockIdx.y + 1) * chunk); its
+ * SLICES slices take every SLICES-th of those rows and are folded through LDS in slice order, so
+ * the result does not depend on scheduling. The sums go to `out + blockIdx.y * n`: the destination
+ * itself (O = T, one chunk holding every row, alpha blend) or a partial row of accumulators
+ * (O = precision<T>, no blend) that sum_partial_rows adds up afterwards. */
+template <class T, class O, int CW, int LANES, int SLICES>
 __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
-    const T* src, T* dst, typename precision<T>::type alpha, size_t m, size_t n) {
+    const T* src, O* out, typename precision<T>::type alpha, size_t m, size_t n, size_t chunk) {
   using P = typename precision<T>::type;
   __shared__ P part[SLICES][LANES * CW + 1];
   const int c = threadIdx.x % LANES, slice = threadIdx.x / LANES;
   const size_t col = ((size_t)blockIdx.x * LANES + c) * CW;
+  const size_t begin = (size_t)blockIdx.y * chunk, end = begin + chunk < m ? begin + chunk : m;
+  O* dst = out + (size_t)blockIdx.y * n;
   P s[CW];
 #pragma unroll
   for (int i = 0; i < CW; ++i) s[i] = (P)0;
   if (col < n) {
-    size_t r = slice;
-    for (; r + 3 * SLICES < m; r += 4 * SLICES) {
+    size_t r = begin + slice;
+    for (; r + 3 * SLICES < end; r += 4 * SLICES) {
       P v[4][CW];
 #pragma unroll
       for (int u = 0; u < 4; ++u) load_pack_nt<T, CW>(src + (r + (size_t)u * SLICES) * n + col, v[u]);
@@ -105,7 +114,7 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
 #pragma unroll
         for (int i = 0; i < CW; ++i) s[i] += v[u][i];
     }
-    for (; r < m; r += SLICES) {
+    for (; r < end; r += SLICES) {
       P v[CW];
       load_pack_nt<T, CW>(src + r * n + col, v);
 #pragma unroll
@@ -116,16 +125,38 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
   for (int i = 0; i < CW; ++i) part[slice][c * CW + i] = s[i];
   __syncthreads();
   const int mine = threadIdx.x;
-  const size_t out = (size_t)blockIdx.x * LANES * CW + mine;
-  if (mine < LANES * CW && out < n) {
+  const size_t at = (size_t)blockIdx.x * LANES * CW + mine;
+  if (mine < LANES * CW && at < n) {
     P t = (P)0;
     for (int i = 0; i < SLICES; ++i) t += part[i][mine];
-    dst[out] = (T)(alpha != (P)0 ? t + alpha * (P)dst[out] : t);
+    dst[at] = (O)(alpha != (P)0 ? t + alpha * (P)dst[at] : t);
   }
 }
 
+/* Row chunks of the two-stage column sum: enough workgroups to fill the GPU when the matrix is
+ * tall and narrow (a [262144, 1024] r32 matrix has 32 column strips), never chunks under 512
+ * rows; 1 when the strips alone are enough or the matrix is short. */
+template <class T> inline size_t reduce_cols_chunks(size_t m, size_t n) {
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  const size_t strips = (n / W + 7) / 8 ? (n / W + 7) / 8 : 1;
+  const size_t want = (size_t)compute_units() * 4;
+  if (strips >= want || n % W != 0) return 1;
+  size_t chunks = (want + strips - 1) / strips;
+  const size_t most = m / 512;
+  if (chunks > most) chunks = most;
+  if (chunks > 1024) chunks = 1024;
+  return chunks > 1 ? chunks : 1;
+}
+
+template <class T> inline size_t reduce_cols_scratch_bytes(size_t m, size_t n) {
+  const size_t chunks = reduce_cols_chunks<T>(m, n);
+  return chunks > 1 ? chunks * n * sizeof(typename precision<T>::type) : 0;
+}
+
+/* scratch: reduce_cols_scratch_bytes(m, n) bytes or NULL (then one workgroup per column strip
+ * walks every row, which leaves most of the GPU idle on tall, narrow matrices). */
 template <class T>
-inline void reduce_cols(const T* src, T* dst, double alpha, size_t m, size_t n, hipStream_t stream) {
+inline void reduce_cols(const T* src, T* dst, void* scratch, double alpha, size_t m, size_t n, hipStream_t stream) {
   if (n == 0) return;
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
@@ -133,11 +164,21 @@ inline void reduce_cols(const T* src, T* dst, double alpha, size_t m, size_t n, 
   if (packed) { /* 8 lanes x one pack = 128 bytes of every row per workgroup */
     const size_t blocks = (n / W + 7) / 8;
     require(blocks < 0x7fffffffull, "reduce_ij_j: too many columns for one grid");
-    reduce_cols_kernel<T, W, 8, 128><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n);
+    const size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;
+    if (chunks > 1) {
+      const size_t chunk = (m + chunks - 1) / chunks;
+      P* partials = static_cast<P*>(scratch);
+      reduce_cols_kernel<T, P, W, 8, 128><<<dim3((unsigned)blocks, (unsigned)chunks), dim3(1024), 0, stream>>>(
+          src, partials, (P)0, m, n, chunk);
+      MP_CHECK_LAUNCH();
+      sum_partial_rows<T>(partials, dst, alpha, (unsigned)chunks, n, stream);
+      return;
+    }
+    reduce_cols_kernel<T, T, W, 8, 128><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n, m);
   } else {
     const size_t blocks = (n + 31) / 32;
     require(blocks < 0x7fffffffull, "reduce_ij_j: too many columns for one grid");
-    reduce_cols_kernel<T, 1, 32, 32><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n);
+    reduce_cols_kernel<T, T, 1, 32, 32><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n, m);
   }
   MP_CHECK_LAUNCH();
 }
@@ -181,12 +222,79 @@ __global__ __launch_bounds__(256) void broadcast_kernel(
   }
 }
 
+/* The destination as one flat array of m*n elements behind a 16-byte aligned base: one pack per
+ * thread in one-shot 256-thread workgroups, the shape that writes fastest on this GPU, whatever
+ * the row length (short rows keep every lane busy). ALIGNED: n % W == 0, so a pack lies inside
+ * one row and the column values are one pack load; otherwise a pack may end in the next row
+ * (n >= W, so in at most one) and its values are gathered one by one. The last workgroup also
+ * writes the m*n % W elements behind the last whole pack. */
+template <class T, int W, bool BY_ROW, bool BLEND, bool ALIGNED>
+__global__ __launch_bounds__(256) void broadcast_flat_kernel(
+    const T* src, T* dst, typename precision<T>::type alpha, size_t total, unsigned n) {
+  using P = typename precision<T>::type;
+  const size_t packs = total / W;
+  const size_t base = (size_t)blockIdx.x * 256 * W; /* first element of the workgroup: uniform, so the */
+  const size_t row0 = base / n;                     /* one 64-bit division is scalar work */
+  const unsigned off = (unsigned)(base - row0 * n) + threadIdx.x * W;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx < packs) {
+    const size_t row = row0 + off / n;
+    const unsigned col = off % n;
+    P out[W];
+    if constexpr (ALIGNED) {
+      if constexpr (BY_ROW) {
+        const P v = (P)src[row];
+#pragma unroll
+        for (int i = 0; i < W; ++i) out[i] = v;
+      } else {
+        load_pack<T, W>(src + col, out);
+      }
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        const bool next = col + i >= n;
+        out[i] = BY_ROW ? (P)src[row + (next ? 1 : 0)] : (P)src[next ? col + i - n : col + i];
+      }
+    }
+    T* o = dst + idx * W;
+    if constexpr (BLEND) {
+      P old[W];
+      load_pack_nt<T, W>(o, old);
+#pragma unroll
+      for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+    }
+    store_pack_nt<T, W>(o, out);
+  }
+  if (W > 1 && blockIdx.x == gridDim.x - 1) {
+    const size_t e = packs * W + threadIdx.x;
+    if (threadIdx.x < W && e < total) {
+      P v = BY_ROW ? (P)src[e / n] : (P)src[e % n];
+      if constexpr (BLEND) v += alpha * (P)dst[e];
+      dst[e] = (T)v;
+    }
+  }
+}
+
 template <class T, bool BY_ROW>
 inline void broadcast(const T* src, T* dst, double alpha, size_t m, size_t n, hipStream_t stream) {
   if (m == 0 || n == 0) return;
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "broadcast: row length must not exceed 2^30");
+  if (aligned16(dst) && n >= (size_t)W) {
+    const size_t total = m * n, blocks = (total / W + 255) / 256 + 1; /* + 1: the tail always has a workgroup */
+    require(blocks < 0x7fffffffull, "broadcast: too many elements for one grid");
+    const dim3 grid((unsigned)blocks), block(256);
+    const bool aligned = n % W == 0 && (BY_ROW || aligned16(src));
+    const bool blend = alpha != 0.0;
+#define MP_FLAT(BLEND_, ALIGNED_) \
+  broadcast_flat_kernel<T, W, BY_ROW, BLEND_, ALIGNED_><<<grid, block, 0, stream>>>(src, dst, (P)alpha, total, (unsigned)n)
+    if (aligned) { if (blend) MP_FLAT(true, true); else MP_FLAT(false, true); }
+    else { if (blend) MP_FLAT(true, false); else MP_FLAT(false, false); }
+#undef MP_FLAT
+    MP_CHECK_LAUNCH();
+    return;
+  }
   const size_t cap = (size_t)compute_units() * 8;
   const dim3 grid((unsigned)(m < cap ? m : cap)), block(256);
   if (alpha != 0.0) broadcast_kernel<T, W, BY_ROW, true><<<grid, block, 0, stream>>>(src, dst, (P)alpha, m, n);

@@ -431,6 +431,24 @@ __global__ __launch_bounds__(FINISH_LANES * FINISH_SLICES) void rmsnorm_dgain_fi
   }
 }
 
+/* dst_j = sum of `rows` partial rows of n accumulators (fixed order, fp64) + alpha * dst_j. */
+template <class T>
+inline void sum_partial_rows(const typename precision<T>::type* partials, T* dst, double alpha, unsigned rows,
+                             size_t n, hipStream_t stream) {
+  using P = typename precision<T>::type;
+  /* wide loads need 16-byte aligned partial rows: fp32 accumulators, n % 4 == 0, aligned scratch */
+  const bool wide = sizeof(P) == 4 && (n % 4) == 0 && aligned16(partials);
+  const dim3 fblock(FINISH_LANES * FINISH_SLICES);
+  if (wide) {
+    const unsigned fin = (unsigned)((n + FINISH_LANES * 4 - 1) / (FINISH_LANES * 4));
+    rmsnorm_dgain_finish<T, 4><<<dim3(fin), fblock, 0, stream>>>(partials, dst, alpha, (int)rows, n);
+  } else {
+    const unsigned fin = (unsigned)((n + FINISH_LANES - 1) / FINISH_LANES);
+    rmsnorm_dgain_finish<T, 1><<<dim3(fin), fblock, 0, stream>>>(partials, dst, alpha, (int)rows, n);
+  }
+  MP_CHECK_LAUNCH();
+}
+
 /* ------------------------------------------------------------------ host dispatch */
 
 /* Partial rows the reverse may write: one per workgroup, at most two workgroups per CU. */
@@ -532,17 +550,7 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
     }
   }
   MP_CHECK_LAUNCH();
-  /* wide loads need 16-byte aligned partial rows: fp32 accumulators, n % 4 == 0, aligned scratch */
-  const bool wide = sizeof(P) == 4 && (n % 4) == 0 && aligned16(partials);
-  const dim3 fblock(FINISH_LANES * FINISH_SLICES);
-  if (wide) {
-    const unsigned fin = (unsigned)((n + FINISH_LANES * 4 - 1) / (FINISH_LANES * 4));
-    rmsnorm_dgain_finish<T, 4><<<dim3(fin), fblock, 0, stream>>>(partials, dg, alpha, (int)rows, n);
-  } else {
-    const unsigned fin = (unsigned)((n + FINISH_LANES - 1) / FINISH_LANES);
-    rmsnorm_dgain_finish<T, 1><<<dim3(fin), fblock, 0, stream>>>(partials, dg, alpha, (int)rows, n);
-  }
-  MP_CHECK_LAUNCH();
+  sum_partial_rows<T>(partials, dg, alpha, rows, n, stream);
 }
 
 template <class T>

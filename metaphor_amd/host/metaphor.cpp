@@ -537,6 +537,14 @@ static double first_touch(Tensor t) {
   return 0.0;
 }
 
+/* column sums with the workspace that lets tall, narrow matrices use the whole GPU */
+static void column_sums(Graph* g, size_t key, const void* src, void* dst, double alpha, size_t m, size_t n) {
+  const len_t bytes = mpReduceScratchBytes((len_t)key, (len_t)m, (len_t)n);
+  void* scratch = bytes ? g->stream->get_scratch(bytes) : nullptr;
+  kernels::reduce_ij_j_scratch(key, src, dst, scratch, alpha, (len_t)m, (len_t)n, g->stream->context);
+  g->launches += bytes ? 2 : 1;
+}
+
 /* src/ops/translate.zig: gx = gz + gx */
 static void translate_reverse(const std::vector<OpDatum>& a) {
   const Tensor x = a[0].t, z = a[2].t;
@@ -571,7 +579,7 @@ static void broadcast_reverse(const std::vector<OpDatum>& a) {
   const double beta = first_touch(x);
   const len_t m = (len_t)y.sizes()[0], n = (len_t)y.sizes()[1];
   if (a[1].e == "i->ij") kernels::reduce_ij_i(dkey(y), y.grad_ptr(), x.grad_ptr(), beta, m, n, x.context());
-  else kernels::reduce_ij_j(dkey(y), y.grad_ptr(), x.grad_ptr(), beta, m, n, x.context());
+  else { column_sums(y.ptr, dkey(y), y.grad_ptr(), x.grad_ptr(), beta, m, n); return; }
   y.ptr->launches++;
 }
 
@@ -729,8 +737,8 @@ Tensor reduce(Tensor x, const char* expr) {
   const len_t m = (len_t)x.sizes()[0], n = (len_t)x.sizes()[1];
   Tensor y = g->tensor(TensorClass::hid, x.dtype(), {e == "ij->i" ? (size_t)m : (size_t)n});
   if (e == "ij->i") kernels::reduce_ij_i(dkey(y), px, y.data_ptr(), 0.0, m, n, y.context());
-  else kernels::reduce_ij_j(dkey(y), px, y.data_ptr(), 0.0, m, n, y.context());
-  g->launches++;
+  else column_sums(g, dkey(y), px, y.data_ptr(), 0.0, m, n);
+  if (e == "ij->i") g->launches++;
   if (g->mode == Mode::train) attach_op(y, reduce_reverse, {x, e, y});
   return y;
 }

@@ -202,6 +202,22 @@ def matrix_op(stem, src, dst, alpha, m, n):
     _call(stem, src.dtype, src.data_ptr(), dst.data_ptr(), float(alpha), m, n)
 
 
+def reduce_ij_j_scratch(src, dst, alpha, m, n, scratch="auto"):
+    """Column sums through the workspace-taking launcher; "auto" sizes the workspace, None passes NULL."""
+    guard = None
+    if isinstance(scratch, str):
+        kernels, _ = lib()
+        nbytes = int(kernels.mpReduceScratchBytes(KEY[src.dtype], m, n))
+        guard = Guarded((nbytes,), torch.uint8) if nbytes else None
+        scratch = guard.t if guard is not None else None
+    _call("reduce_ij_j_scratch", src.dtype, src.data_ptr(), dst.data_ptr(),
+          scratch.data_ptr() if scratch is not None else None, float(alpha), m, n)
+    if guard is not None:
+        torch.cuda.synchronize()
+        guard.check("reduce scratch")
+    return guard is not None
+
+
 def softmax_scratch(dtype, m, n):
     kernels, _ = lib()
     nbytes = int(kernels.mpSoftmaxScratchBytes(KEY[dtype], m, n))

@@ -271,6 +271,26 @@ def test_reduce_and_broadcast(dtype, shift):
                 dst.check(stem)
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_column_sums_with_workspace(dtype):
+    """Tall matrices: the rows are split into chunks whose partial rows a second kernel adds up."""
+    r = rng(16)
+    used = 0
+    for (m, n) in [(3, 2), (700, 8), (5000, 64), (4097, 1024), (20000, 40), (1500, 1027), (33, 64)]:
+        for alpha in (0.0, 1.0):
+            for scratch in ("auto", None):
+                G.say(f"reduce_ij_j_scratch dtype={dtype} shape=({m},{n}) alpha={alpha} scratch={scratch}")
+                src = G.dev(r.normal(0, 1, (m, n)), dtype)
+                dst = G.dev(r.normal(0, 1, n), dtype)
+                before = G.host(dst.t).copy()
+                used += bool(G.reduce_ij_j_scratch(src.t, dst.t, alpha, m, n, scratch))
+                ref = O.reduce_ij_j(G.host(src.t), before if alpha else None, alpha)
+                scale = np.abs(G.host(src.t).astype(np.float64)).sum(axis=0) + abs(alpha) * np.abs(before.astype(np.float64))
+                G.compare(dst.t, ref, dtype, f"reduce_ij_j_scratch ({m},{n}) alpha {alpha}", rowwise=False, scale=scale)
+                dst.check("column sums")
+    assert used > 0, "no shape took the two-stage path"
+
+
 def test_reference_example_reductions():
     # src/examples/experimental.zig:19-34
     f32 = torch.float32
