@@ -75,3 +75,26 @@ def test_config_rejects_non_gfx_architectures(tmp_path, monkeypatch):
     monkeypatch.setattr(kernelgen, "CONFIG", str(cfg))
     with pytest.raises(ValueError):
         kernelgen.load_config()
+
+
+def test_headers_compile_as_plain_c_and_link(tmp_path):
+    """The boundary is a C ABI: a C11 translation unit includes the three headers, takes the
+    address of a launcher and of a device utility, and links against the two libraries (nothing
+    is called: there is no GPU here)."""
+    import subprocess
+    src = tmp_path / "abi.c"
+    src.write_text(
+        '#include "tensor_types.h"\n#include "device_utils.h"\n#include "kernel_decls.h"\n'
+        "typedef void (*softmax_fn)(const void*, void*, void*, len_t, len_t, StreamContext);\n"
+        "typedef StreamContext (*init_fn)(void);\n"
+        "int main(void) {\n"
+        "  softmax_fn f = launch_softmax_ij_j_r32;\n"
+        "  init_fn g = mpInitStream;\n"
+        "  StreamContext c; c.hip_stream.ptr = 0; c.blas_handle.ptr = 0;\n"
+        "  return (f != 0 && g != 0 && sizeof c == 2 * sizeof(void*) && sizeof(r16) == 2) ? 0 : 1;\n"
+        "}\n")
+    exe = tmp_path / "abi"
+    cmd = ["gcc", "-std=c11", "-Wall", "-Werror", "-I", os.path.join(ROOT, "include"), str(src), "-o", str(exe),
+           "-L", ffi.LIB_DIR, "-lmp_kernels", "-ldev_utils", f"-Wl,-rpath,{ffi.LIB_DIR}", "-Wl,-rpath-link,/opt/rocm/lib"]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr
