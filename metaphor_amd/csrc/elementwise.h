@@ -36,12 +36,15 @@ __device__ __forceinline__ void ew_apply(const F& f, const P (&a)[NIN > 0 ? NIN 
 /* One wavefront per workgroup and one pack per stream per lane measured fastest on MI355X for
  * pure streaming (larger workgroups or deeper unrolling lose 3-8 % of HBM bandwidth). */
 constexpr int EW_BLOCK = 64;
+/* Kernels that only write (fill, sequence) want 256-thread workgroups: 4.6 -> 6.5 TB/s measured;
+ * everything that also reads is fastest with single-wave workgroups. */
+template <int NIN> constexpr int ew_block() { return NIN == 0 ? 256 : EW_BLOCK; }
 
 /* F::apply(const P (&in)[NIN], P (&out)[NOUT]) computes one element. */
 template <class T, int W, int NIN, int NOUT, int UNROLL, class F>
-__global__ __launch_bounds__(EW_BLOCK) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, size_t n, F f) {
+__global__ __launch_bounds__(ew_block<NIN>()) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, size_t n, F f) {
   using P = typename precision<T>::type;
-  constexpr int NA = NIN > 0 ? NIN : 1;
+  constexpr int NA = NIN > 0 ? NIN : 1, EW_BLOCK = ew_block<NIN>();
   const size_t npacks = n / W;
   const size_t base = (size_t)blockIdx.x * (EW_BLOCK * UNROLL) + threadIdx.x;
 
@@ -94,6 +97,7 @@ __global__ __launch_bounds__(EW_BLOCK) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, si
 template <class T, int NIN, int NOUT, int UNROLL, class F>
 inline void ew_launch(const EwPtrs<NIN, NOUT>& ptrs, size_t n, F f, hipStream_t stream) {
   if (n == 0) return;
+  constexpr int EW_BLOCK = ew_block<NIN>();
   require(n / EW_BLOCK < 0x7fffffffull, "elementwise launch: too many elements for one grid");
   bool packed = true;
   for (int s = 0; s < NIN; ++s) packed = packed && aligned16(ptrs.in[s]);
