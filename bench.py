@@ -120,6 +120,34 @@ def time_each(sets, iters):
     return [a.elapsed_time(b) for a, b in fwd], [a.elapsed_time(b) for a, b in rev]
 
 
+def graph_forward_ms(sets, replays=50):
+    """Per-launch time of the forward launcher when the launches of all buffer sets are captured
+    once into a HIP graph and replayed: what a launch-bound workload (cfg1: a 3 us kernel behind
+    ~10 us of host-side launch work) costs once the host is out of the loop. The last replay is
+    checked against the eager result."""
+    import torch
+    for s in sets:
+        s.forward()
+    torch.cuda.synchronize()
+    eager = [s.y.clone() for s in sets]
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        for s in sets:
+            s.forward()
+    for s in sets:
+        s.y.zero_()
+    a, b = _events(2)
+    graph.replay()
+    torch.cuda.synchronize()
+    a.record()
+    for _ in range(replays):
+        graph.replay()
+    b.record()
+    torch.cuda.synchronize()
+    same = all(torch.equal(s.y, e) for s, e in zip(sets, eager))
+    return a.elapsed_time(b) / (replays * len(sets)), same
+
+
 def rates(w, fwd_ms, rev_ms):
     out = {"fwd_ms": round(_median(fwd_ms), 5),
            "fwd_GBps": round(w.fwd_bytes / (_median(fwd_ms) * 1e-3) / 1e9, 1)}
@@ -229,6 +257,10 @@ def main():
                      "avg_launch_ms": round(avg_ms, 5), "launches_timed": len(dom_ms)},
         name: rates(w, fwd_ms, rev_ms),
     }
+    if name == "cfg1":
+        g_ms, same = graph_forward_ms(sets)
+        line[name].update({"fwd_graph_ms": round(g_ms, 5), "fwd_graph_matches_eager": same,
+                           "fwd_graph_GBps": round(w.fwd_bytes / (g_ms * 1e-3) / 1e9, 1)})
 
     if name in MFMA_PEAK_TFLOPS:  # the matrix product is priced in flops against the matrix cores
         tf = w.rev_flops / (avg_ms * 1e-3) / 1e12
@@ -251,6 +283,11 @@ def main():
             f_ms, r_ms = time_each(osets, k)
             extra[other] = rates(osets[0], f_ms, r_ms)
             extra[other]["workload"] = W.DESCRIPTION[other]
+            if other == "cfg1":  # launch-bound: also the rate with the host out of the loop
+                g_ms, same = graph_forward_ms(osets)
+                extra[other]["fwd_graph_ms"] = round(g_ms, 5)
+                extra[other]["fwd_graph_GBps"] = round(osets[0].fwd_bytes / (g_ms * 1e-3) / 1e9, 1)
+                extra[other]["fwd_graph_matches_eager"] = same
             del osets
             torch.cuda.empty_cache()
         line["other_workloads"] = extra

@@ -1,0 +1,61 @@
+"""The launchers under HIP graph capture: they enqueue kernels only (no allocation, no memset
+nodes: the shared-row softmax clears its slots with a fill kernel), so a captured sequence can be
+replayed. Every replay is checked against the eager result, with eager work and synchronisation
+between replays."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_lib as G
+from metaphor_amd import workloads as W
+
+pytestmark = pytest.mark.gpu
+
+
+def test_replays_of_a_captured_forward_and_reverse_sequence_match_eager():
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(7)
+    f32 = torch.float32
+    m, n = 64, 4096
+    x = torch.randn(m, n, generator=gen, device="cuda")
+    gain = 1 + 0.02 * torch.randn(n, generator=gen, device="cuda")
+    dy = torch.randn(m, n, generator=gen, device="cuda")
+    y, dx, dg = torch.empty_like(x), torch.empty_like(x), torch.empty_like(gain)
+    nscratch = W.rmsnorm_reverse_scratch(f32, m, n)
+    # long rows: the shared-row softmax kernels with their slot-clearing kernel inside the graph
+    lm, ln = 8, 50257
+    logits = 3 * torch.randn(lm, ln, generator=gen, device="cuda")
+    p, dp, dl = torch.empty_like(logits), torch.randn(lm, ln, generator=gen, device="cuda"), torch.empty_like(logits)
+    fs, rs = W.softmax_scratch(f32, lm, ln), W.softmax_reverse_scratch(f32, lm, ln)
+    assert fs is not None and rs is not None
+    a, b, c, d = (torch.rand(10007, generator=gen, device="cuda") * 4 - 2 for _ in range(4))
+    e = torch.empty_like(a)
+
+    def sequence():
+        W.rmsnorm_forward(x, gain, y, 1e-6)
+        W.rmsnorm_reverse(x, gain, dy, dx, dg, nscratch, 1e-6)
+        W.softmax_forward(logits, p, fs)
+        W.softmax_reverse(p, dp, dl, 0.0, rs)
+        W.fused_forward(a, b, c, d, e)
+
+    outputs = (y, dx, dg, p, dl, e)
+    G.say("eager sequence")
+    sequence()
+    torch.cuda.synchronize()
+    eager = [t.clone() for t in outputs]
+    graph = torch.cuda.CUDAGraph()
+    G.say("capture")
+    with torch.cuda.graph(graph):
+        sequence()
+    for replay in range(4):
+        for t in outputs:
+            t.fill_(float("nan"))
+        torch.cuda.synchronize()
+        G.say(f"replay {replay}")
+        graph.replay()
+        torch.cuda.synchronize()
+        for got, ref in zip(outputs, eager):
+            assert torch.equal(got, ref), f"replay {replay} differs from the eager result"
+        # eager work of the program between replays
+        W.softmax_forward(logits, p, fs)
+        torch.cuda.synchronize()
