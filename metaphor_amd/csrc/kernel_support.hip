@@ -30,6 +30,16 @@ extern "C" len_t mpSoftmaxScratchBytes(len_t dtype, len_t m, len_t n) {
   }
 }
 
+// The same for launch_rmsnorm_ij_j_<dtype>: one word per workgroup of a shared row.
+extern "C" len_t mpRmsnormScratchBytes(len_t dtype, len_t m, len_t n) {
+  switch (dtype) {
+    case MP_R16: return mp::rmsnorm_scratch_bytes<r16>(m, n);
+    case MP_R32: return mp::rmsnorm_scratch_bytes<r32>(m, n);
+    case MP_R64: return mp::rmsnorm_scratch_bytes<r64>(m, n);
+    default: mp::require(false, "mpRmsnormScratchBytes: dtype must be 0, 1 or 2"); return 0;
+  }
+}
+
 // The same for launch_softmax_ij_j_reverse_<dtype>: one word per workgroup of a shared row.
 extern "C" len_t mpSoftmaxReverseScratchBytes(len_t dtype, len_t m, len_t n) {
   switch (dtype) {

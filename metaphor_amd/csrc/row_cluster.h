@@ -1,0 +1,100 @@
+/*
+ * What the kernels that share one long row between several workgroups have in common: the
+ * scratch words the workgroups of a row publish their partial results in, the bounded wait for
+ * the partners, the small kernel that clears the words before a launch, and the tuning knobs of
+ * the tests. Used by the softmax and RMSNorm launchers; no counterpart in the reference, whose
+ * row kernels give a row to one 32-lane warp (src/cuda/nvcc_src/reduce_ij_i.cu:3-33).
+ */
+#ifndef MP_ROW_CLUSTER_H
+#define MP_ROW_CLUSTER_H
+
+#include "row_dispatch.h"
+
+#if defined(__cplusplus) && defined(__HIPCC__)
+
+namespace mp {
+
+/* workgroup size of the shared-row kernels, and the most workgroups one row is split over (one
+ * lane of the first wavefront polls each partner) */
+constexpr int CLUSTER_THREADS = 1024, CLUSTER_MAX = WAVE;
+
+/* Makes the compiler forget what it knows about a register-held pack, so that widened copies
+ * of a whole chunk are not kept alive from one phase of a kernel to the next. */
+template <class V> __device__ __forceinline__ void forget(V& v) {
+  typedef unsigned words_t __attribute__((ext_vector_type(sizeof(V) / 4)));
+  words_t w = __builtin_bit_cast(words_t, v);
+  asm volatile("" : "+v"(w));
+  v = __builtin_bit_cast(V, w);
+}
+
+template <class P> struct slot_word { using type = unsigned; };
+template <> struct slot_word<double> { using type = unsigned long long; };
+
+template <class Word> __global__ __launch_bounds__(256) void cluster_zero_slots(Word* slots, size_t words) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < words) slots[i] = 0;
+}
+
+/* Diagnostic knobs of the cluster path (set through mpSetClusterTuning). */
+struct ClusterTuning {
+  int packs_per_block = 0; /* 0: one pack per thread less than the register tile holds */
+  unsigned spin_limit = 1u << 22;
+};
+inline ClusterTuning& cluster_tuning() {
+  static ClusterTuning t;
+  return t;
+}
+
+/* Sums over the C workgroups that share a row. Every workgroup calls this with its NVAL partial
+ * sums; all threads return with the row totals in vals, and the result says whether every
+ * partner was heard from. `mine` points at this row's C * NVAL scratch words, zero before the
+ * kernel started; a published word is never zero (+0 is stored as -0), so non-zero means
+ * published. Workgroups of a row publish before they wait, and the wait ends after spin_limit
+ * polls whatever happens: a caller that gets `false` computes the totals some other way (it
+ * re-reads the row), so every wave reaches the end of its kernel under any scheduling.
+ * bc: NVAL + 1 words of LDS. Contains one barrier; all CLUSTER_THREADS threads must call it. */
+template <int NVAL, class P>
+__device__ __forceinline__ bool cluster_exchange_sums(typename slot_word<P>::type* mine, int C, int rank,
+                                                      P (&vals)[NVAL], unsigned spin_limit, P* bc, int lane) {
+  using Word = typename slot_word<P>::type;
+  if (lane == 0) {
+#pragma unroll
+    for (int v = 0; v < NVAL; ++v) {
+      const P part = vals[v] == (P)0 ? -(P)0 : vals[v];
+      __hip_atomic_store(mine + (size_t)rank * NVAL + v, __builtin_bit_cast(Word, part), __ATOMIC_RELAXED,
+                         __HIP_MEMORY_SCOPE_AGENT);
+    }
+  }
+  if (lane < WAVE) { /* wave 0: lane r waits for workgroup r of this row */
+    Word w[NVAL];
+    bool heard = true;
+    if (lane < C) {
+      for (unsigned spins = 0;; ++spins) {
+        heard = true;
+#pragma unroll
+        for (int v = 0; v < NVAL; ++v) {
+          w[v] = __hip_atomic_load(mine + (size_t)lane * NVAL + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          heard = heard && w[v] != 0;
+        }
+        if (heard || spins >= spin_limit) break;
+        __builtin_amdgcn_s_sleep(4);
+      }
+    }
+    const P missing = wave_allreduce<AddOP>(heard ? (P)0 : (P)1); /* every lane takes part */
+#pragma unroll
+    for (int v = 0; v < NVAL; ++v) {
+      const P total = wave_allreduce<AddOP>(lane < C && heard ? __builtin_bit_cast(P, w[v]) : (P)0);
+      if (lane == 0) bc[v] = total;
+    }
+    if (lane == 0) bc[NVAL] = missing;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int v = 0; v < NVAL; ++v) vals[v] = bc[v];
+  return bc[NVAL] == (P)0;
+}
+
+}  // namespace mp
+
+#endif
+#endif

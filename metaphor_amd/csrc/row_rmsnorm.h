@@ -18,7 +18,7 @@
 #ifndef MP_ROW_RMSNORM_H
 #define MP_ROW_RMSNORM_H
 
-#include "row_dispatch.h"
+#include "row_cluster.h"
 
 #if defined(__cplusplus) && defined(__HIPCC__)
 
@@ -163,6 +163,126 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_fwd_stream(
     }
     if (W > 1 && edge != (size_t)-1) yr[edge] = (T)((P)xr[edge] * r * (P)gain[edge]);
   }
+}
+
+/* ------------------------------------------------------------------ shared-row forward */
+
+/* Rows too long for one workgroup's registers: C consecutive workgroups share a row. Each keeps
+ * its chunk of x in registers in the storage type, publishes its part of sum x^2, waits (bounded)
+ * for the others and writes its chunk of y: the row is read once. A workgroup that stops
+ * waiting reads the whole row again for the sum, which is why the path is not taken in place. */
+constexpr int NORM_CLUSTER_NV = 5; /* packs per thread: 20 registers, two workgroups a CU */
+
+template <class T, int W>
+__global__ __launch_bounds__(CLUSTER_THREADS, 8) void rmsnorm_fwd_cluster(
+    const T* x, const T* gain, T* y, typename precision<T>::type eps,
+    typename slot_word<typename precision<T>::type>::type* slots,
+    size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
+  using P = typename precision<T>::type;
+  using V = typename vec_of<T, W>::type;
+  constexpr int G = CLUSTER_THREADS, NV = NORM_CLUSTER_NV;
+  __shared__ P red[2][G / WAVE];
+  __shared__ P bc[2];
+  const int lane = threadIdx.x;
+  const size_t row = blockIdx.x / (unsigned)C;
+  const int rank = (int)(blockIdx.x % (unsigned)C);
+  const T* xr = x + row * n;
+  T* yr = y + row * n;
+  const RowGeom<T, W> g(xr, n, true);
+  const T* body = xr + g.head;
+  const int lo = rank * packs_per_block;
+  const int hi = lo + packs_per_block < g.nvec ? lo + packs_per_block : g.nvec;
+
+  V v[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = lo + k * G + lane;
+    if (p < hi) {
+      v[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(body + (size_t)p * W));
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[k][i] = (T)0;
+    }
+  }
+  P edge = (P)0; /* rank 0 also holds the row's head / tail scalars */
+  size_t edge_at = (size_t)-1;
+  if (W > 1 && rank == 0) {
+    if (lane < g.head) edge_at = (size_t)lane;
+    else if (lane - g.head < g.tail) edge_at = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
+    if (edge_at != (size_t)-1) edge = (P)xr[edge_at];
+  }
+
+  P ss = edge * edge;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) ss += (P)v[k][i] * (P)v[k][i];
+  ss = group_allreduce<AddOP, G>(ss, red[0], lane);
+#pragma unroll
+  for (int k = 0; k < NV; ++k) forget(v[k]);
+
+  if (C > 1) {
+    P sums[1] = {ss};
+    const bool complete = cluster_exchange_sums<1>(slots + (size_t)row * C, C, rank, sums, spin_limit, bc, lane);
+    ss = sums[0];
+    if (!complete) { /* gave up waiting: the whole row's sum here */
+      P t = (P)0;
+      for (int p = lane; p < g.nvec; p += G) {
+        P u[W];
+        load_pack<T, W>(body + (size_t)p * W, u);
+#pragma unroll
+        for (int i = 0; i < W; ++i) t += u[i] * u[i];
+      }
+      if (W > 1) {
+        size_t e = (size_t)-1;
+        if (lane < g.head) e = (size_t)lane;
+        else if (lane - g.head < g.tail) e = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
+        if (e != (size_t)-1) t += (P)xr[e] * (P)xr[e];
+      }
+      ss = group_allreduce<AddOP, G>(t, red[1], lane);
+    }
+  }
+
+  const P r = rsqrt_of(ss / (P)n + eps);
+  T* ybody = yr + g.head;
+  const T* gbody = gain + g.head;
+  const bool gain_packed = (reinterpret_cast<uintptr_t>(gbody) & 15u) == 0;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = lo + k * G + lane;
+    if (p < hi) {
+      P gv[W], out[W];
+      if (gain_packed) {
+        load_pack<T, W>(gbody + (size_t)p * W, gv);
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) gv[i] = (P)gbody[(size_t)p * W + i];
+      }
+#pragma unroll
+      for (int i = 0; i < W; ++i) out[i] = (P)v[k][i] * r * gv[i];
+      store_pack_nt<T, W>(ybody + (size_t)p * W, out);
+    }
+  }
+  if (edge_at != (size_t)-1) yr[edge_at] = (T)(edge * r * (P)gain[edge_at]);
+}
+
+/* Workgroups per row when the forward shares rows; 0 when it does not. */
+template <class T> inline int rmsnorm_cluster_size(size_t packs) {
+  const int regime = row_regime_override();
+  if (regime != REGIME_AUTO && regime != REGIME_CLUSTER) return 0;
+  constexpr size_t resident = (size_t)NORM_BLOCK * max_nv_for<T>(32); /* what one workgroup holds */
+  if (regime == REGIME_AUTO && packs <= resident) return 0;
+  constexpr size_t tile = (size_t)CLUSTER_THREADS * NORM_CLUSTER_NV;
+  size_t ppb = (size_t)cluster_tuning().packs_per_block;
+  if (ppb == 0 || ppb > tile) ppb = tile;
+  const size_t c = (packs + ppb - 1) / ppb;
+  return c >= 1 && c <= (size_t)CLUSTER_MAX ? (int)c : 0;
+}
+
+template <class T> inline size_t rmsnorm_scratch_bytes(size_t m, size_t n) {
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  const int c = rmsnorm_cluster_size<T>((n + W - 1) / W);
+  return c > 1 ? m * (size_t)c * sizeof(typename precision<T>::type) : 0;
 }
 
 /* ------------------------------------------------------------------ resident reverse */
@@ -463,7 +583,7 @@ inline size_t rmsnorm_reverse_scratch_bytes(size_t m, size_t n) {
 }
 
 template <class T>
-inline void rmsnorm_forward(const T* x, const T* gain, T* y, double eps, size_t m, size_t n,
+inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, double eps, size_t m, size_t n,
                             hipStream_t stream) {
   if (m == 0 || n == 0) return;
   using P = typename precision<T>::type;
@@ -478,6 +598,24 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, double eps, size_t 
   }
   const bool ragged = !(aligned16(x) && aligned16(gain) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
+  {
+    const int C = rmsnorm_cluster_size<T>((n + W - 1) / W);
+    const bool shareable = scratch != nullptr && static_cast<const void*>(x) != static_cast<const void*>(y);
+    if (C >= 1 && (C == 1 || shareable) && m * (size_t)C < 0x7fffffffull) {
+      using Word = typename slot_word<P>::type;
+      Word* slots = static_cast<Word*>(scratch);
+      const int ppb = (int)(((n + W - 1) / W + C - 1) / C);
+      require(ppb <= CLUSTER_THREADS * NORM_CLUSTER_NV, "rmsnorm: cluster chunk exceeds the register tile");
+      if (C > 1) {
+        const size_t words = m * (size_t)C;
+        cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
+      }
+      rmsnorm_fwd_cluster<T, W><<<dim3((unsigned)(m * C)), dim3(CLUSTER_THREADS), 0, stream>>>(
+          x, gain, y, (P)eps, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+      MP_CHECK_LAUNCH();
+      return;
+    }
+  }
   const size_t packs = (n + W - 1) / W;
   /* Short rows: one-shot 256-thread workgroups (each loads the gain it needs, which stays in L2)
    * beat persistent 1024-thread ones: r32 n = 256: 5.5 -> 6.3 TB/s, n = 1024: 6.0 -> 6.4; r16 wants

@@ -20,7 +20,7 @@
 #ifndef MP_ROW_SOFTMAX_H
 #define MP_ROW_SOFTMAX_H
 
-#include "row_dispatch.h"
+#include "row_cluster.h"
 #include <type_traits>
 
 #if defined(__cplusplus) && defined(__HIPCC__)
@@ -245,7 +245,6 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
  * before it waits, so with in-order dispatch the wait is short; if spin_limit polls pass
  * anyway, the workgroup stops waiting and folds the whole row itself (one extra read of the row),
  * so every wave reaches the end whatever the scheduling. */
-constexpr int CLUSTER_THREADS = 1024, CLUSTER_MAX = WAVE;
 /* packs per thread: 24 registers of row data, so that two workgroups fit a CU (64 registers) */
 template <class T> constexpr int cluster_nv() {
   /* r16 chunks stay in their storage type (four registers a pack) and are widened where they are
@@ -253,18 +252,6 @@ template <class T> constexpr int cluster_nv() {
   if (sizeof(T) == 2) return 24 / 4;
   return 24 / ((PACK_BYTES / (int)sizeof(T)) * (int)(sizeof(typename precision<T>::type) / 4));
 }
-
-/* Makes the compiler forget what it knows about a register-held pack, so that widened copies
- * of a whole chunk are not kept alive from one phase of a kernel to the next. */
-template <class V> __device__ __forceinline__ void forget(V& v) {
-  typedef unsigned words_t __attribute__((ext_vector_type(sizeof(V) / 4)));
-  words_t w = __builtin_bit_cast(words_t, v);
-  asm volatile("" : "+v"(w));
-  v = __builtin_bit_cast(V, w);
-}
-
-template <class P> struct slot_word { using type = unsigned; };
-template <> struct slot_word<double> { using type = unsigned long long; };
 
 template <class T, int W>
 __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
@@ -421,21 +408,6 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
     }
     if (edge_at != (size_t)-1) yr[edge_at] = (T)(edge * scale);
   }
-}
-
-template <class Word> __global__ __launch_bounds__(256) void cluster_zero_slots(Word* slots, size_t words) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i < words) slots[i] = 0;
-}
-
-/* Diagnostic knobs of the cluster path (set through mpSetClusterTuning). */
-struct ClusterTuning {
-  int packs_per_block = 0; /* 0: one pack per thread less than the register tile holds */
-  unsigned spin_limit = 1u << 22;
-};
-inline ClusterTuning& cluster_tuning() {
-  static ClusterTuning t;
-  return t;
 }
 
 /* Workgroups per row on the cluster path; 0 when the row does not take it. */
@@ -618,31 +590,10 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_rev_cluster(
   dot = group_allreduce<AddOP, G>(dot, red[0], lane);
 
   if (C > 1) {
-    if (lane == 0) {
-      const P part = dot == (P)0 ? -(P)0 : dot;
-      __hip_atomic_store(slots + (size_t)row * C + rank, __builtin_bit_cast(Word, part), __ATOMIC_RELAXED,
-                         __HIP_MEMORY_SCOPE_AGENT);
-    }
-    if (lane < WAVE) { /* wave 0: lane r waits for workgroup r of this row */
-      Word w = 1;
-      if (lane < C) {
-        Word* theirs = slots + (size_t)row * C + lane;
-        for (unsigned spins = 0;; ++spins) {
-          w = __hip_atomic_load(theirs, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if (w != 0 || spins >= spin_limit) break;
-          __builtin_amdgcn_s_sleep(4);
-        }
-      }
-      const P missing = wave_allreduce<AddOP>(w != 0 ? (P)0 : (P)1); /* every lane takes part */
-      const P total = wave_allreduce<AddOP>(lane < C && w != 0 ? __builtin_bit_cast(P, w) : (P)0);
-      if (lane == 0) {
-        bc[0] = total;
-        bc[1] = missing;
-      }
-    }
-    __syncthreads();
-    dot = bc[0];
-    if (bc[1] != (P)0) { /* gave up waiting: the whole row's dot product here */
+    P sums[1] = {dot};
+    const bool complete = cluster_exchange_sums<1>(slots + (size_t)row * C, C, rank, sums, spin_limit, bc, lane);
+    dot = sums[0];
+    if (!complete) { /* gave up waiting: the whole row's dot product here */
       P d = (P)0;
       for (int p = lane; p < g.nvec; p += G) {
         P u[W], v[W];

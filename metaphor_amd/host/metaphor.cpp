@@ -702,7 +702,9 @@ Tensor rmsnorm(Tensor x, Tensor gain, double eps) {
   void* pg = gain.data_ptr();
   Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
   const size_t n = x.sizes().back(), m = x.len() / n;
-  kernels::rmsnorm_ij_j(dkey(z), px, pg, z.data_ptr(), eps, (len_t)m, (len_t)n, z.context());
+  const len_t bytes = mpRmsnormScratchBytes((len_t)dkey(z), (len_t)m, (len_t)n);
+  void* scratch = bytes ? z.stream()->get_scratch(bytes) : nullptr;
+  kernels::rmsnorm_ij_j(dkey(z), px, pg, z.data_ptr(), scratch, eps, (len_t)m, (len_t)n, z.context());
   g->launches++;
   if (g->mode == Mode::train) attach_op(z, rmsnorm_reverse, {x, gain, eps, z});
   return z;

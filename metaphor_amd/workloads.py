@@ -47,6 +47,19 @@ def blas_ctx():
 
 # ------------------------------------------------------------------ launch wrappers
 
+def _workspace(scratch, size_fn, dtype, m, n, what):
+    """Pointer of a caller-owned workspace after checking that it is large enough for THIS dtype
+    and shape: a workspace sized for another dtype would be overrun on the GPU."""
+    if scratch is None:
+        return None
+    kernels, _ = ffi.load()
+    need = int(getattr(kernels, size_fn)(KEY[dtype], m, n))
+    have = scratch.numel() * scratch.element_size()
+    if have < need:
+        raise ValueError(f"{what}: workspace of {have} bytes, {need} needed for {DTYPE_NAME[dtype]} [{m},{n}]")
+    return scratch.data_ptr()
+
+
 def permutate(src, dst, alpha=0.0):
     rows, cols = src.shape
     _launch("permutate_ij_ji", src.dtype, src.data_ptr(), dst.data_ptr(), float(alpha), rows, cols)
@@ -69,7 +82,7 @@ def softmax_scratch(dtype, m, n):
 def softmax_forward(x, y, scratch=None):
     m, n = x.shape
     _launch("softmax_ij_j", x.dtype, x.data_ptr(), y.data_ptr(),
-            scratch.data_ptr() if scratch is not None else None, m, n)
+            _workspace(scratch, "mpSoftmaxScratchBytes", x.dtype, m, n, "softmax_forward"), m, n)
 
 
 def softmax_reverse_scratch(dtype, m, n):
@@ -82,12 +95,20 @@ def softmax_reverse_scratch(dtype, m, n):
 def softmax_reverse(y, dy, dx, alpha=0.0, scratch=None):
     m, n = y.shape
     _launch("softmax_ij_j_reverse", y.dtype, y.data_ptr(), dy.data_ptr(), dx.data_ptr(),
-            scratch.data_ptr() if scratch is not None else None, float(alpha), m, n)
+            _workspace(scratch, "mpSoftmaxReverseScratchBytes", y.dtype, m, n, "softmax_reverse"), float(alpha), m, n)
 
 
-def rmsnorm_forward(x, gain, y, eps):
+def rmsnorm_scratch(dtype, m, n):
+    """Workspace for launch_rmsnorm_ij_j (None when the rows fit one workgroup)."""
+    kernels, _ = ffi.load()
+    nbytes = int(kernels.mpRmsnormScratchBytes(KEY[dtype], m, n))
+    return torch.empty(nbytes, dtype=torch.uint8, device="cuda") if nbytes else None
+
+
+def rmsnorm_forward(x, gain, y, eps, scratch=None):
     m, n = x.shape
-    _launch("rmsnorm_ij_j", x.dtype, x.data_ptr(), gain.data_ptr(), y.data_ptr(), float(eps), m, n)
+    _launch("rmsnorm_ij_j", x.dtype, x.data_ptr(), gain.data_ptr(), y.data_ptr(),
+            _workspace(scratch, "mpRmsnormScratchBytes", x.dtype, m, n, "rmsnorm_forward"), float(eps), m, n)
 
 
 def rmsnorm_reverse_scratch(dtype, m, n):
@@ -99,7 +120,8 @@ def rmsnorm_reverse_scratch(dtype, m, n):
 def rmsnorm_reverse(x, gain, dy, dx, dgain, scratch, eps, alpha=0.0):
     m, n = x.shape
     _launch("rmsnorm_ij_j_reverse", x.dtype, x.data_ptr(), gain.data_ptr(), dy.data_ptr(), dx.data_ptr(),
-            dgain.data_ptr(), scratch.data_ptr(), float(eps), float(alpha), m, n)
+            dgain.data_ptr(), _workspace(scratch, "mpRmsnormReverseScratchBytes", x.dtype, m, n, "rmsnorm_reverse"),
+            float(eps), float(alpha), m, n)
 
 
 def fused_forward(a, b, c, d, e):

@@ -254,9 +254,20 @@ def softmax_reverse(y, dy, dx, alpha=0.0, scratch="auto"):
         guard.check("softmax reverse scratch")
 
 
-def rmsnorm(x, g, y, eps):
+def rmsnorm(x, g, y, eps, scratch="auto"):
+    """scratch: "auto" sizes and passes the workspace the launcher asks for, None passes NULL."""
     m, n = x.shape
-    _call("rmsnorm_ij_j", x.dtype, x.data_ptr(), g.data_ptr(), y.data_ptr(), float(eps), m, n)
+    guard = None
+    if isinstance(scratch, str):
+        kernels, _ = lib()
+        nbytes = int(kernels.mpRmsnormScratchBytes(KEY[x.dtype], m, n))
+        guard = Guarded((nbytes,), torch.uint8) if nbytes else None
+        scratch = guard.t if guard is not None else None
+    _call("rmsnorm_ij_j", x.dtype, x.data_ptr(), g.data_ptr(), y.data_ptr(),
+          scratch.data_ptr() if scratch is not None else None, float(eps), m, n)
+    if guard is not None:
+        torch.cuda.synchronize()
+        guard.check("rmsnorm scratch")
 
 
 def rmsnorm_scratch(dtype, m, n):

@@ -549,6 +549,46 @@ def test_rmsnorm_forward_unaligned_and_in_place(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("packs,spin", [(0, 1 << 22), (64, 1 << 22), (3, 1 << 22), (64, 0), (1000, 2)],
+                         ids=["default", "64packs", "3packs", "64packs-nowait", "1000packs-2polls"])
+def test_rmsnorm_forward_cluster_path(dtype, packs, spin):
+    """Several workgroups per row exchanging their parts of sum x^2 through scratch; with a poll
+    limit of 0 or 2 most workgroups give up waiting and read the whole row themselves."""
+    r = rng(52)
+    G.set_regime(CLUSTER)
+    G.set_cluster_tuning(packs, spin)
+    eps = 1e-6
+    for (m, n) in [(3, 7), (5, 64), (4, 1000), (6, 2048), (33, 5000), (2, 50257), (2, 151936), (130, 777)]:
+        for shift in (0, 1):
+            G.say(f"rmsnorm cluster dtype={dtype} packs={packs} spin={spin} shape=({m},{n}) shift={shift}")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            g = G.dev(r.normal(1, 0.02, n), dtype, shift)
+            y = G.Guarded((m, n), dtype, shift)
+            G.rmsnorm(x.t, g.t, y.t, eps)
+            G.compare(y.t, O.rmsnorm_ij_j(G.host(x.t), G.host(g.t), eps), dtype,
+                      f"rmsnorm cluster ({m},{n}) packs {packs} spin {spin}")
+            for b in (x, g, y):
+                b.check("rmsnorm cluster")
+
+
+def test_rmsnorm_long_rows_in_place_and_without_scratch():
+    r = rng(53)
+    f32 = torch.float32
+    for (m, n) in [(3, 151936), (4, 50257)]:
+        x = G.dev(r.normal(0, 1, (m, n)), f32)
+        g = G.dev(r.normal(1, 0.02, n), f32)
+        ref = O.rmsnorm_ij_j(G.host(x.t), G.host(g.t), 1e-6)
+        y = G.Guarded((m, n), f32)
+        G.say(f"rmsnorm NULL scratch ({m},{n})")
+        G.rmsnorm(x.t, g.t, y.t, 1e-6, scratch=None)
+        G.compare(y.t, ref, f32, f"rmsnorm no scratch ({m},{n})")
+        G.say(f"rmsnorm long rows in place ({m},{n})")
+        G.rmsnorm(x.t, g.t, x.t, 1e-6)
+        G.compare(x.t, ref, f32, f"rmsnorm in place ({m},{n})")
+        x.check("in place")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 @pytest.mark.parametrize("regime", REGIMES)
 def test_rmsnorm_reverse_all_regimes(dtype, regime):
     r = rng(60 + regime)
