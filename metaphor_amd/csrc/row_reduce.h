@@ -176,9 +176,10 @@ inline void reduce_cols(const T* src, T* dst, void* scratch, double alpha, size_
     }
     reduce_cols_kernel<T, T, W, 8, 128><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n, m);
   } else {
-    const size_t blocks = (n + 31) / 32;
+    /* rows that are not pack-aligned: one element per lane, a wavefront per 64-element row segment */
+    const size_t blocks = (n + 63) / 64;
     require(blocks < 0x7fffffffull, "reduce_ij_j: too many columns for one grid");
-    reduce_cols_kernel<T, T, 1, 32, 32><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n, m);
+    reduce_cols_kernel<T, T, 1, 64, 16><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n, m);
   }
   MP_CHECK_LAUNCH();
 }
