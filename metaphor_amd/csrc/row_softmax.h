@@ -414,10 +414,14 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
 template <class T> inline int cluster_size(size_t packs) {
   const int regime = row_regime_override();
   if (regime != REGIME_AUTO && regime != REGIME_CLUSTER) return 0;
-  if (regime == REGIME_AUTO && packs <= (size_t)CLUSTER_THREADS * 2) return 0; /* one workgroup, two packs each */
+  /* up to two packs per thread a resident workgroup is the better kernel; measured exceptions: r32
+   * rows of exactly 2048 packs (n = 8192: 5.8 resident, 6.1 here), and r16 chunks want the whole
+   * register tile (n = 49152: 5.4 -> 5.7 TB/s) where r32 is better one pack per thread below it */
+  const size_t resident = (size_t)CLUSTER_THREADS * 2 - (sizeof(T) >= 4 ? 1 : 0);
+  if (regime == REGIME_AUTO && packs <= resident) return 0;
   constexpr size_t tile = (size_t)CLUSTER_THREADS * cluster_nv<T>();
   size_t ppb = (size_t)cluster_tuning().packs_per_block;
-  if (ppb == 0) ppb = tile - CLUSTER_THREADS;
+  if (ppb == 0) ppb = sizeof(T) == 2 ? tile : tile - CLUSTER_THREADS;
   if (ppb > tile) ppb = tile;
   const size_t c = (packs + ppb - 1) / ppb;
   return c >= 1 && c <= (size_t)CLUSTER_MAX ? (int)c : 0;
