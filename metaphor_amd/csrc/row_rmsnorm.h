@@ -504,6 +504,160 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
   }
 }
 
+/* ------------------------------------------------------------------ shared-row reverse */
+
+/* Rows too long for one workgroup's registers, pack-aligned: the grid is S slices of C
+ * consecutive workgroups. The C workgroups of a slice share every row of the slice
+ * (rows slice, slice + S, ...): each keeps the dg sums of its chunk in registers for the whole
+ * kernel and, per row, its chunk of x, dy and (from L2) the gain; the two row sums (x^2 and dy*g*x) are
+ * exchanged through scratch once per row, so x and dy are read once. All S * C workgroups fit the
+ * GPU at once (one per CU: the kernel may use 128 registers a thread), which keeps the per-row waits short; a workgroup that stops waiting
+ * reads the whole row for the sums, so the kernel ends under any scheduling. Not taken when dx
+ * overwrites x or dy. One partial row of dg per slice. */
+/* packs of x, dy (and, per row, gain) per thread, in the storage type; the dg sums beside them are
+ * wider for r16 (eight fp32 a pack), which leaves room for two */
+template <class T> constexpr int norm_rev_cluster_nv() { return sizeof(T) == 2 ? 2 : 4; }
+
+template <class T, int W, bool BLEND>
+__global__ __launch_bounds__(CLUSTER_THREADS, 4) void rmsnorm_rev_cluster(
+    const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
+    typename precision<T>::type eps, typename precision<T>::type alpha,
+    typename slot_word<typename precision<T>::type>::type* slots,
+    size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
+  using P = typename precision<T>::type;
+  using V = typename vec_of<T, W>::type;
+  constexpr int G = CLUSTER_THREADS, NV = norm_rev_cluster_nv<T>();
+  __shared__ P red[2][2][G / WAVE];
+  __shared__ P bc[3];
+  const int lane = threadIdx.x;
+  const int rank = (int)(blockIdx.x % (unsigned)C);
+  const size_t slice = blockIdx.x / (unsigned)C, S = gridDim.x / (unsigned)C;
+  const int nvec = (int)(n / W);
+  const int lo = rank * packs_per_block;
+  const int hi = lo + packs_per_block < nvec ? lo + packs_per_block : nvec;
+
+  P acc[NV][W];
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) acc[k][i] = (P)0;
+
+  /* A partner that is not running yet (the GPU shared with other work) is waited for once: after
+   * the first wait that runs out, this workgroup stops waiting for the rest of the kernel (it
+   * still publishes its sums first, so its partners are never held up by it). */
+  unsigned patience = spin_limit;
+  int parity = 0;
+  for (size_t row = slice; row < m; row += S, parity ^= 1) {
+    const size_t off = row * n;
+    V xv[NV], dv[NV], gv[NV]; /* the gain chunk comes from L2 every row: registers go to the dg sums */
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * G + lane;
+      if (p < hi) {
+        xv[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(x + off + (size_t)p * W));
+        dv[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(dy + off + (size_t)p * W));
+        gv[k] = *reinterpret_cast<const V*>(gain + (size_t)p * W);
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) xv[k][i] = dv[k][i] = gv[k][i] = (T)0;
+      }
+    }
+    P ss = (P)0, c = (P)0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        const P xf = (P)xv[k][i];
+        ss += xf * xf;
+        c += (P)dv[k][i] * (P)gv[k][i] * xf;
+      }
+    group_allreduce_sum2<G>(ss, c, red[parity][0], red[parity][1], lane);
+    /* the chunk stays in the storage type: widened copies must not live across the exchange,
+     * nor a widened gain across the loop */
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      forget(xv[k]);
+      forget(dv[k]);
+      forget(gv[k]);
+    }
+
+    if (C > 1) {
+      P sums[2] = {ss, c};
+      const bool complete = cluster_exchange_sums<2>(slots + row * (size_t)C * 2, C, rank, sums, patience, bc, lane);
+      ss = sums[0];
+      c = sums[1];
+      if (!complete) { /* gave up waiting: both sums over the whole row here, and no waiting for later rows */
+        patience = 0;
+        P s2 = (P)0, c2 = (P)0;
+        for (int p = lane; p < nvec; p += G) {
+          P u[W], d[W], g[W];
+          load_pack<T, W>(x + off + (size_t)p * W, u);
+          load_pack<T, W>(dy + off + (size_t)p * W, d);
+          load_pack<T, W>(gain + (size_t)p * W, g);
+#pragma unroll
+          for (int i = 0; i < W; ++i) {
+            s2 += u[i] * u[i];
+            c2 += d[i] * g[i] * u[i];
+          }
+        }
+        /* the barrier inside the exchange lies between the last read of red[parity] and this reuse */
+        group_allreduce_sum2<G>(s2, c2, red[parity][0], red[parity][1], lane);
+        ss = s2;
+        c = c2;
+      }
+    }
+    const P r = rsqrt_of(ss / (P)n + eps);
+    const P cc = c / (P)n * r * r;
+
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * G + lane;
+      if (p < hi) {
+        P out[W];
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+          const P xf = (P)xv[k][i], df = (P)dv[k][i];
+          out[i] = r * (df * (P)gv[k][i] - xf * cc);
+          acc[k][i] += df * xf * r;
+        }
+        if constexpr (BLEND) {
+          P old[W];
+          load_pack<T, W>(dx + off + (size_t)p * W, old);
+#pragma unroll
+          for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+        }
+        store_pack_nt<T, W>(dx + off + (size_t)p * W, out);
+      }
+    }
+  }
+
+  P* mine = partials + slice * n;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = lo + k * G + lane;
+    if (p < hi) {
+#pragma unroll
+      for (int i = 0; i < W; ++i) mine[(size_t)p * W + i] = acc[k][i];
+    }
+  }
+}
+
+/* Workgroups per row when the reverse shares rows (pack-aligned operands only); 0 when not. */
+template <class T> inline int rmsnorm_rev_cluster_size(size_t n) {
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  if (n % W != 0) return 0;
+  const size_t packs = n / W;
+  const int regime = row_regime_override();
+  if (regime != REGIME_AUTO && regime != REGIME_CLUSTER) return 0;
+  constexpr size_t resident = (size_t)NORM_BLOCK * max_nv_for<T>(16); /* what the resident reverse holds */
+  if (regime == REGIME_AUTO && packs <= resident) return 0;
+  constexpr size_t tile = (size_t)CLUSTER_THREADS * norm_rev_cluster_nv<T>();
+  size_t ppb = (size_t)cluster_tuning().packs_per_block;
+  if (ppb == 0 || ppb > tile) ppb = tile;
+  const size_t c = (packs + ppb - 1) / ppb;
+  return c >= 1 && c <= (size_t)CLUSTER_MAX ? (int)c : 0;
+}
+
 /* dg_j = sum over partial rows (fixed order, fp64) + alpha * dg_j. A workgroup owns
  * FINISH_LANES * CW columns; its FINISH_SLICES slices split the partial rows, and a thread keeps
  * up to eight CW-wide loads in flight (CW = 4 when the partial rows are 16-byte aligned). */
@@ -579,7 +733,9 @@ inline size_t rmsnorm_reverse_partial_rows(size_t m) {
 
 template <class T>
 inline size_t rmsnorm_reverse_scratch_bytes(size_t m, size_t n) {
-  return rmsnorm_reverse_partial_rows(m) * n * sizeof(typename precision<T>::type);
+  /* the partial rows of dg, then (shared rows only) two words per row and workgroup of the row */
+  const size_t c = (size_t)rmsnorm_rev_cluster_size<T>(n);
+  return (rmsnorm_reverse_partial_rows(m) * n + (c > 1 ? m * c * 2 : 0)) * sizeof(typename precision<T>::type);
 }
 
 template <class T>
@@ -666,7 +822,13 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
   /* four register arrays per thread (x, dy, gain, dg sums): 16 registers each when packed,
    * 8 elements each on the element-wise path */
   constexpr int MAXNV = W == 1 ? 8 : max_nv_for<T>(16);
-  const RowPlan plan = plan_row((n + W - 1) / W, MAXNV, 1, true);
+  /* shared rows: pack-aligned operands, dx distinct from x and dy (a workgroup that stops waiting
+   * re-reads the row), and rows beyond the resident kernel unless the regime is forced */
+  const bool distinct = static_cast<const void*>(dx) != static_cast<const void*>(x) &&
+                        static_cast<const void*>(dx) != static_cast<const void*>(dy);
+  const int C = W > 1 && distinct ? rmsnorm_rev_cluster_size<T>(n) : 0;
+  const bool force_shared = C >= 1 && row_regime_override() == REGIME_CLUSTER;
+  const RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row((n + W - 1) / W, MAXNV, 1, true);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     rows = (unsigned)(need < max_rows ? need : max_rows);
@@ -674,7 +836,28 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
     if (blend) rmsnorm_rev_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
     else rmsnorm_rev_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
   });
-  if (!resident) {
+  bool shared = false;
+  if constexpr (W > 1) {
+    if (!resident && C >= 1) {
+      using Word = typename slot_word<P>::type;
+      size_t S = (size_t)compute_units() / (size_t)C; /* every workgroup resident at once: one per CU (up to 128 registers a thread) */
+      if (S > m) S = m;
+      if (S == 0) S = 1;
+      rows = (unsigned)S;
+      const int ppb = (int)((n / W + C - 1) / C);
+      require(ppb <= CLUSTER_THREADS * norm_rev_cluster_nv<T>(), "rmsnorm reverse: cluster chunk exceeds the register tile");
+      Word* slots = reinterpret_cast<Word*>(partials + rmsnorm_reverse_partial_rows(m) * n);
+      if (C > 1) {
+        const size_t words = m * (size_t)C * 2;
+        cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
+      }
+      const dim3 grid((unsigned)(S * C)), block(CLUSTER_THREADS);
+      if (blend) rmsnorm_rev_cluster<T, W, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+      else rmsnorm_rev_cluster<T, W, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+      shared = true;
+    }
+  }
+  if (!resident && !shared) {
     rows = (unsigned)max_rows;
     const dim3 grid(rows), block(STREAM_THREADS);
     constexpr int NA = W == 1 ? 16 : stream_acc_packs<T>();

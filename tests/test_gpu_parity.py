@@ -617,6 +617,58 @@ def test_rmsnorm_reverse_all_regimes(dtype, regime):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("packs,spin", [(0, 1 << 22), (64, 1 << 22), (64, 0), (1000, 2)],
+                         ids=["default", "64packs", "64packs-nowait", "1000packs-2polls"])
+def test_rmsnorm_reverse_cluster_path(dtype, packs, spin):
+    """Slices of workgroups sharing every row of the slice, two row sums exchanged per row; with a
+    poll limit of 0 or 2 most workgroups give up waiting and read the whole row themselves."""
+    r = rng(62)
+    G.set_regime(CLUSTER)
+    G.set_cluster_tuning(packs, spin)
+    eps = 1e-6
+    for (m, n) in [(3, 8), (5, 64), (4, 1000), (700, 2048), (33, 5000), (2, 50264), (3, 151936), (130, 776)]:
+        for alpha in (0.0, 1.0):
+            G.say(f"rmsnorm rev cluster dtype={dtype} packs={packs} spin={spin} shape=({m},{n}) alpha={alpha}")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype)
+            g = G.dev(r.normal(1, 0.02, n), dtype)
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dx = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dg = G.dev(r.normal(0, 1, n), dtype)
+            hdx, hdg = G.host(dx.t).copy(), G.host(dg.t).copy()
+            scratch, nbytes = G.rmsnorm_scratch(dtype, m, n)
+            G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, eps, alpha)
+            rdx, rdg = O.rmsnorm_ij_j_reverse(G.host(x.t), G.host(g.t), G.host(dy.t), eps,
+                                              hdx if alpha else None, hdg if alpha else None, alpha)
+            sdx, sdg = G.rmsnorm_reverse_scales(G.host(x.t), G.host(g.t), G.host(dy.t), eps,
+                                                hdx if alpha else None, hdg if alpha else None, alpha)
+            G.compare(dx.t, rdx, dtype, f"rmsnorm rev cluster dx ({m},{n}) packs {packs} spin {spin}", scale=sdx)
+            G.compare(dg.t, rdg, dtype, f"rmsnorm rev cluster dg ({m},{n}) packs {packs} spin {spin}",
+                      rowwise=False, scale=sdg)
+            for gd in (x, g, dy, dx, dg, scratch):
+                gd.check("rmsnorm rev cluster")
+
+
+def test_rmsnorm_reverse_long_rows_in_place():
+    # dx written over dy: the shared-row path must not be taken
+    r = rng(63)
+    f32 = torch.float32
+    m, n = 3, 151936
+    x = G.dev(r.normal(0, 1, (m, n)), f32)
+    g = G.dev(r.normal(1, 0.02, n), f32)
+    dy = G.dev(r.normal(0, 1, (m, n)), f32)
+    dg = G.Guarded((n,), f32)
+    rdx, rdg = O.rmsnorm_ij_j_reverse(G.host(x.t), G.host(g.t), G.host(dy.t), 1e-6)
+    sdx, sdg = G.rmsnorm_reverse_scales(G.host(x.t), G.host(g.t), G.host(dy.t), 1e-6)
+    scratch, _ = G.rmsnorm_scratch(f32, m, n)
+    G.say("rmsnorm rev long rows, dx over dy")
+    G.rmsnorm_reverse(x.t, g.t, dy.t, dy.t, dg.t, scratch.t, 1e-6, 0.0)
+    G.compare(dy.t, rdx, f32, "rmsnorm rev in place dx", scale=sdx)
+    G.compare(dg.t, rdg, f32, "rmsnorm rev in place dg", rowwise=False, scale=sdg)
+    for gd in (dy, dg, scratch):
+        gd.check("rmsnorm rev in place")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 def test_rmsnorm_reverse_unaligned(dtype):
     r = rng(61)
     eps = 1e-6
