@@ -24,9 +24,12 @@ namespace mp {
 
 /* One group of G threads per row; groups of 16, 32 or 64 lanes share a 256-thread workgroup
  * (several rows per wavefront below 64), wider groups own one row per workgroup. */
-template <class T, int W, int G>
+/* DOT: every element is multiplied by vec[column] first (a matrix-vector product, one dot
+ * product per row). dst[row] = scale * sum + blend * dst[row]; blend == 0 never reads dst. */
+template <class T, int W, int G, bool DOT>
 __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
-    const T* src, T* dst, typename precision<T>::type alpha, size_t m, size_t n) {
+    const T* src, const T* vec, T* dst, typename precision<T>::type scale, typename precision<T>::type blend,
+    size_t m, size_t n) {
   using P = typename precision<T>::type;
   constexpr int BLOCK = G < 256 ? 256 : G, RPB = BLOCK / G, U = 4;
   __shared__ P slots[G < WAVE ? 1 : G / WAVE];
@@ -38,43 +41,60 @@ __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
   const T* r = src + row * n;
   const RowGeom<T, W> g(r, n, true);
   const T* body = r + g.head;
+  const T* vbody = vec + g.head; /* DOT only: the vector entries of the packed columns */
+  const bool vec_packed = DOT && (reinterpret_cast<uintptr_t>(vbody) & 15u) == 0;
   P s = (P)0;
   for (int p0 = lane; p0 < g.nvec; p0 += G * U) {
-    P buf[U][W];
+    P buf[U][W], wv[U][W];
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const int p = p0 + u * G;
       if (p < g.nvec) {
         load_pack_nt<T, W>(body + (size_t)p * W, buf[u]);
+        if constexpr (DOT) {
+          if (vec_packed) {
+            load_pack<T, W>(vbody + (size_t)p * W, wv[u]);
+          } else {
+#pragma unroll
+            for (int i = 0; i < W; ++i) wv[u][i] = (P)vbody[(size_t)p * W + i];
+          }
+        }
       } else {
 #pragma unroll
-        for (int i = 0; i < W; ++i) buf[u][i] = (P)0;
+        for (int i = 0; i < W; ++i) buf[u][i] = wv[u][i] = (P)0;
       }
     }
 #pragma unroll
     for (int u = 0; u < U; ++u)
 #pragma unroll
-      for (int i = 0; i < W; ++i) s += buf[u][i];
+      for (int i = 0; i < W; ++i) s += DOT ? buf[u][i] * wv[u][i] : buf[u][i];
   }
   if (W > 1) {
-    if (lane < g.head) s += (P)r[lane];
-    else if (lane - g.head < g.tail) s += (P)body[(size_t)g.nvec * W + (lane - g.head)];
+    size_t e = (size_t)-1;
+    if (lane < g.head) e = (size_t)lane;
+    else if (lane - g.head < g.tail) e = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
+    if (e != (size_t)-1) s += DOT ? (P)r[e] * (P)vec[e] : (P)r[e];
   }
   s = group_allreduce<AddOP, G>(s, slots, lane);
-  if (live && lane == 0) dst[row] = (T)(alpha != (P)0 ? s + alpha * (P)dst[row] : s);
+  if (live && lane == 0) dst[row] = (T)(blend != (P)0 ? scale * s + blend * (P)dst[row] : scale * s);
 }
 
+/* dst[i] = scale * sum_j src[i,j] (* vec[j] when vec is given) + blend * dst[i] */
 template <class T>
-inline void reduce_rows(const T* src, T* dst, double alpha, size_t m, size_t n, hipStream_t stream) {
+inline void reduce_rows(const T* src, const T* vec, T* dst, double scale, double blend, size_t m, size_t n,
+                        hipStream_t stream) {
   if (m == 0) return;
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  require(n <= 0x40000000ull, "reduce_ij_i: row length must not exceed 2^30");
-  require(m < 0x7fffffffull, "reduce_ij_i: too many rows for one grid");
+  require(n <= 0x40000000ull, "row sums: row length must not exceed 2^30");
+  require(m < 0x7fffffffull, "row sums: too many rows for one grid");
   const size_t packs = (n + W - 1) / W;
-#define MP_ROWS_LAUNCH(G_) \
-  reduce_rows_kernel<T, W, G_><<<dim3((unsigned)((m + (G_ < 256 ? 256 / G_ : 1) - 1) / (G_ < 256 ? 256 / G_ : 1))), \
-                              dim3(G_ < 256 ? 256 : G_), 0, stream>>>(src, dst, (P)alpha, m, n)
+#define MP_ROWS_LAUNCH(G_)                                                                                          \
+  do {                                                                                                              \
+    const dim3 grid((unsigned)((m + (G_ < 256 ? 256 / G_ : 1) - 1) / (G_ < 256 ? 256 / G_ : 1))), block(G_ < 256 ? 256 : G_); \
+    if (vec) reduce_rows_kernel<T, W, G_, true><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, m, n); \
+    else reduce_rows_kernel<T, W, G_, false><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, m, n);   \
+  } while (0)
   if (packs <= 16) MP_ROWS_LAUNCH(16);
   else if (packs <= 32) MP_ROWS_LAUNCH(32);
   else if (packs <= 256) MP_ROWS_LAUNCH(64);
@@ -84,16 +104,23 @@ inline void reduce_rows(const T* src, T* dst, double alpha, size_t m, size_t n, 
   MP_CHECK_LAUNCH();
 }
 
+template <class T>
+inline void reduce_rows(const T* src, T* dst, double alpha, size_t m, size_t n, hipStream_t stream) {
+  reduce_rows<T>(src, nullptr, dst, 1.0, alpha, m, n, stream);
+}
+
 /* ------------------------------------------------------------------ column sums */
 
 /* A workgroup owns LANES*CW columns of the rows [blockIdx.y * chunk, (blockIdx.y + 1) * chunk); its
  * SLICES slices take every SLICES-th of those rows and are folded through LDS in slice order, so
  * the result does not depend on scheduling. The sums go to `out + blockIdx.y * n`: the destination
  * itself (O = T, one chunk holding every row, alpha blend) or a partial row of accumulators
- * (O = precision<T>, no blend) that sum_partial_rows adds up afterwards. */
-template <class T, class O, int CW, int LANES, int SLICES>
+ * (O = precision<T>, no blend) that sum_partial_rows adds up afterwards. WEIGHTED: row r counts
+ * weight[r] times (a vector-matrix product). */
+template <class T, class O, int CW, int LANES, int SLICES, bool WEIGHTED>
 __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
-    const T* src, O* out, typename precision<T>::type alpha, size_t m, size_t n, size_t chunk) {
+    const T* src, const T* weight, O* out, typename precision<T>::type scale, typename precision<T>::type blend,
+    size_t m, size_t n, size_t chunk) {
   using P = typename precision<T>::type;
   __shared__ P part[SLICES][LANES * CW + 1];
   const int c = threadIdx.x % LANES, slice = threadIdx.x / LANES;
@@ -106,19 +133,23 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
   if (col < n) {
     size_t r = begin + slice;
     for (; r + 3 * SLICES < end; r += 4 * SLICES) {
-      P v[4][CW];
+      P v[4][CW], w[4];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) load_pack_nt<T, CW>(src + (r + (size_t)u * SLICES) * n + col, v[u]);
+      for (int u = 0; u < 4; ++u) {
+        load_pack_nt<T, CW>(src + (r + (size_t)u * SLICES) * n + col, v[u]);
+        w[u] = WEIGHTED ? (P)weight[r + (size_t)u * SLICES] : (P)1;
+      }
 #pragma unroll
       for (int u = 0; u < 4; ++u)
 #pragma unroll
-        for (int i = 0; i < CW; ++i) s[i] += v[u][i];
+        for (int i = 0; i < CW; ++i) s[i] += WEIGHTED ? w[u] * v[u][i] : v[u][i];
     }
     for (; r < end; r += SLICES) {
       P v[CW];
       load_pack_nt<T, CW>(src + r * n + col, v);
+      const P w = WEIGHTED ? (P)weight[r] : (P)1;
 #pragma unroll
-      for (int i = 0; i < CW; ++i) s[i] += v[i];
+      for (int i = 0; i < CW; ++i) s[i] += WEIGHTED ? w * v[i] : v[i];
     }
   }
 #pragma unroll
@@ -129,7 +160,7 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
   if (mine < LANES * CW && at < n) {
     P t = (P)0;
     for (int i = 0; i < SLICES; ++i) t += part[i][mine];
-    dst[at] = (O)(alpha != (P)0 ? t + alpha * (P)dst[at] : t);
+    dst[at] = (O)(blend != (P)0 ? scale * t + blend * (P)dst[at] : scale * t);
   }
 }
 
@@ -153,33 +184,106 @@ template <class T> inline size_t reduce_cols_scratch_bytes(size_t m, size_t n) {
   return chunks > 1 ? chunks * n * sizeof(typename precision<T>::type) : 0;
 }
 
-/* scratch: reduce_cols_scratch_bytes(m, n) bytes or NULL (then one workgroup per column strip
+/* dst[j] = scale * sum_i (weight[i] *) src[i,j] + blend * dst[j].
+ * scratch: reduce_cols_scratch_bytes(m, n) bytes or NULL (then one workgroup per column strip
  * walks every row, which leaves most of the GPU idle on tall, narrow matrices). */
 template <class T>
-inline void reduce_cols(const T* src, T* dst, void* scratch, double alpha, size_t m, size_t n, hipStream_t stream) {
+inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, double scale, double blend, size_t m,
+                        size_t n, hipStream_t stream) {
   if (n == 0) return;
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   const bool packed = aligned16(src) && (n % W) == 0;
+#define MP_COLS(O_, CW_, L_, S_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)                                                        \
+  do {                                                                                                                       \
+    if (weight) reduce_cols_kernel<T, O_, CW_, L_, S_, true><<<GRID_, dim3(1024), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_); \
+    else reduce_cols_kernel<T, O_, CW_, L_, S_, false><<<GRID_, dim3(1024), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_);       \
+  } while (0)
   if (packed) { /* 8 lanes x one pack = 128 bytes of every row per workgroup */
     const size_t blocks = (n / W + 7) / 8;
-    require(blocks < 0x7fffffffull, "reduce_ij_j: too many columns for one grid");
+    require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
     const size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;
     if (chunks > 1) {
       const size_t chunk = (m + chunks - 1) / chunks;
       P* partials = static_cast<P*>(scratch);
-      reduce_cols_kernel<T, P, W, 8, 128><<<dim3((unsigned)blocks, (unsigned)chunks), dim3(1024), 0, stream>>>(
-          src, partials, (P)0, m, n, chunk);
+      MP_COLS(P, W, 8, 128, dim3((unsigned)blocks, (unsigned)chunks), partials, (P)scale, (P)0, chunk);
       MP_CHECK_LAUNCH();
-      sum_partial_rows<T>(partials, dst, alpha, (unsigned)chunks, n, stream);
+      sum_partial_rows<T>(partials, dst, blend, (unsigned)chunks, n, stream);
       return;
     }
-    reduce_cols_kernel<T, T, W, 8, 128><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n, m);
+    MP_COLS(T, W, 8, 128, dim3((unsigned)blocks), dst, (P)scale, (P)blend, m);
   } else {
     /* rows that are not pack-aligned: one element per lane, a wavefront per 64-element row segment */
     const size_t blocks = (n + 63) / 64;
-    require(blocks < 0x7fffffffull, "reduce_ij_j: too many columns for one grid");
-    reduce_cols_kernel<T, T, 1, 64, 16><<<dim3((unsigned)blocks), dim3(1024), 0, stream>>>(src, dst, (P)alpha, m, n, m);
+    require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
+    MP_COLS(T, 1, 64, 16, dim3((unsigned)blocks), dst, (P)scale, (P)blend, m);
+  }
+#undef MP_COLS
+  MP_CHECK_LAUNCH();
+}
+
+template <class T>
+inline void reduce_cols(const T* src, T* dst, void* scratch, double alpha, size_t m, size_t n, hipStream_t stream) {
+  reduce_cols<T>(src, nullptr, dst, scratch, 1.0, alpha, m, n, stream);
+}
+
+/* c[i,l] = scale * a[i] * b[l] + blend * c[i,l]: the product of a column and a row vector, written
+ * like a broadcast (flat, one pack per thread) when c is pack-aligned. */
+template <class T, int W, bool BLEND>
+__global__ __launch_bounds__(256) void outer_flat_kernel(
+    const T* a, const T* b, T* c, typename precision<T>::type scale, typename precision<T>::type blend,
+    size_t total, unsigned n) {
+  using P = typename precision<T>::type;
+  const size_t packs = total / W;
+  const size_t base = (size_t)blockIdx.x * 256 * W;
+  const size_t row0 = base / n;
+  const unsigned off = (unsigned)(base - row0 * n) + threadIdx.x * W;
+  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (idx < packs) {
+    const size_t row = row0 + off / n;
+    const unsigned col = off % n;
+    P out[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      const bool next = col + i >= n; /* n >= W: a pack ends in the next row at most */
+      out[i] = scale * (P)a[row + (next ? 1 : 0)] * (P)b[next ? col + i - n : col + i];
+    }
+    T* o = c + idx * W;
+    if constexpr (BLEND) {
+      P old[W];
+      load_pack_nt<T, W>(o, old);
+#pragma unroll
+      for (int i = 0; i < W; ++i) out[i] += blend * old[i];
+    }
+    store_pack_nt<T, W>(o, out);
+  }
+  if (blockIdx.x == gridDim.x - 1) {
+    const size_t e = packs * W + threadIdx.x;
+    if (threadIdx.x < W && e < total) {
+      P v = scale * (P)a[e / n] * (P)b[e % n];
+      if constexpr (BLEND) v += blend * (P)c[e];
+      c[e] = (T)v;
+    }
+  }
+}
+
+template <class T>
+inline void outer_product(const T* a, const T* b, T* c, double scale, double blend, size_t m, size_t n, hipStream_t stream) {
+  if (m == 0 || n == 0) return;
+  using P = typename precision<T>::type;
+  require(n <= 0x40000000ull, "outer product: row length must not exceed 2^30");
+  const size_t total = m * n;
+  if (aligned16(c) && n >= (size_t)(PACK_BYTES / sizeof(T))) {
+    constexpr int W = PACK_BYTES / (int)sizeof(T);
+    const size_t blocks = (total / W + 255) / 256 + 1;
+    require(blocks < 0x7fffffffull, "outer product: too many elements for one grid");
+    if (blend != 0.0) outer_flat_kernel<T, W, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n);
+    else outer_flat_kernel<T, W, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n);
+  } else {
+    const size_t blocks = (total + 255) / 256 + 1;
+    require(blocks < 0x7fffffffull, "outer product: too many elements for one grid");
+    if (blend != 0.0) outer_flat_kernel<T, 1, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n);
+    else outer_flat_kernel<T, 1, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n);
   }
   MP_CHECK_LAUNCH();
 }

@@ -75,7 +75,9 @@ def test_permutate_involution_at_size():
 
 
 GEMM_SHAPES = [(1, 1, 1), (3, 2, 2), (2, 3, 4), (5, 7, 3), (1, 64, 9), (9, 64, 1), (33, 1, 17), (64, 64, 64),
-               (129, 255, 65), (256, 1024, 96), (7, 4099, 5)]
+               (129, 255, 65), (256, 1024, 96), (7, 4099, 5),
+               # products with a vector run on the row / column sum kernels
+               (1, 5000, 300), (300, 5000, 1), (129, 1, 255), (1, 4099, 7), (2000, 33, 1), (1, 777, 1)]
 FORMS = [("ij_jk_ik", False, False), ("ij_kj_ik", False, True), ("ji_jk_ik", True, False)]
 
 
