@@ -181,7 +181,7 @@ static int fused_chain(mp::Stream stream) {
     dump("chain_selu_mul_sub_da", a.native_grad<float>()); dump("chain_selu_mul_sub_db", b.native_grad<float>());
     dump("chain_selu_mul_sub_dc", c.native_grad<float>());
 
-    /* not in the table as a whole: relu is eager, its operand selu(add(a,b)) is a chain */
+    /* not in the table as a whole: relu takes its own kernel, its operand selu(add(a,b)) is a chain */
     G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
     l = G->launches;
     mp::Tensor r2 = mp::ops::relu(mp::ops::selu(mp::ops::add(a, b)));
@@ -189,6 +189,17 @@ static int fused_chain(mp::Stream stream) {
     CHECK(G->launches == l + 2);
     r2.reverse(mp::ReverseCleanup::free);
     dump("chain_relu_selu_add_da", a.native_grad<float>());
+
+    /* relu defers like the other elementwise ops: relu(hadamard(add, add)) is one kernel each way */
+    G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+    l = G->launches;
+    mp::Tensor r3 = mp::ops::relu(mp::ops::hadamard(mp::ops::add(a, b), mp::ops::add(c, d)));
+    dump("chain_relu_mul_add_add", r3.native<float>());
+    CHECK(G->launches == l + 1);
+    l = G->launches;
+    r3.reverse(mp::ReverseCleanup::free);
+    CHECK(G->launches == l + 2); /* the seed fill and one reverse kernel */
+    dump("chain_relu_mul_add_add_da", a.native_grad<float>()); dump("chain_relu_mul_add_add_dc", c.native_grad<float>());
 
     /* sub alone is not a chain: per-op kernel and the per-op reverse (gx += gz, gy -= gz) */
     G->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);

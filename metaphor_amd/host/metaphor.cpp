@@ -297,6 +297,7 @@ static void addition_reverse(const std::vector<OpDatum>& a);
 static void subtraction_reverse(const std::vector<OpDatum>& a);
 static void hadamard_reverse(const std::vector<OpDatum>& a);
 static void selu_reverse(const std::vector<OpDatum>& a);
+static void relu_reverse(const std::vector<OpDatum>& a);
 static void chain_reverse(const std::vector<OpDatum>& a);
 
 static const char* pending_name(Pending op) {
@@ -305,6 +306,7 @@ static const char* pending_name(Pending op) {
     case Pending::sub: return "sub";
     case Pending::hadamard: return "mul";
     case Pending::selu: return "selu";
+    case Pending::relu: return "relu";
     default: return "?";
   }
 }
@@ -319,7 +321,7 @@ static bool spell(Graph* g, Tensor t, std::string& out, std::vector<Tensor>& lea
     out += pending_name(node.pending);
     out += '(';
     if (!spell(g, node.in0, out, leaves, budget)) return false;
-    if (node.pending != Pending::selu) {
+    if (node.pending != Pending::selu && node.pending != Pending::relu) {
       out += ',';
       if (!spell(g, node.in1, out, leaves, budget)) return false;
     }
@@ -388,11 +390,12 @@ void materialise(Tensor t) {
   /* anything else: one launch per op, as the reference's forward_impl does */
   if (in0.len() == 0 || in1.len() == 0) panic("materialise: an input of a pending node was freed");
   void* p0 = in0.data_ptr();
-  if (op == Pending::selu) {
+  if (op == Pending::selu || op == Pending::relu) {
     void* pz = take_buffer();
-    kernels::selu(key, p0, pz, (len_t)n, ctx);
+    if (op == Pending::selu) kernels::selu(key, p0, pz, (len_t)n, ctx);
+    else kernels::relu(key, p0, pz, (len_t)n, ctx);
     g->launches++;
-    if (g->mode == Mode::train) attach_op(t, selu_reverse, {in0, t});
+    if (g->mode == Mode::train) attach_op(t, op == Pending::selu ? selu_reverse : relu_reverse, {in0, t});
     return;
   }
   void* p1 = in1.data_ptr();
@@ -668,16 +671,8 @@ Tensor hadamard(Tensor x, Tensor y) {
 
 Tensor selu(Tensor x) { return defer(x.ptr, Pending::selu, x, x); }
 
-/* src/ops/relu.zig:13-37 */
-Tensor relu(Tensor x) {
-  Graph* g = x.ptr;
-  void* px = x.data_ptr();
-  Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
-  kernels::relu(dkey(z), px, z.data_ptr(), (len_t)z.len(), z.context());
-  g->launches++;
-  if (g->mode == Mode::train) attach_op(z, relu_reverse, {x, z});
-  return z;
-}
+/* src/ops/relu.zig:13-37, deferred like the other elementwise ops */
+Tensor relu(Tensor x) { return defer(x.ptr, Pending::relu, x, x); }
 
 Tensor softmax(Tensor x, const char* expr) {
   if (std::strcmp(expr, "ij|j") != 0) panic("softmax: only the row form \"ij|j\" exists");

@@ -15,7 +15,7 @@
  * Errors follow the reference: an impossible request panics (prints and aborts), nothing returns
  * a status.
  *
- * What is new here is where the kernels come from. add / sub / hadamard / selu do not launch:
+ * What is new here is where the kernels come from. add / sub / hadamard / selu / relu do not launch:
  * they record a pending node. A pending node is materialised when something needs its bytes (a
  * non-elementwise op, data_ptr(), native(), reverse()). At that point the recorded expression is
  * written out with its leaves numbered in order of first appearance and looked up in the table
@@ -153,7 +153,7 @@ class TensorAllocator {
   std::unordered_map<size_t, std::vector<void*>> cache_;
 };
 
-enum class Pending : int { none = 0, add, sub, hadamard, selu };
+enum class Pending : int { none = 0, add, sub, hadamard, selu, relu };
 
 /* deferred elementwise nodes: record, query, compute */
 Tensor defer(Graph* g, Pending op, Tensor x, Tensor y);

@@ -72,6 +72,12 @@ def test_host_library_end_to_end(tmp_path):
          O.selu_reverse(a64 + b64, np.ones_like(a64)) * (O.selu(a64 + b64) >= 0), "relu(selu(add)) da",
          rowwise=False)
     del sa32
+    w4 = (a64 + b64) * (c64 + dd.astype(np.float64))
+    _cmp(_load(d, "chain_relu_mul_add_add"), np.maximum(w4, 0.0), "relu(mul(add,add))", rowwise=False)
+    live = (_load(d, "chain_relu_mul_add_add") > 0).astype(np.float64)  # the slope the r32 kernel saw
+    _cmp(_load(d, "chain_relu_mul_add_add_da"), live * (c64 + dd.astype(np.float64)), "relu(mul(add,add)) da",
+         rowwise=False, rtol=2e-5)
+    _cmp(_load(d, "chain_relu_mul_add_add_dc"), live * (a64 + b64), "relu(mul(add,add)) dc", rowwise=False, rtol=2e-5)
     _cmp(_load(d, "plain_sub"), a64 - b64, "sub", rowwise=False)
     assert np.all(_load(d, "plain_sub_da") == 1.0) and np.all(_load(d, "plain_sub_db") == -1.0)
 
