@@ -17,8 +17,15 @@ def _selu(x):
     return torch.where(x > 0, lam * x, lam * alp * torch.expm1(torch.clamp(x, max=0.0)))
 
 
+def _relu(x):
+    """relu with the reference's convention at the kink: slope 1 at exactly 0 (a >= 0 passes the
+    gradient, src/cuda/nvcc_src/relu_reverse.cu:12-14); torch.relu takes slope 0 there, and
+    half-precision operands hit exact zeros often."""
+    return torch.where(x >= 0, x, torch.zeros_like(x))
+
+
 TORCH_OP = {"add": torch.add, "sub": torch.sub, "mul": torch.mul, "neg": torch.neg,
-            "relu": torch.relu, "selu": _selu}
+            "relu": _relu, "selu": _selu}
 
 
 def _torch_eval(node, leaves):
