@@ -325,6 +325,15 @@ def generate():
                 changed.append(path)
     if _write_if_changed(os.path.join(HOST_DIR, "chains.hpp"), host_table(chains)):
         changed.append(os.path.join(HOST_DIR, "chains.hpp"))
+    # a chain taken out of chains.json takes its generated sources with it
+    wanted = {c["name"] + suffix for c in chains for suffix in (".hip", "_reverse.hip")}
+    for name in sorted(os.listdir(SRC_DIR)):
+        path = os.path.join(SRC_DIR, name)
+        if name.endswith(".hip") and name not in wanted:
+            with open(path) as f:
+                if "GENERATED by metaphor_amd/chaingen.py" in f.read(400):
+                    os.remove(path)
+                    changed.append(path)
     return changed
 
 
