@@ -39,7 +39,7 @@ typedef struct { void* ptr; } PaddedPtr;
 
 typedef struct {
   PaddedPtr hip_stream;   /* hipStream_t */
-  PaddedPtr blas_handle;  /* rocblas_handle made by mpInitStream; NULL for a borrowed stream */
+  PaddedPtr blas_handle;  /* BLAS state (handle + workspace) made by mpInitStream / mpAdoptStream; NULL for a borrowed stream */
 } StreamContext;
 
 /* SELU constants of the fused-chain workload (self-normalising networks' alpha and

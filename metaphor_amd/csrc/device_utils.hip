@@ -65,28 +65,22 @@ extern "C" StreamContext mpInitStream() {
   context.hip_stream.ptr = reinterpret_cast<void*>(hip_stream);
   /* the matrix-product launchers find their library handle here, bound to this stream
    * (device_utils.cu:72-86 does the same with cuBLAS) */
-  rocblas_handle blas = nullptr;
-  ROCBLAS_ASSERT(rocblas_create_handle(&blas));
-  ROCBLAS_ASSERT(rocblas_set_stream(blas, hip_stream));
-  context.blas_handle.ptr = reinterpret_cast<void*>(blas);
+  context.blas_handle.ptr = mpCreateBlasContext(hip_stream);
   return context;
 }
 
 extern "C" StreamContext mpAdoptStream(void* hip_stream) {
-  rocblas_handle blas = nullptr;
-  ROCBLAS_ASSERT(rocblas_create_handle(&blas));
-  ROCBLAS_ASSERT(rocblas_set_stream(blas, static_cast<hipStream_t>(hip_stream)));
   StreamContext context;
   context.hip_stream.ptr = hip_stream;
-  context.blas_handle.ptr = reinterpret_cast<void*>(blas);
+  context.blas_handle.ptr = mpCreateBlasContext(static_cast<hipStream_t>(hip_stream));
   return context;
 }
 
 extern "C" void mpReleaseStream(StreamContext stream) {
-  if (get_handle(stream) != nullptr) ROCBLAS_ASSERT(rocblas_destroy_handle(get_handle(stream)));
+  mpDestroyBlasContext(get_blas(stream));
 }
 
 extern "C" void mpDeinitStream(StreamContext stream) {
-  if (get_handle(stream) != nullptr) ROCBLAS_ASSERT(rocblas_destroy_handle(get_handle(stream)));
+  mpDestroyBlasContext(get_blas(stream));
   HIP_ASSERT(hipStreamDestroy(get_stream(stream)));
 }

@@ -4,7 +4,7 @@
  * Sgemm / Dgemm behind mp_gemm<T>) and of the column-major argument swap in
  * src/cuda/nvcc_src/inner_product_ij_jk_ik.cu:12-26.
  *
- * The handle travels in the second slot of the StreamContext, as the reference's cuBLAS handle
+ * The handle travels behind the second slot of the StreamContext, as the reference's cuBLAS handle
  * does (src/cuda/kernel_header.h:58-60); mpInitStream creates it and binds it to the stream.
  * r16 multiplies half inputs with fp32 accumulation (the up-cast rule of
  * src/cuda/tensor_types.h:51-69; the reference's cublasHgemm accumulates in half), r32 and r64
@@ -20,8 +20,24 @@
 
 #include <rocblas/rocblas.h>
 
+/* What the second slot of a StreamContext points to: the rocBLAS handle bound to the stream and a
+ * workspace the vector products may split their rows through (owned here, so a launcher
+ * allocates nothing). Made by mpInitStream / mpAdoptStream, released by mpDeinitStream /
+ * mpReleaseStream; work that uses the workspace is ordered by the stream. */
+struct MpBlasContext {
+  rocblas_handle rocblas;
+  void* workspace;
+  size_t workspace_bytes;
+  hipStream_t stream;
+};
+constexpr size_t MP_BLAS_WORKSPACE_BYTES = 16u << 20;
+
+inline MpBlasContext* get_blas(StreamContext context) {
+  return static_cast<MpBlasContext*>(context.blas_handle.ptr);
+}
 inline rocblas_handle get_handle(StreamContext context) {
-  return static_cast<rocblas_handle>(context.blas_handle.ptr);
+  MpBlasContext* c = get_blas(context);
+  return c ? c->rocblas : nullptr;
 }
 
 #define ROCBLAS_ASSERT(err) (mpHandleBlasError((err), __FILE__, __LINE__))
@@ -30,6 +46,20 @@ inline void mpHandleBlasError(rocblas_status err, const char* file, int line) {
     fprintf(stderr, "rocBLAS failure (%s) in %s at line %d\n", rocblas_status_to_string(err), file, line);
     exit(EXIT_FAILURE);
   }
+}
+
+inline MpBlasContext* mpCreateBlasContext(hipStream_t stream) {
+  MpBlasContext* c = new MpBlasContext{nullptr, nullptr, MP_BLAS_WORKSPACE_BYTES, stream};
+  ROCBLAS_ASSERT(rocblas_create_handle(&c->rocblas));
+  ROCBLAS_ASSERT(rocblas_set_stream(c->rocblas, stream));
+  HIP_ASSERT(hipMalloc(&c->workspace, c->workspace_bytes));
+  return c;
+}
+inline void mpDestroyBlasContext(MpBlasContext* c) {
+  if (c == nullptr) return;
+  HIP_ASSERT(hipFree(c->workspace));
+  ROCBLAS_ASSERT(rocblas_destroy_handle(c->rocblas));
+  delete c;
 }
 
 namespace mp {
@@ -54,10 +84,13 @@ inline void gemm_row_major(StreamContext ctx, bool a_transposed, bool b_transpos
     const T* B = static_cast<const T*>(b);
     T* C = static_cast<T*>(c);
     hipStream_t stream = get_stream(ctx);
+    MpBlasContext* blas = get_blas(ctx); /* may be absent: the column sums then walk all rows per strip */
+    void* ws = blas ? blas->workspace : nullptr;
+    const size_t ws_bytes = blas ? blas->workspace_bytes : 0;
     if (n == 1) outer_product<T>(A, B, C, alpha, beta, m, k, stream);
     else if (k == 1 && !a_transposed) reduce_rows<T>(A, B, C, alpha, beta, m, n, stream);
-    else if (k == 1) reduce_cols<T>(A, B, C, nullptr, alpha, beta, n, m, stream);
-    else if (!b_transposed) reduce_cols<T>(B, A, C, nullptr, alpha, beta, n, k, stream);
+    else if (k == 1) reduce_cols<T>(A, B, C, ws, alpha, beta, n, m, stream, ws_bytes);
+    else if (!b_transposed) reduce_cols<T>(B, A, C, ws, alpha, beta, n, k, stream, ws_bytes);
     else reduce_rows<T>(B, A, C, alpha, beta, k, n, stream);
     return;
   }

@@ -189,7 +189,7 @@ template <class T> inline size_t reduce_cols_scratch_bytes(size_t m, size_t n) {
  * walks every row, which leaves most of the GPU idle on tall, narrow matrices). */
 template <class T>
 inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, double scale, double blend, size_t m,
-                        size_t n, hipStream_t stream) {
+                        size_t n, hipStream_t stream, size_t scratch_bytes = ~(size_t)0) {
   if (n == 0) return;
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
@@ -202,7 +202,9 @@ inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, do
   if (packed) { /* 8 lanes x one pack = 128 bytes of every row per workgroup */
     const size_t blocks = (n / W + 7) / 8;
     require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
-    const size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;
+    size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;
+    const size_t fit = scratch_bytes / (n * sizeof(P)); /* partial rows the workspace holds */
+    if (chunks > fit) chunks = fit;
     if (chunks > 1) {
       const size_t chunk = (m + chunks - 1) / chunks;
       P* partials = static_cast<P*>(scratch);
