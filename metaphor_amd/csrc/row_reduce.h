@@ -344,6 +344,19 @@ __global__ __launch_bounds__(256) void broadcast_flat_kernel(
   const size_t row0 = base / n;                     /* one 64-bit division is scalar work */
   const unsigned off = (unsigned)(base - row0 * n) + threadIdx.x * W;
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  /* ragged column values: the workgroup's 256 * W consecutive elements need a window of 256 * W
+   * consecutive (wrapping) entries of src; it is fetched with coalesced element loads into LDS once
+   * instead of W scattered loads per thread */
+  __shared__ T window[(!ALIGNED && !BY_ROW) ? 256 * W : 1];
+  if constexpr (!ALIGNED && !BY_ROW) {
+    const unsigned first = (unsigned)(base - row0 * n); /* column of the workgroup's first element */
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      const unsigned t = threadIdx.x + 256u * i;
+      window[t] = src[(first + t) % n];
+    }
+    __syncthreads();
+  }
   if (idx < packs) {
     const size_t row = row0 + off / n;
     const unsigned col = off % n;
@@ -360,7 +373,7 @@ __global__ __launch_bounds__(256) void broadcast_flat_kernel(
 #pragma unroll
       for (int i = 0; i < W; ++i) {
         const bool next = col + i >= n;
-        out[i] = BY_ROW ? (P)src[row + (next ? 1 : 0)] : (P)src[next ? col + i - n : col + i];
+        out[i] = BY_ROW ? (P)src[row + (next ? 1 : 0)] : (P)window[threadIdx.x * W + i];
       }
     }
     T* o = dst + idx * W;
