@@ -15,6 +15,9 @@
  * sits in slot p ^ (r / W)), which keeps the 128-bit LDS writes aligned and spreads the transposed
  * reads over the banks. r16 tiles are gathered as 32-bit words (two neighbouring columns at
  * once) and separated in registers, so a thread issues W/2 LDS reads per output pack.
+ * Operands whose rows are not 16-byte aligned (an odd row length, a shifted base) keep 128-bit
+ * global accesses: every row segment is peeled so that its packs are aligned in memory, and only
+ * the LDS side goes element by element.
  * HBM-bound: 2 * sizeof(T) bytes per element (3 when alpha != 0).
  */
 #ifndef MP_PERMUTATE_H
@@ -77,11 +80,55 @@ __global__ __launch_bounds__(tp_threads<T>()) void permutate_kernel(
       *reinterpret_cast<VA*>(&tile[r * TC + ((p ^ (r / W)) & (CP - 1)) * W]) = v[s];
     }
   } else {
-    for (int idx = tid; idx < TR * TC; idx += THREADS) {
-      const int r = idx / TC, c = idx % TC;
-      T x = (T)0;
-      if (r0 + r < rows && c0 + c < cols) x = src[(r0 + r) * cols + c0 + c];
-      tile[tp_at<W>(r, c)] = x;
+    /* Source rows whose length or base breaks the 16-byte alignment: each row's 128-byte segment
+     * is peeled into [head scalars][packs aligned in MEMORY][tail scalars]; head and tail together
+     * are exactly one pack's worth of elements, so the CP slots of a row still move W elements
+     * each: CP - 1 aligned packs and one slot of scalars. A segment cut short by the matrix edge
+     * is read element by element. Everything lands in LDS element by element. */
+    const int len = cols - c0 < (size_t)TC ? (int)(cols - c0) : TC; /* uniform over the workgroup */
+    T v[STEPS][W];
+    /* tile column of element i of slot q of a row whose head is h elements long, -1: none */
+    auto column = [&](int q, int h, int i) -> int {
+      if (len != TC) return q * W + i < len ? q * W + i : -1;
+      if (q < CP - (h ? 1 : 0)) return h + q * W + i;
+      return i < h ? i : TC - W + i; /* the last slot of a misaligned row: its head and its tail */
+    };
+    auto head = [&](int r) -> int {
+      const T* seg = src + (r0 + r) * cols + c0;
+      return (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(seg) & 15u)) & 15u) / sizeof(T));
+    };
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int idx = s * THREADS + tid, r = idx / CP, q = idx % CP;
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[s][i] = (T)0;
+      if (r0 + r < rows) {
+        const T* seg = src + (r0 + r) * cols + c0;
+        const int h = head(r);
+        if (len == TC && q < CP - (h ? 1 : 0)) {
+          const V pack = __builtin_nontemporal_load(reinterpret_cast<const V*>(seg + h + q * W));
+#pragma unroll
+          for (int i = 0; i < W; ++i) v[s][i] = pack[i];
+        } else {
+#pragma unroll
+          for (int i = 0; i < W; ++i) {
+            const int c = column(q, h, i);
+            if (c >= 0) v[s][i] = seg[c];
+          }
+        }
+      }
+    }
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int idx = s * THREADS + tid, r = idx / CP, q = idx % CP;
+      if (r0 + r < rows) {
+        const int h = head(r);
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+          const int c = column(q, h, i);
+          if (c >= 0) tile[tp_at<W>(r, c)] = v[s][i];
+        }
+      }
     }
   }
   __syncthreads();
@@ -137,13 +184,36 @@ __global__ __launch_bounds__(tp_threads<T>()) void permutate_kernel(
     for (int s = 0; s < STEPS; ++s)
       if (at[s] != npos) __builtin_nontemporal_store(out[s], reinterpret_cast<V*>(dst + at[s]));
   } else {
-    for (int idx = tid; idx < TR * TC; idx += THREADS) {
-      const int j = idx / TR, i = idx % TR;
-      if (c0 + j < cols && r0 + i < rows) {
-        T* o = dst + (c0 + j) * rows + r0 + i;
-        T x = tile[tp_at<W>(i, j)];
-        if constexpr (BLEND) x = (T)((P)x + alpha * (P)*o);
-        *o = x;
+    /* Destination rows that break the alignment: the same peeling on the way out. The LDS gather
+     * is element by element in any case, so a pack may start at any row of the tile. */
+    const int len = rows - r0 < (size_t)TR ? (int)(rows - r0) : TR;
+#pragma unroll
+    for (int s = 0; s < STEPS; ++s) {
+      const int idx = s * THREADS + tid, j = idx / RP, q = idx % RP;
+      if (c0 + j >= cols) continue;
+      T* seg = dst + (c0 + j) * rows + r0;
+      const int h = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(seg) & 15u)) & 15u) / sizeof(T));
+      if (len == TR && q < RP - (h ? 1 : 0)) {
+        const int i0 = h + q * W;
+        V out;
+#pragma unroll
+        for (int e = 0; e < W; ++e) out[e] = tile[tp_at<W>(i0 + e, j)];
+        if constexpr (BLEND) {
+          const V old = *reinterpret_cast<const V*>(seg + i0);
+#pragma unroll
+          for (int e = 0; e < W; ++e) out[e] = (T)((P)out[e] + alpha * (P)old[e]);
+        }
+        __builtin_nontemporal_store(out, reinterpret_cast<V*>(seg + i0));
+      } else {
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+          const int i = len == TR ? (e < h ? e : TR - W + e) : q * W + e;
+          if (i < len) {
+            T x = tile[tp_at<W>(i, j)];
+            if constexpr (BLEND) x = (T)((P)x + alpha * (P)seg[i]);
+            seg[i] = x;
+          }
+        }
       }
     }
   }

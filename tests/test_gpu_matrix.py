@@ -19,9 +19,10 @@ def rng(seed):
 
 
 # rows x cols: single element, vectors, tiles exactly, one past a tile, ragged both ways,
-# odd sizes that force the scalar paths on one side or both
+# odd sizes that force the peeled (memory-aligned) paths on one side or both, with whole tiles and cut ones
 TRANSPOSE_SHAPES = [(1, 1), (1, 7), (7, 1), (3, 2), (64, 64), (128, 128), (65, 64), (64, 65), (129, 257),
-                    (32, 1000), (1000, 32), (8, 4096), (50257, 3), (100, 104), (104, 100), (1027, 513)]
+                    (32, 1000), (1000, 32), (8, 4096), (50257, 3), (100, 104), (104, 100), (1027, 513),
+                    (520, 777), (1030, 66), (2049, 130)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
