@@ -237,14 +237,14 @@ template <class OP> __device__ __forceinline__ double fold_swap32(double v) {
                    __builtin_bit_cast(double, ((unsigned long long)hi1 << 32) | lo1));
 }
 
-/* OP folded over the S = 16, 32 or 64 lanes of an aligned sub-group of the wave; every lane of
+/* OP folded over the S = 8, 16, 32 or 64 lanes of an aligned sub-group of the wave; every lane of
  * the sub-group returns the result. All 64 lanes must execute it. */
 template <class OP, int S, class P> __device__ __forceinline__ P lanes_allreduce(P v) {
-  static_assert(S == 16 || S == 32 || S == 64, "sub-groups of 16, 32 or 64 lanes");
+  static_assert(S == 8 || S == 16 || S == 32 || S == 64, "sub-groups of 8, 16, 32 or 64 lanes");
   v = OP::apply(v, dpp_move<DPP_XOR1>(v));
   v = OP::apply(v, dpp_move<DPP_XOR2>(v));
   v = OP::apply(v, dpp_move<DPP_HALF_MIRROR>(v));
-  v = OP::apply(v, dpp_move<DPP_MIRROR>(v));
+  if constexpr (S >= 16) v = OP::apply(v, dpp_move<DPP_MIRROR>(v));
   if constexpr (S >= 32) v = fold_swap16<OP>(v);
   if constexpr (S >= 64) v = fold_swap32<OP>(v);
   return v;

@@ -6,8 +6,9 @@
  * HBM once. HBM streams fastest here with many small waves each moving one or two packs, so
  * the plan takes the narrowest group that covers the row at a target NV (2 for softmax, 1 for
  * RMSNorm) and only lets NV grow once the group is 1024 threads wide:
- *   G = 16, 32         several short rows per wavefront, DPP reductions inside 16- or
- *                      32-lane parts of the wave, so rows of a few hundred bytes keep all lanes busy;
+ *   G = 8, 16, 32      several short rows per wavefront, DPP reductions inside 8-, 16- or
+ *                      32-lane parts of the wave, so rows of a few hundred bytes keep all lanes busy
+ *                      (8 lanes only for rows of at most eight packs, one pack a lane);
  *   G = 64             one wavefront per row, cross-lane (DPP / permlane-swap) reductions only;
  *   G = 128 ... 1024   per-wave partials combined through LDS with one barrier per reduction;
  *   stream             rows too long for registers: an online first pass and a second pass that
@@ -52,9 +53,12 @@ struct RowPlan {
 };
 
 /* nv_target: packs per thread the automatic plan aims for before it widens the group.
- * subwave: the kernel also comes in groups of 16 and 32 lanes (several rows per wavefront), which
- * keeps every lane busy on rows shorter than a wavefront's worth of packs. */
-inline RowPlan plan_row(size_t packs, int max_nv, int nv_target, bool subwave = false) {
+ * min_group: 64, or 16 or 8 when the kernel also comes in groups of 8, 16 and 32 lanes (several
+ * rows per wavefront), which keeps every lane busy on rows shorter than a wavefront's worth of
+ * packs. Ragged rows need 16: a group's first lanes hold one head or tail element each, and a row
+ * of two-byte values can have fourteen of them. */
+inline RowPlan plan_row(size_t packs, int max_nv, int nv_target, int min_group = WAVE) {
+  const bool subwave = min_group < WAVE;
   static const int ladder[] = {16, 32, 64, 128, 256, 512, 1024};
   constexpr int RUNGS = 7;
   int forced = row_regime_override();
@@ -62,6 +66,7 @@ inline RowPlan plan_row(size_t packs, int max_nv, int nv_target, bool subwave = 
   if (forced == REGIME_STREAM) return RowPlan{0, 0};
   const int first_rung = subwave ? 0 : 2;
   if (forced == REGIME_AUTO) {
+    if (min_group <= 8 && packs <= 8) return RowPlan{8, 1};
     const int want = nv_target < max_nv ? nv_target : max_nv;
     for (int r = first_rung; r < RUNGS; ++r) {
       const int nv = packs_per_thread(packs, ladder[r], want);
@@ -88,6 +93,7 @@ template <int MAXNV, bool SUBWAVE = false, class F> inline bool for_row_plan(con
 #define MP_PLAN_GROUP(G_) \
   MP_PLAN_CASE(G_, 1) MP_PLAN_CASE(G_, 2) MP_PLAN_CASE(G_, 4) MP_PLAN_CASE(G_, 8) MP_PLAN_CASE(G_, 16)
   if constexpr (SUBWAVE) {
+    MP_PLAN_CASE(8, 1)
     MP_PLAN_GROUP(16)
     MP_PLAN_GROUP(32)
   }

@@ -779,7 +779,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
    * nothing beats the persistent kernel below 32 packs a row. Measured on the MI355X. */
   constexpr int ONESHOT = 256;
   const int nv_target = sizeof(T) == 2 ? 2 : 1;
-  const RowPlan shot = plan_row(packs, MAXNV, nv_target, true);
+  const RowPlan shot = plan_row(packs, MAXNV, nv_target, ragged ? 16 : 8);
   const bool take_shot = row_regime_override() == REGIME_AUTO && shot.G > 0 && shot.G <= ONESHOT &&
                          (sizeof(T) != 2 || packs >= 32);
   if (take_shot) {
@@ -797,7 +797,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
       return;
     }
   }
-  const RowPlan plan = plan_row(packs, MAXNV, 1, true);
+  const RowPlan plan = plan_row(packs, MAXNV, 1, ragged ? 16 : 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
@@ -828,7 +828,7 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
                         static_cast<const void*>(dx) != static_cast<const void*>(dy);
   const int C = W > 1 && distinct ? rmsnorm_rev_cluster_size<T>(n) : 0;
   const bool force_shared = C >= 1 && row_regime_override() == REGIME_CLUSTER;
-  const RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row((n + W - 1) / W, MAXNV, 1, true);
+  const RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row((n + W - 1) / W, MAXNV, 1, 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     rows = (unsigned)(need < max_rows ? need : max_rows);

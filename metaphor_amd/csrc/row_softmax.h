@@ -678,7 +678,7 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   }
   const bool ragged = !(aligned16(x) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(64);
-  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, true);
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, ragged ? 16 : 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n);
@@ -745,7 +745,7 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   }
   const bool ragged = !(aligned16(y) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, true);
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, ragged ? 16 : 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) {
