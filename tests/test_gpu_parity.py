@@ -306,7 +306,7 @@ def test_reference_example_reductions():
 # ------------------------------------------------------------------ softmax
 
 SOFTMAX_SHAPES = [(1, 1), (3, 7), (5, 64), (4, 65), (1031, 16), (9, 256), (7, 1000), (256, 1024), (6, 2048),
-                  (3, 5000), (5, 8192), (2, 20000), (2, 50257), (1, 151936), (1030, 33)]
+                  (3, 5000), (5, 8192), (2, 20000), (2, 50257), (1, 151936), (1030, 33), (2051, 8), (515, 32)]
 
 
 def _softmax_inputs(r, m, n, dtype, masked):
@@ -509,7 +509,7 @@ def test_softmax_reverse_unaligned(dtype):
 # ------------------------------------------------------------------ RMSNorm
 
 NORM_SHAPES = [(1, 1), (3, 7), (17, 64), (1031, 16), (259, 128), (33, 256), (64, 4096), (5, 1000), (300, 1024), (3, 50257),
-               (2, 70001), (1025, 128), (40, 8192), (3, 32768), (2, 300000)]
+               (2, 70001), (1025, 128), (40, 8192), (3, 32768), (2, 300000), (2051, 8), (515, 32)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
