@@ -90,9 +90,10 @@ def elementwise(n=1 << 28):
 
 
 def matrix():
-    print("| dtype | shape | reduce_ij_i | reduce_ij_j | reduce_ij_j_scratch | broadcast_i_ij | broadcast_j_ij | "
-          "permutate | A.v | u.A |")
-    print("|---|---|---|---|---|---|---|---|---|---|")
+    # reduce_ij_j twice: through a bare stream context (no workspace) and through one made by the library
+    print("| dtype | shape | reduce_ij_i | reduce_ij_j bare | reduce_ij_j | reduce_ij_j_scratch | broadcast_i_ij | "
+          "broadcast_j_ij | permutate | A.v | u.A |")
+    print("|---|---|---|---|---|---|---|---|---|---|---|")
     kernels, _ = ffi.load()
     for dt in (torch.float32, torch.float16):
         es = torch.empty(0, dtype=dt).element_size()
@@ -108,6 +109,8 @@ def matrix():
             cells = [
                 _rate(B, _time(lambda: L("reduce_ij_i", x.data_ptr(), oi.data_ptr(), 0.0, m, n))),
                 _rate(B, _time(lambda: L("reduce_ij_j", x.data_ptr(), oj.data_ptr(), 0.0, m, n))),
+                _rate(B, _time(lambda: ffi.invoke(kernels.reduce_ij_j, W.KEY[dt], x.data_ptr(), oj.data_ptr(), 0.0, m, n,
+                                                  W.blas_ctx()))),
                 _rate(B, _time(lambda: L("reduce_ij_j_scratch", x.data_ptr(), oj.data_ptr(),
                                          sc.data_ptr() if nb else None, 0.0, m, n))),
                 _rate(B, _time(lambda: L("broadcast_i_ij", vi.data_ptr(), x.data_ptr(), 0.0, m, n))),

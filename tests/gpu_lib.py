@@ -314,6 +314,13 @@ class BlasStream:
         utils.mpStreamSynchronize(self.sc)
         utils.mpDeinitStream(self.sc)
 
+    def matrix_op(self, stem, src, dst, alpha, m, n):
+        """reduce_ij_j and its like on this stream, whose context owns a workspace."""
+        kernels, utils = lib()
+        torch.cuda.synchronize()
+        getattr(kernels, stem)[KEY[src.dtype]](src.data_ptr(), dst.data_ptr(), float(alpha), m, n, self.sc)
+        utils.mpStreamSynchronize(self.sc)
+
     def inner_product(self, form, a, b, alpha, c, beta, m, n, k):
         """form: "ij_jk_ik", "ij_kj_ik" or "ji_jk_ik"."""
         kernels, utils = lib()

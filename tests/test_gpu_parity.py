@@ -291,6 +291,26 @@ def test_column_sums_with_workspace(dtype):
     assert used > 0, "no shape took the two-stage path"
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_column_sums_on_a_library_stream(dtype):
+    """launch_reduce_ij_j has the reference's signature (no workspace): on a stream made by
+    mpInitStream it splits tall matrices through the workspace that the stream context owns."""
+    r = rng(17)
+    with G.BlasStream() as stream:
+        for (m, n) in [(3, 2), (5000, 64), (4097, 1024), (20000, 40), (1500, 1027), (70000, 256)]:
+            for alpha in (0.0, -0.5):
+                G.say(f"reduce_ij_j on a library stream dtype={dtype} shape=({m},{n}) alpha={alpha}")
+                src = G.dev(r.normal(0, 1, (m, n)), dtype)
+                dst = G.dev(r.normal(0, 1, n), dtype)
+                before = G.host(dst.t).copy()
+                stream.matrix_op("reduce_ij_j", src.t, dst.t, alpha, m, n)
+                ref = O.reduce_ij_j(G.host(src.t), before if alpha else None, alpha)
+                scale = np.abs(G.host(src.t).astype(np.float64)).sum(axis=0) + abs(alpha) * np.abs(before.astype(np.float64))
+                G.compare(dst.t, ref, dtype, f"reduce_ij_j ({m},{n}) alpha {alpha}", rowwise=False, scale=scale)
+                dst.check("column sums")
+                src.check("column sums source")
+
+
 def test_reference_example_reductions():
     # src/examples/experimental.zig:19-34
     f32 = torch.float32
