@@ -127,6 +127,11 @@ template <class P> __device__ __forceinline__ P relu_slope(P x) { return x >= (P
  * ------------------------------------------------------------------------------------- */
 
 template <class T, int W> struct vec_of { typedef T type __attribute__((ext_vector_type(W))); };
+/* The same pack behind a pointer that is only element-aligned. The hardware moves a misaligned
+ * 128-bit global access as one instruction; measured on the MI355X with a 1 GiB copy, loads shifted
+ * by 2 ... 14 bytes run at the aligned rate (6.2 TB/s) and shifted stores at 5.9. LDS accesses of
+ * this type are split by the compiler. */
+template <class T, int W> struct loose_vec_of { typedef T type __attribute__((ext_vector_type(W), aligned(sizeof(T)))); };
 
 /* Load W consecutive elements (one pack when W > 1; p must be 16-byte aligned then). */
 template <class T, int W, class P>
@@ -179,6 +184,35 @@ __device__ __forceinline__ void store_pack_nt(T* p, const P (&in)[W]) {
     for (int i = 0; i < W; ++i) v[i] = (T)in[i];
     __builtin_nontemporal_store(v, reinterpret_cast<V*>(p));
   }
+}
+
+/* The four accessors above for packs that start at any element (see loose_vec_of). */
+template <class T, int W, class P>
+__device__ __forceinline__ void load_pack_loose(const T* p, P (&out)[W]) {
+  const typename vec_of<T, W>::type v = *reinterpret_cast<const typename loose_vec_of<T, W>::type*>(p);
+#pragma unroll
+  for (int i = 0; i < W; ++i) out[i] = (P)v[i];
+}
+template <class T, int W, class P>
+__device__ __forceinline__ void load_pack_nt_loose(const T* p, P (&out)[W]) {
+  const typename vec_of<T, W>::type v =
+      __builtin_nontemporal_load(reinterpret_cast<const typename loose_vec_of<T, W>::type*>(p));
+#pragma unroll
+  for (int i = 0; i < W; ++i) out[i] = (P)v[i];
+}
+template <class T, int W, class P>
+__device__ __forceinline__ void store_pack_loose(T* p, const P (&in)[W]) {
+  typename vec_of<T, W>::type v;
+#pragma unroll
+  for (int i = 0; i < W; ++i) v[i] = (T)in[i];
+  *reinterpret_cast<typename loose_vec_of<T, W>::type*>(p) = v;
+}
+template <class T, int W, class P>
+__device__ __forceinline__ void store_pack_nt_loose(T* p, const P (&in)[W]) {
+  typename vec_of<T, W>::type v;
+#pragma unroll
+  for (int i = 0; i < W; ++i) v[i] = (T)in[i];
+  __builtin_nontemporal_store(v, reinterpret_cast<typename loose_vec_of<T, W>::type*>(p));
 }
 
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }

@@ -16,14 +16,18 @@
  * reads over the banks. r16 tiles are gathered as 32-bit words (two neighbouring columns at
  * once) and separated in registers, so a thread issues W/2 LDS reads per output pack.
  * Operands whose rows are not 16-byte aligned (an odd row length, a shifted base) keep 128-bit
- * global accesses: every row segment is peeled so that its packs are aligned in memory, and only
- * the LDS side goes element by element.
+ * accesses, global and LDS: their packs simply start at any element. A misaligned 128-byte row
+ * segment touches two cache lines, which costs this kernel more than it costs a copy (measured:
+ * 16384 x 16384 r32 with the source shifted by one element 4.9 TB/s, the destination 5.0, both
+ * 4.2; [20000, 50257] r32 3.7, r16 4.4; element-wise fallbacks reached 2.9 and 1.7 there).
  * HBM-bound: 2 * sizeof(T) bytes per element (3 when alpha != 0).
  */
 #ifndef MP_PERMUTATE_H
 #define MP_PERMUTATE_H
 
 #include "kernel_header.h"
+
+#include <type_traits>
 
 #if defined(__cplusplus) && defined(__HIPCC__)
 
@@ -41,6 +45,9 @@ __device__ __forceinline__ int tp_at(int r, int c) {
   return r * (TP_COL_PACKS * W) + (((c / W) ^ (r / W)) & (TP_COL_PACKS - 1)) * W + (c % W);
 }
 
+/* VIN / VOUT: the source / destination rows are 16-byte aligned (base and row length), so every
+ * pack is whole and aligned. Otherwise packs start at any element (see loose_vec_of), the pack that
+ * the matrix edge cuts moves element by element, and stores pay about 5 % for the misalignment. */
 template <class T, bool VIN, bool VOUT, bool BLEND>
 __global__ __launch_bounds__(tp_threads<T>()) void permutate_kernel(
     const T* __restrict__ src, T* __restrict__ dst, typename precision<T>::type alpha,
@@ -49,29 +56,46 @@ __global__ __launch_bounds__(tp_threads<T>()) void permutate_kernel(
   constexpr int W = pack_width<T>(), THREADS = tp_threads<T>(), RP = TP_ROW_PACKS, CP = TP_COL_PACKS;
   constexpr int TR = RP * W, TC = CP * W, STEPS = TR * CP / THREADS; /* packs per thread, in and out */
   using V = typename vec_of<T, W>::type;
+  using VI = typename std::conditional<VIN, V, typename loose_vec_of<T, W>::type>::type;
+  using VO = typename std::conditional<VOUT, V, typename loose_vec_of<T, W>::type>::type;
   typedef V __attribute__((may_alias)) VA;
   __shared__ __align__(16) T tile[TR * TC];
 
   const int tid = threadIdx.x;
   const size_t r0 = (size_t)(blockIdx.x % tiles_r) * TR, c0 = (size_t)(blockIdx.x / tiles_r) * TC;
 
-  if constexpr (VIN) {
+  {
     V v[STEPS];
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
+    /* a pack is loaded whole when it lies inside the matrix; every load is issued before the first
+     * is waited for: any other pack reads the first pack of the source instead and is zeroed below */
+    auto whole = [&](int s) -> bool {
       const int idx = s * THREADS + tid, r = idx / CP, p = idx % CP;
-      /* every load is issued before the first is waited for: a pack outside the matrix reads the
-       * first pack of the source instead and is zeroed below */
-      const bool inside = r0 + r < rows && c0 + (size_t)p * W < cols;
-      const T* from = inside ? src + (r0 + r) * cols + c0 + (size_t)p * W : src;
-      v[s] = __builtin_nontemporal_load(reinterpret_cast<const V*>(from));
+      return r0 + r < rows && c0 + (size_t)p * W + W <= cols;
+    };
+    if (VIN || cols >= (size_t)W) { /* uniform: a source narrower than a pack has no first pack */
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        const int idx = s * THREADS + tid, r = idx / CP, p = idx % CP;
+        const T* from = whole(s) ? src + (r0 + r) * cols + c0 + (size_t)p * W : src;
+        v[s] = __builtin_nontemporal_load(reinterpret_cast<const VI*>(from));
+      }
     }
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
-      const int idx = s * THREADS + tid, r = idx / CP, p = idx % CP;
-      if (!(r0 + r < rows && c0 + (size_t)p * W < cols)) {
+      if (!whole(s)) {
 #pragma unroll
         for (int i = 0; i < W; ++i) v[s][i] = (T)0;
+        if constexpr (!VIN) { /* the pack that the right edge cuts */
+          const int idx = s * THREADS + tid, r = idx / CP, p = idx % CP;
+          if (r0 + r < rows) {
+            const T* row = src + (r0 + r) * cols;
+#pragma unroll
+            for (int i = 0; i < W; ++i) {
+              const size_t c = c0 + (size_t)p * W + i;
+              if (c < cols) v[s][i] = row[c];
+            }
+          }
+        }
       }
     }
 #pragma unroll
@@ -79,140 +103,93 @@ __global__ __launch_bounds__(tp_threads<T>()) void permutate_kernel(
       const int idx = s * THREADS + tid, r = idx / CP, p = idx % CP;
       *reinterpret_cast<VA*>(&tile[r * TC + ((p ^ (r / W)) & (CP - 1)) * W]) = v[s];
     }
-  } else {
-    /* Source rows whose length or base breaks the 16-byte alignment: each row's 128-byte segment
-     * is peeled into [head scalars][packs aligned in MEMORY][tail scalars]; head and tail together
-     * are exactly one pack's worth of elements, so the CP slots of a row still move W elements
-     * each: CP - 1 aligned packs and one slot of scalars. A segment cut short by the matrix edge
-     * is read element by element. Everything lands in LDS element by element. */
-    const int len = cols - c0 < (size_t)TC ? (int)(cols - c0) : TC; /* uniform over the workgroup */
-    T v[STEPS][W];
-    /* tile column of element i of slot q of a row whose head is h elements long, -1: none */
-    auto column = [&](int q, int h, int i) -> int {
-      if (len != TC) return q * W + i < len ? q * W + i : -1;
-      if (q < CP - (h ? 1 : 0)) return h + q * W + i;
-      return i < h ? i : TC - W + i; /* the last slot of a misaligned row: its head and its tail */
-    };
-    auto head = [&](int r) -> int {
-      const T* seg = src + (r0 + r) * cols + c0;
-      return (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(seg) & 15u)) & 15u) / sizeof(T));
-    };
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int idx = s * THREADS + tid, r = idx / CP, q = idx % CP;
-#pragma unroll
-      for (int i = 0; i < W; ++i) v[s][i] = (T)0;
-      if (r0 + r < rows) {
-        const T* seg = src + (r0 + r) * cols + c0;
-        const int h = head(r);
-        if (len == TC && q < CP - (h ? 1 : 0)) {
-          const V pack = __builtin_nontemporal_load(reinterpret_cast<const V*>(seg + h + q * W));
-#pragma unroll
-          for (int i = 0; i < W; ++i) v[s][i] = pack[i];
-        } else {
-#pragma unroll
-          for (int i = 0; i < W; ++i) {
-            const int c = column(q, h, i);
-            if (c >= 0) v[s][i] = seg[c];
-          }
-        }
-      }
-    }
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s) {
-      const int idx = s * THREADS + tid, r = idx / CP, q = idx % CP;
-      if (r0 + r < rows) {
-        const int h = head(r);
-#pragma unroll
-        for (int i = 0; i < W; ++i) {
-          const int c = column(q, h, i);
-          if (c >= 0) tile[tp_at<W>(r, c)] = v[s][i];
-        }
-      }
-    }
   }
   __syncthreads();
 
-  /* Output element (j, i) of the tile is source element (i, j). */
-  if constexpr (VOUT) {
-    /* Gather every output pack from LDS first (always inside the tile), then fetch the old
-     * values when blending, then store: no step waits for the one before it. */
-    V out[STEPS];
-    size_t at[STEPS]; /* element offset of each output pack in dst, or npos outside the matrix */
-    constexpr size_t npos = ~(size_t)0;
+  /* Output element (j, i) of the tile is source element (i, j). Gather every output pack from LDS
+   * first (always inside the tile), then fetch the old values when blending, then store: no step
+   * waits for the one before it. */
+  V out[STEPS];
+  size_t at[STEPS]; /* element offset in dst of each output pack that is stored whole, else npos */
+  constexpr size_t npos = ~(size_t)0;
+  /* output pack s of this thread: destination row j, first column i (r16: the packs 2s and 2s + 1
+   * are neighbouring destination rows, gathered together) */
+  auto where = [&](int s, size_t& i, size_t& j) {
     if constexpr (sizeof(T) == 2) {
-      /* Two output rows (source columns 2*jp and 2*jp + 1) per step: 32-bit words hold both. */
-#pragma unroll
-      for (int s = 0; s < STEPS / 2; ++s) {
-        const int idx = s * THREADS + tid, jp = idx / RP, ip = idx % RP;
-        unsigned w[W];
-#pragma unroll
-        for (int e = 0; e < W; ++e) w[e] = *reinterpret_cast<const tp_word*>(&tile[tp_at<W>(ip * W + e, 2 * jp)]);
-        typedef unsigned words_t __attribute__((ext_vector_type(W / 2)));
-        words_t lo, hi;
-#pragma unroll
-        for (int e = 0; e < W / 2; ++e) {
-          lo[e] = (w[2 * e] & 0xffffu) | (w[2 * e + 1] << 16);
-          hi[e] = (w[2 * e] >> 16) | (w[2 * e + 1] & 0xffff0000u);
-        }
-        out[2 * s] = __builtin_bit_cast(V, lo);
-        out[2 * s + 1] = __builtin_bit_cast(V, hi);
-        const size_t i = r0 + (size_t)ip * W, j = c0 + 2 * jp;
-        at[2 * s] = (j < cols && i < rows) ? j * rows + i : npos;
-        at[2 * s + 1] = (j + 1 < cols && i < rows) ? (j + 1) * rows + i : npos;
-      }
+      const int idx = (s / 2) * THREADS + tid;
+      j = c0 + 2 * (idx / RP) + (s & 1);
+      i = r0 + (size_t)(idx % RP) * W;
     } else {
+      const int idx = s * THREADS + tid;
+      j = c0 + idx / RP;
+      i = r0 + (size_t)(idx % RP) * W;
+    }
+  };
+  if constexpr (sizeof(T) == 2) {
+    /* Two output rows (source columns 2*jp and 2*jp + 1) per step: 32-bit words hold both. */
 #pragma unroll
-      for (int s = 0; s < STEPS; ++s) {
-        const int idx = s * THREADS + tid, j = idx / RP, ip = idx % RP;
+    for (int s = 0; s < STEPS / 2; ++s) {
+      const int idx = s * THREADS + tid, jp = idx / RP, ip = idx % RP;
+      unsigned w[W];
 #pragma unroll
-        for (int e = 0; e < W; ++e) out[s][e] = tile[tp_at<W>(ip * W + e, j)];
-        const size_t i = r0 + (size_t)ip * W, jj = c0 + j;
-        at[s] = (jj < cols && i < rows) ? jj * rows + i : npos;
+      for (int e = 0; e < W; ++e) w[e] = *reinterpret_cast<const tp_word*>(&tile[tp_at<W>(ip * W + e, 2 * jp)]);
+      typedef unsigned words_t __attribute__((ext_vector_type(W / 2)));
+      words_t lo, hi;
+#pragma unroll
+      for (int e = 0; e < W / 2; ++e) {
+        lo[e] = (w[2 * e] & 0xffffu) | (w[2 * e + 1] << 16);
+        hi[e] = (w[2 * e] >> 16) | (w[2 * e + 1] & 0xffff0000u);
       }
+      out[2 * s] = __builtin_bit_cast(V, lo);
+      out[2 * s + 1] = __builtin_bit_cast(V, hi);
     }
-    if constexpr (BLEND) {
-      V old[STEPS];
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s) old[s] = *reinterpret_cast<const V*>(dst + (at[s] != npos ? at[s] : 0));
-#pragma unroll
-      for (int s = 0; s < STEPS; ++s)
-#pragma unroll
-        for (int e = 0; e < W; ++e) out[s][e] = (T)((P)out[s][e] + alpha * (P)old[s][e]);
-    }
-#pragma unroll
-    for (int s = 0; s < STEPS; ++s)
-      if (at[s] != npos) __builtin_nontemporal_store(out[s], reinterpret_cast<V*>(dst + at[s]));
   } else {
-    /* Destination rows that break the alignment: the same peeling on the way out. The LDS gather
-     * is element by element in any case, so a pack may start at any row of the tile. */
-    const int len = rows - r0 < (size_t)TR ? (int)(rows - r0) : TR;
 #pragma unroll
     for (int s = 0; s < STEPS; ++s) {
-      const int idx = s * THREADS + tid, j = idx / RP, q = idx % RP;
-      if (c0 + j >= cols) continue;
-      T* seg = dst + (c0 + j) * rows + r0;
-      const int h = (int)(((16u - (unsigned)(reinterpret_cast<uintptr_t>(seg) & 15u)) & 15u) / sizeof(T));
-      if (len == TR && q < RP - (h ? 1 : 0)) {
-        const int i0 = h + q * W;
-        V out;
+      const int idx = s * THREADS + tid, j = idx / RP, ip = idx % RP;
 #pragma unroll
-        for (int e = 0; e < W; ++e) out[e] = tile[tp_at<W>(i0 + e, j)];
-        if constexpr (BLEND) {
-          const V old = *reinterpret_cast<const V*>(seg + i0);
+      for (int e = 0; e < W; ++e) out[s][e] = tile[tp_at<W>(ip * W + e, j)];
+    }
+  }
 #pragma unroll
-          for (int e = 0; e < W; ++e) out[e] = (T)((P)out[e] + alpha * (P)old[e]);
+  for (int s = 0; s < STEPS; ++s) {
+    size_t i, j;
+    where(s, i, j);
+    at[s] = j < cols && i + W <= rows ? j * rows + i : npos;
+  }
+  if constexpr (BLEND) {
+    if (VOUT || rows >= (size_t)W) { /* uniform: a destination narrower than a pack has no first pack */
+      V old[STEPS];
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) old[s] = *reinterpret_cast<const VO*>(dst + (at[s] != npos ? at[s] : 0));
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s)
+        if (at[s] != npos) {
+#pragma unroll
+          for (int e = 0; e < W; ++e) out[s][e] = (T)((P)out[s][e] + alpha * (P)old[s][e]);
         }
-        __builtin_nontemporal_store(out, reinterpret_cast<V*>(seg + i0));
-      } else {
+    }
+  }
 #pragma unroll
-        for (int e = 0; e < W; ++e) {
-          const int i = len == TR ? (e < h ? e : TR - W + e) : q * W + e;
-          if (i < len) {
-            T x = tile[tp_at<W>(i, j)];
-            if constexpr (BLEND) x = (T)((P)x + alpha * (P)seg[i]);
-            seg[i] = x;
-          }
+  for (int s = 0; s < STEPS; ++s)
+    if (at[s] != npos) __builtin_nontemporal_store(out[s], reinterpret_cast<VO*>(dst + at[s]));
+  if constexpr (!VOUT) {
+    /* the pack of each destination row that the bottom edge cuts: only in the last tile of a band */
+    if (rows - r0 < (size_t)TR && rows % W != 0) {
+#pragma unroll
+      for (int s = 0; s < STEPS; ++s) {
+        size_t i, j;
+        where(s, i, j);
+        if (j < cols && i < rows && i + W > rows) {
+          T* to = dst + j * rows + i;
+          const int left = (int)(rows - i);
+#pragma unroll
+          for (int e = 0; e < W; ++e)
+            if (e < left) {
+              T x = out[s][e];
+              if constexpr (BLEND) x = (T)((P)x + alpha * (P)to[e]);
+              to[e] = x;
+            }
         }
       }
     }
