@@ -44,30 +44,51 @@ __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
   const T* vbody = vec + g.head; /* DOT only: the vector entries of the packed columns */
   const bool vec_packed = DOT && (reinterpret_cast<uintptr_t>(vbody) & 15u) == 0;
   P s = (P)0;
-  for (int p0 = lane; p0 < g.nvec; p0 += G * U) {
-    P buf[U][W], wv[U][W];
+  if constexpr (DOT && sizeof(T) == 2) {
+    /* v_dot2_f32_f16 on the packs as loaded: two exact half products added to an fp32 sum per
+     * instruction, instead of two conversions and a multiply-add per element */
+    using V = typename vec_of<T, W>::type;
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    for (int p0 = lane; p0 < g.nvec; p0 += G * U) {
+      V a[U], b[U];
 #pragma unroll
-    for (int u = 0; u < U; ++u) {
-      const int p = p0 + u * G;
-      if (p < g.nvec) {
-        load_pack_nt<T, W>(body + (size_t)p * W, buf[u]);
-        if constexpr (DOT) {
-          if (vec_packed) {
-            load_pack<T, W>(vbody + (size_t)p * W, wv[u]);
-          } else {
-#pragma unroll
-            for (int i = 0; i < W; ++i) wv[u][i] = (P)vbody[(size_t)p * W + i];
-          }
+      for (int u = 0; u < U; ++u) {
+        const int p = p0 + u * G;
+        if (p < g.nvec) {
+          a[u] = __builtin_nontemporal_load(reinterpret_cast<const V*>(body + (size_t)p * W));
+          b[u] = *reinterpret_cast<const typename loose_vec_of<T, W>::type*>(vbody + (size_t)p * W);
+        } else {
+          a[u] = b[u] = V{};
         }
-      } else {
-#pragma unroll
-        for (int i = 0; i < W; ++i) buf[u][i] = wv[u][i] = (P)0;
       }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < W; i += 2)
+          s = __builtin_amdgcn_fdot2(half2_t{a[u][i], a[u][i + 1]}, half2_t{b[u][i], b[u][i + 1]}, s, false);
     }
+  } else {
+    for (int p0 = lane; p0 < g.nvec; p0 += G * U) {
+      P buf[U][W], wv[U][W];
 #pragma unroll
-    for (int u = 0; u < U; ++u)
+      for (int u = 0; u < U; ++u) {
+        const int p = p0 + u * G;
+        if (p < g.nvec) {
+          load_pack_nt<T, W>(body + (size_t)p * W, buf[u]);
+          if constexpr (DOT) {
+            if (vec_packed) load_pack<T, W>(vbody + (size_t)p * W, wv[u]);
+            else load_pack_loose<T, W>(vbody + (size_t)p * W, wv[u]); /* the row's packs are aligned, the vector's not */
+          }
+        } else {
 #pragma unroll
-      for (int i = 0; i < W; ++i) s += DOT ? buf[u][i] * wv[u][i] : buf[u][i];
+          for (int i = 0; i < W; ++i) buf[u][i] = wv[u][i] = (P)0;
+        }
+      }
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int i = 0; i < W; ++i) s += DOT ? buf[u][i] * wv[u][i] : buf[u][i];
+    }
   }
   if (W > 1) {
     size_t e = (size_t)-1;
@@ -116,8 +137,10 @@ inline void reduce_rows(const T* src, T* dst, double alpha, size_t m, size_t n, 
  * the result does not depend on scheduling. The sums go to `out + blockIdx.y * n`: the destination
  * itself (O = T, one chunk holding every row, alpha blend) or a partial row of accumulators
  * (O = precision<T>, no blend) that sum_partial_rows adds up afterwards. WEIGHTED: row r counts
- * weight[r] times (a vector-matrix product). */
-template <class T, class O, int CW, int LANES, int SLICES, bool WEIGHTED>
+ * weight[r] times (a vector-matrix product). LOOSE: rows that are not 16-byte aligned (an odd row
+ * length, a shifted base); the packs then start at any element, which a streaming read does not
+ * feel, and the pack that the end of the row cuts is read element by element. */
+template <class T, class O, int CW, int LANES, int SLICES, bool WEIGHTED, bool LOOSE>
 __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
     const T* src, const T* weight, O* out, typename precision<T>::type scale, typename precision<T>::type blend,
     size_t m, size_t n, size_t chunk) {
@@ -130,13 +153,25 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
   P s[CW];
 #pragma unroll
   for (int i = 0; i < CW; ++i) s[i] = (P)0;
+  const bool whole = col + CW <= n;
+  auto fetch = [&](size_t row, P(&v)[CW]) {
+    const T* p = src + row * n + col;
+    if constexpr (!LOOSE) {
+      load_pack_nt<T, CW>(p, v);
+    } else if (whole) {
+      load_pack_nt_loose<T, CW>(p, v);
+    } else {
+#pragma unroll
+      for (int i = 0; i < CW; ++i) v[i] = col + i < n ? (P)p[i] : (P)0;
+    }
+  };
   if (col < n) {
     size_t r = begin + slice;
     for (; r + 3 * SLICES < end; r += 4 * SLICES) {
       P v[4][CW], w[4];
 #pragma unroll
       for (int u = 0; u < 4; ++u) {
-        load_pack_nt<T, CW>(src + (r + (size_t)u * SLICES) * n + col, v[u]);
+        fetch(r + (size_t)u * SLICES, v[u]);
         w[u] = WEIGHTED ? (P)weight[r + (size_t)u * SLICES] : (P)1;
       }
 #pragma unroll
@@ -146,7 +181,7 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
     }
     for (; r < end; r += SLICES) {
       P v[CW];
-      load_pack_nt<T, CW>(src + r * n + col, v);
+      fetch(r, v);
       const P w = WEIGHTED ? (P)weight[r] : (P)1;
 #pragma unroll
       for (int i = 0; i < CW; ++i) s[i] += WEIGHTED ? w * v[i] : v[i];
@@ -169,9 +204,10 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
  * rows; 1 when the strips alone are enough or the matrix is short. */
 template <class T> inline size_t reduce_cols_chunks(size_t m, size_t n) {
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  const size_t strips = (n / W + 7) / 8 ? (n / W + 7) / 8 : 1;
+  const size_t lanes = n % W == 0 ? 8 : 64; /* as reduce_cols picks them (a shifted base aside) */
+  const size_t strips = ((n + W - 1) / W + lanes - 1) / lanes;
   const size_t want = (size_t)compute_units() * 4;
-  if (strips >= want || n % W != 0) return 1;
+  if (strips >= want) return 1;
   size_t chunks = (want + strips - 1) / strips;
   const size_t most = m / 512;
   if (chunks > most) chunks = most;
@@ -193,33 +229,37 @@ inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, do
   if (n == 0) return;
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  const bool packed = aligned16(src) && (n % W) == 0;
-#define MP_COLS(O_, CW_, L_, S_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)                                                        \
+  const bool loose = !(aligned16(src) && (n % W) == 0);
+#define MP_COLS_AS(O_, LANES_, LOOSE_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)                                                     \
   do {                                                                                                                       \
-    if (weight) reduce_cols_kernel<T, O_, CW_, L_, S_, true><<<GRID_, dim3(1024), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_); \
-    else reduce_cols_kernel<T, O_, CW_, L_, S_, false><<<GRID_, dim3(1024), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_);       \
+    if (weight) reduce_cols_kernel<T, O_, W, LANES_, 1024 / LANES_, true, LOOSE_><<<GRID_, dim3(1024), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_); \
+    else reduce_cols_kernel<T, O_, W, LANES_, 1024 / LANES_, false, LOOSE_><<<GRID_, dim3(1024), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_);       \
   } while (0)
-  if (packed) { /* 8 lanes x one pack = 128 bytes of every row per workgroup */
-    const size_t blocks = (n / W + 7) / 8;
-    require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
-    size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;
-    const size_t fit = scratch_bytes / (n * sizeof(P)); /* partial rows the workspace holds */
-    if (chunks > fit) chunks = fit;
-    if (chunks > 1) {
-      const size_t chunk = (m + chunks - 1) / chunks;
-      P* partials = static_cast<P*>(scratch);
-      MP_COLS(P, W, 8, 128, dim3((unsigned)blocks, (unsigned)chunks), partials, (P)scale, (P)0, chunk);
-      MP_CHECK_LAUNCH();
-      sum_partial_rows<T>(partials, dst, blend, (unsigned)chunks, n, stream);
-      return;
-    }
-    MP_COLS(T, W, 8, 128, dim3((unsigned)blocks), dst, (P)scale, (P)blend, m);
-  } else {
-    /* rows that are not pack-aligned: one element per lane, a wavefront per 64-element row segment */
-    const size_t blocks = (n + 63) / 64;
-    require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
-    MP_COLS(T, 1, 64, 16, dim3((unsigned)blocks), dst, (P)scale, (P)blend, m);
+#define MP_COLS(O_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)                              \
+  do {                                                                              \
+    if (loose) MP_COLS_AS(O_, 64, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);       \
+    else MP_COLS_AS(O_, 8, false, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);             \
+  } while (0)
+  /* aligned rows: 8 lanes x one pack = 128 bytes, one cache line, of every row per workgroup (many
+   * strips, so narrow matrices still spread); rows that are not: a wavefront per kilobyte of a
+   * row, because a misaligned 128-byte segment would touch two lines for the data of one
+   * (measured on r32 [20000, 50257]: 3.4 TB/s with 8 lanes, one element per lane 4.3) */
+  const size_t lanes = loose ? 64 : 8;
+  const size_t blocks = ((n + W - 1) / W + lanes - 1) / lanes;
+  require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
+  size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;
+  const size_t fit = scratch_bytes / (n * sizeof(P)); /* partial rows the workspace holds */
+  if (chunks > fit) chunks = fit;
+  if (chunks > 1) {
+    const size_t chunk = (m + chunks - 1) / chunks;
+    P* partials = static_cast<P*>(scratch);
+    MP_COLS(P, dim3((unsigned)blocks, (unsigned)chunks), partials, (P)scale, (P)0, chunk);
+    MP_CHECK_LAUNCH();
+    sum_partial_rows<T>(partials, dst, blend, (unsigned)chunks, n, stream);
+    return;
   }
+  MP_COLS(T, dim3((unsigned)blocks), dst, (P)scale, (P)blend, m);
+#undef MP_COLS_AS
 #undef MP_COLS
   MP_CHECK_LAUNCH();
 }
@@ -329,13 +369,15 @@ __global__ __launch_bounds__(256) void broadcast_kernel(
   }
 }
 
-/* The destination as one flat array of m*n elements behind a 16-byte aligned base: one pack per
- * thread in one-shot 256-thread workgroups, the shape that writes fastest on this GPU, whatever
- * the row length (short rows keep every lane busy). ALIGNED: n % W == 0, so a pack lies inside
- * one row and the column values are one pack load; otherwise a pack may end in the next row
- * (n >= W, so in at most one) and its values are gathered one by one. The last workgroup also
- * writes the m*n % W elements behind the last whole pack. */
-template <class T, int W, bool BY_ROW, bool BLEND, bool ALIGNED>
+/* The destination as one flat array of m*n elements: one pack per thread in one-shot 256-thread
+ * workgroups, the shape that writes fastest on this GPU, whatever the row length (short rows keep
+ * every lane busy). ALIGNED: n % W == 0 and 16-byte aligned column values, so a pack lies inside
+ * one row and its values are one aligned pack load; otherwise a pack may end in the next row
+ * (n >= W, so in at most one): the column values are then a pack that starts at any element, or,
+ * for the one pack per row that wraps, W single loads. DALIGNED: the destination base is 16-byte
+ * aligned; a destination that is not costs about 5 % (packs that start at any element). The last
+ * workgroup also writes the m*n % W elements behind the last whole pack. */
+template <class T, int W, bool BY_ROW, bool BLEND, bool ALIGNED, bool DALIGNED>
 __global__ __launch_bounds__(256) void broadcast_flat_kernel(
     const T* src, T* dst, typename precision<T>::type alpha, size_t total, unsigned n) {
   using P = typename precision<T>::type;
@@ -344,46 +386,38 @@ __global__ __launch_bounds__(256) void broadcast_flat_kernel(
   const size_t row0 = base / n;                     /* one 64-bit division is scalar work */
   const unsigned off = (unsigned)(base - row0 * n) + threadIdx.x * W;
   const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
-  /* ragged column values: the workgroup's 256 * W consecutive elements need a window of 256 * W
-   * consecutive (wrapping) entries of src; it is fetched with coalesced element loads into LDS once
-   * instead of W scattered loads per thread */
-  __shared__ T window[(!ALIGNED && !BY_ROW) ? 256 * W : 1];
-  if constexpr (!ALIGNED && !BY_ROW) {
-    const unsigned first = (unsigned)(base - row0 * n); /* column of the workgroup's first element */
-#pragma unroll
-    for (int i = 0; i < W; ++i) {
-      const unsigned t = threadIdx.x + 256u * i;
-      window[t] = src[(first + t) % n];
-    }
-    __syncthreads();
-  }
   if (idx < packs) {
     const size_t row = row0 + off / n;
     const unsigned col = off % n;
     P out[W];
-    if constexpr (ALIGNED) {
-      if constexpr (BY_ROW) {
-        const P v = (P)src[row];
+    if constexpr (BY_ROW) {
+      const P here = (P)src[row];
+      if constexpr (ALIGNED) {
 #pragma unroll
-        for (int i = 0; i < W; ++i) out[i] = v;
+        for (int i = 0; i < W; ++i) out[i] = here;
       } else {
-        load_pack<T, W>(src + col, out);
+        const P there = col + W > n ? (P)src[row + 1] : here; /* a wrapping pack is never in the last row */
+#pragma unroll
+        for (int i = 0; i < W; ++i) out[i] = col + i >= n ? there : here;
       }
+    } else if constexpr (ALIGNED) {
+      load_pack<T, W>(src + col, out);
+    } else if (col + W <= n) {
+      load_pack_loose<T, W>(src + col, out);
     } else {
 #pragma unroll
-      for (int i = 0; i < W; ++i) {
-        const bool next = col + i >= n;
-        out[i] = BY_ROW ? (P)src[row + (next ? 1 : 0)] : (P)window[threadIdx.x * W + i];
-      }
+      for (int i = 0; i < W; ++i) out[i] = (P)src[col + i >= n ? col + i - n : col + i];
     }
     T* o = dst + idx * W;
     if constexpr (BLEND) {
       P old[W];
-      load_pack_nt<T, W>(o, old);
+      if constexpr (DALIGNED) load_pack_nt<T, W>(o, old);
+      else load_pack_nt_loose<T, W>(o, old);
 #pragma unroll
       for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
     }
-    store_pack_nt<T, W>(o, out);
+    if constexpr (DALIGNED) store_pack_nt<T, W>(o, out);
+    else store_pack_nt_loose<T, W>(o, out);
   }
   if (W > 1 && blockIdx.x == gridDim.x - 1) {
     const size_t e = packs * W + threadIdx.x;
@@ -401,20 +435,24 @@ inline void broadcast(const T* src, T* dst, double alpha, size_t m, size_t n, hi
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "broadcast: row length must not exceed 2^30");
-  if (aligned16(dst) && n >= (size_t)W) {
+  if (n >= (size_t)W) {
     const size_t total = m * n, blocks = (total / W + 255) / 256 + 1; /* + 1: the tail always has a workgroup */
     require(blocks < 0x7fffffffull, "broadcast: too many elements for one grid");
     const dim3 grid((unsigned)blocks), block(256);
     const bool aligned = n % W == 0 && (BY_ROW || aligned16(src));
     const bool blend = alpha != 0.0;
+#define MP_FLAT_AS(BLEND_, ALIGNED_, DALIGNED_) \
+  broadcast_flat_kernel<T, W, BY_ROW, BLEND_, ALIGNED_, DALIGNED_><<<grid, block, 0, stream>>>(src, dst, (P)alpha, total, (unsigned)n)
 #define MP_FLAT(BLEND_, ALIGNED_) \
-  broadcast_flat_kernel<T, W, BY_ROW, BLEND_, ALIGNED_><<<grid, block, 0, stream>>>(src, dst, (P)alpha, total, (unsigned)n)
+  do { if (aligned16(dst)) MP_FLAT_AS(BLEND_, ALIGNED_, true); else MP_FLAT_AS(BLEND_, ALIGNED_, false); } while (0)
     if (aligned) { if (blend) MP_FLAT(true, true); else MP_FLAT(false, true); }
     else { if (blend) MP_FLAT(true, false); else MP_FLAT(false, false); }
 #undef MP_FLAT
+#undef MP_FLAT_AS
     MP_CHECK_LAUNCH();
     return;
   }
+  /* rows shorter than a pack */
   const size_t cap = (size_t)compute_units() * 8;
   const dim3 grid((unsigned)(m < cap ? m : cap)), block(256);
   if (alpha != 0.0) broadcast_kernel<T, W, BY_ROW, true><<<grid, block, 0, stream>>>(src, dst, (P)alpha, m, n);
