@@ -511,15 +511,20 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
  * (rows slice, slice + S, ...): each keeps the dg sums of its chunk in registers for the whole
  * kernel and, per row, its chunk of x, dy and (from L2) the gain; the two row sums (x^2 and dy*g*x) are
  * exchanged through scratch once per row, so x and dy are read once. All S * C workgroups fit the
- * GPU at once (one per CU: the kernel may use 128 registers a thread), which keeps the per-row waits short; a workgroup that stops waiting
+ * GPU at once (one or two per CU, see norm_rev_cluster_per_cu), which keeps the per-row waits short; a workgroup that stops waiting
  * reads the whole row for the sums, so the kernel ends under any scheduling. Not taken when dx
  * overwrites x or dy. One partial row of dg per slice. */
-/* packs of x, dy (and, per row, gain) per thread, in the storage type; the dg sums beside them are
- * wider for r16 (eight fp32 a pack), which leaves room for two */
-template <class T> constexpr int norm_rev_cluster_nv() { return sizeof(T) == 2 ? 2 : 4; }
+/* Two packs of x, dy and (per row) gain per thread, in the storage type, and the dg sums beside
+ * them. Four-byte and wider types then fit 64 registers with a small spill, which lets two
+ * workgroups share a CU; measured on r32 against four packs and one workgroup per CU:
+ * n = 32768 4.5 -> 5.5 TB/s, 65536 4.2 -> 5.4, 131072 4.6 -> 5.0. The dg sums of r16 are four
+ * times as wide as its packs: it spills heavily at 64 registers (3.1 TB/s) and keeps one
+ * workgroup per CU and 128 registers (4.5). */
+template <class T> constexpr int norm_rev_cluster_nv() { return 2; }
+template <class T> constexpr int norm_rev_cluster_per_cu() { return sizeof(T) == 2 ? 1 : 2; }
 
 template <class T, int W, bool BLEND>
-__global__ __launch_bounds__(CLUSTER_THREADS, 4) void rmsnorm_rev_cluster(
+__global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) void rmsnorm_rev_cluster(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha,
     typename slot_word<typename precision<T>::type>::type* slots,
@@ -840,7 +845,7 @@ inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* 
   if constexpr (W > 1) {
     if (!resident && C >= 1) {
       using Word = typename slot_word<P>::type;
-      size_t S = (size_t)compute_units() / (size_t)C; /* every workgroup resident at once: one per CU (up to 128 registers a thread) */
+      size_t S = (size_t)compute_units() * norm_rev_cluster_per_cu<T>() / (size_t)C; /* every workgroup resident at once */
       if (S > m) S = m;
       if (S == 0) S = 1;
       rows = (unsigned)S;
