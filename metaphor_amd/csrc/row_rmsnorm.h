@@ -20,6 +20,8 @@
 
 #include "row_cluster.h"
 
+#include <type_traits>
+
 #if defined(__cplusplus) && defined(__HIPCC__)
 
 namespace mp {
@@ -287,10 +289,57 @@ template <class T> inline size_t rmsnorm_scratch_bytes(size_t m, size_t n) {
 
 /* ------------------------------------------------------------------ resident reverse */
 
-/* Rows must be pack-aligned (n % W == 0, every base 16-byte aligned) or W must be 1, so that
- * a thread owns the same columns in every row and can keep their dg sums in registers.
- * partials holds gridDim.x rows of n values of precision<T>. */
-template <class T, int W, int G, int NV, bool BLEND>
+/* A row of the reverse kernels as packs counted from its first element: npk = ceil(n / W) packs,
+ * the last of which holds `last` elements (W when n is a multiple of W). A thread owns the same
+ * columns in every row and keeps their dg sums in registers, whatever the alignment:
+ * LOOSE = false: every operand 16-byte aligned and n % W == 0, so every pack is whole and aligned;
+ * LOOSE = true: packs start at any element (see loose_vec_of; free for these streaming reads,
+ * about 5 % on the stores) and the cut pack of a row moves element by element, zero-filled. */
+template <class T, int W, bool LOOSE> struct RowPacks {
+  using P = typename precision<T>::type;
+  using V = typename vec_of<T, W>::type;
+  using VL = typename std::conditional<LOOSE, typename loose_vec_of<T, W>::type, V>::type;
+  int npk, last;
+  __device__ __forceinline__ explicit RowPacks(size_t n)
+      : npk(LOOSE ? (int)((n + W - 1) / W) : (int)(n / W)),
+        last(LOOSE ? (int)(n - (size_t)((int)((n + W - 1) / W) - 1) * W) : W) {}
+  /* elements of pack p that exist (p < npk) */
+  __device__ __forceinline__ int valid(int p) const { return LOOSE && p == npk - 1 ? last : W; }
+  /* pack p < npk of the row at `row`, in the storage type */
+  template <bool NT> __device__ __forceinline__ V raw(const T* row, int p) const {
+    const T* at = row + (size_t)(unsigned)p * W;
+    if (!LOOSE || valid(p) == W) {
+      if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const VL*>(at));
+      else return *reinterpret_cast<const VL*>(at);
+    }
+    V v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) v[i] = i < last ? at[i] : (T)0;
+    return v;
+  }
+  template <bool NT> __device__ __forceinline__ void load(const T* row, int p, P (&out)[W]) const {
+    const V v = raw<NT>(row, p);
+#pragma unroll
+    for (int i = 0; i < W; ++i) out[i] = (P)v[i];
+  }
+  __device__ __forceinline__ void store(T* row, int p, const P (&in)[W]) const {
+    T* at = row + (size_t)(unsigned)p * W;
+    if (!LOOSE || valid(p) == W) {
+      V v;
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[i] = (T)in[i];
+      __builtin_nontemporal_store(v, reinterpret_cast<VL*>(at));
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i)
+        if (i < last) at[i] = (T)in[i];
+    }
+  }
+};
+
+
+/* partials holds gridDim.x rows of n values of precision<T>. */
+template <class T, int W, int G, int NV, bool BLEND, bool LOOSE>
 __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
@@ -300,7 +349,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
   __shared__ P comb[RPB > 1 ? NORM_BLOCK * NV * W : 1]; /* one row of dg sums per group of the workgroup */
 
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
-  const int nvec = (int)(n / W);
+  const RowPacks<T, W, LOOSE> rp(n);
 
   P gv[NV][W], acc[NV][W];
 #pragma unroll
@@ -308,7 +357,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
     const int p = k * G + lane;
 #pragma unroll
     for (int i = 0; i < W; ++i) acc[k][i] = gv[k][i] = (P)0;
-    if (p < nvec) load_pack<T, W>(gain + (size_t)p * W, gv[k]);
+    if (p < rp.npk) rp.template load<false>(gain, p, gv[k]);
   }
 
   int parity = 0;
@@ -321,9 +370,9 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = k * G + lane;
-      if (live && p < nvec) {
-        load_pack_nt<T, W>(x + off + (size_t)p * W, xv[k]);
-        load_pack_nt<T, W>(dy + off + (size_t)p * W, dv[k]);
+      if (live && p < rp.npk) {
+        rp.template load<true>(x + off, p, xv[k]);
+        rp.template load<true>(dy + off, p, dv[k]);
       } else {
 #pragma unroll
         for (int i = 0; i < W; ++i) xv[k][i] = dv[k][i] = (P)0;
@@ -346,7 +395,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
 #pragma unroll
       for (int k = 0; k < NV; ++k) {
         const int p = k * G + lane;
-        if (p < nvec) {
+        if (p < rp.npk) {
           P out[W];
 #pragma unroll
           for (int i = 0; i < W; ++i) {
@@ -355,11 +404,11 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
           }
           if constexpr (BLEND) {
             P old[W];
-            load_pack<T, W>(dx + off + (size_t)p * W, old);
+            rp.template load<false>(dx + off, p, old);
 #pragma unroll
             for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
           }
-          store_pack_nt<T, W>(dx + off + (size_t)p * W, out);
+          rp.store(dx + off, p, out);
         }
       }
     }
@@ -367,7 +416,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
      * workgroup drift apart and its contiguous 16 KiB bursts dissolve into scattered kilobytes
      * (measured: r32 n = 256 5.3 TB/s without, 5.9 with). Rows that leave lanes idle are the exception. */
     if constexpr (G <= WAVE) {
-      if (nvec >= G) __syncthreads();
+      if (rp.npk >= G) __syncthreads();
     }
   }
 
@@ -390,9 +439,10 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = k * G + lane;
-      if (p < nvec) {
+      if (p < rp.npk) {
 #pragma unroll
-        for (int i = 0; i < W; ++i) mine[(size_t)p * W + i] = acc[k][i];
+        for (int i = 0; i < W; ++i)
+          if (i < rp.valid(p)) mine[(size_t)p * W + i] = acc[k][i];
       }
     }
   }
@@ -401,16 +451,15 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
 /* ------------------------------------------------------------------ streaming reverse */
 
 /* Rows too long to keep x and dy in registers: they are read twice (the second read mostly from
- * cache). Same alignment rule as the resident reverse. NA > 0: a thread still keeps the dg sums
- * of its NA packs of columns in registers and the workgroup writes one partial row at the end.
- * NA == 0 (rows beyond 1024 * NA packs): each workgroup adds every row it processes into its
- * partial row in memory (first row: overwrite). */
+ * cache). NA > 0: a thread still keeps the dg sums of its NA packs of columns in registers and the
+ * workgroup writes one partial row at the end. NA == 0 (rows beyond 1024 * NA packs): each
+ * workgroup adds every row it processes into its partial row in memory (first row: overwrite). */
 template <class T> constexpr int stream_acc_packs() {
   using P = typename precision<T>::type;
   return 64 / ((PACK_BYTES / (int)sizeof(T)) * (int)(sizeof(P) / 4)); /* 64 registers of sums */
 }
 
-template <class T, int W, int NA, bool BLEND>
+template <class T, int W, int NA, bool BLEND, bool LOOSE>
 __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
@@ -418,7 +467,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
   constexpr int G = STREAM_THREADS, U = 2;
   __shared__ P slots[2][2][G / WAVE];
   const int lane = threadIdx.x;
-  const int nvec = (int)(n / W);
+  const RowPacks<T, W, LOOSE> rp(n);
   P* mine = partials + (size_t)blockIdx.x * n;
   int parity = 0;
   bool first = true;
@@ -431,15 +480,15 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
   for (size_t row = blockIdx.x; row < m; row += gridDim.x, parity ^= 1, first = false) {
     const size_t off = row * n;
     P ss = (P)0, c = (P)0;
-    for (int p0 = lane; p0 < nvec; p0 += G * U) {
+    for (int p0 = lane; p0 < rp.npk; p0 += G * U) {
       P xv[U][W], dv[U][W], gv[U][W];
 #pragma unroll
       for (int u = 0; u < U; ++u) {
         const int p = p0 + u * G;
-        if (p < nvec) {
-          load_pack<T, W>(x + off + (size_t)p * W, xv[u]);
-          load_pack<T, W>(dy + off + (size_t)p * W, dv[u]);
-          load_pack<T, W>(gain + (size_t)p * W, gv[u]);
+        if (p < rp.npk) {
+          rp.template load<false>(x + off, p, xv[u]);
+          rp.template load<false>(dy + off, p, dv[u]);
+          rp.template load<false>(gain, p, gv[u]);
         } else {
 #pragma unroll
           for (int i = 0; i < W; ++i) xv[u][i] = dv[u][i] = gv[u][i] = (P)0;
@@ -459,36 +508,36 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
 
     auto finish_pack = [&](int p, P (&sum)[W], bool in_registers) {
       P xv[W], dv[W], gv[W], out[W];
-      load_pack_nt<T, W>(x + off + (size_t)p * W, xv);
-      load_pack_nt<T, W>(dy + off + (size_t)p * W, dv);
-      load_pack<T, W>(gain + (size_t)p * W, gv);
+      rp.template load<true>(x + off, p, xv);
+      rp.template load<true>(dy + off, p, dv);
+      rp.template load<false>(gain, p, gv);
 #pragma unroll
       for (int i = 0; i < W; ++i) {
         out[i] = r * (dv[i] * gv[i] - xv[i] * cc);
         const P t = dv[i] * xv[i] * r;
         if (in_registers) {
           sum[i] += t;
-        } else {
+        } else if (i < rp.valid(p)) {
           P* slot = mine + (size_t)p * W + i;
           *slot = first ? t : *slot + t;
         }
       }
       if constexpr (BLEND) {
         P old[W];
-        load_pack<T, W>(dx + off + (size_t)p * W, old);
+        rp.template load<false>(dx + off, p, old);
 #pragma unroll
         for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
       }
-      store_pack_nt<T, W>(dx + off + (size_t)p * W, out);
+      rp.store(dx + off, p, out);
     };
     if constexpr (NA > 0) {
 #pragma unroll
       for (int k = 0; k < NA; ++k) {
         const int p = k * G + lane;
-        if (p < nvec) finish_pack(p, acc[k], true);
+        if (p < rp.npk) finish_pack(p, acc[k], true);
       }
     } else {
-      for (int p = lane; p < nvec; p += G) finish_pack(p, acc[0], false);
+      for (int p = lane; p < rp.npk; p += G) finish_pack(p, acc[0], false);
     }
   }
 
@@ -496,9 +545,10 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
 #pragma unroll
     for (int k = 0; k < NA; ++k) {
       const int p = k * G + lane;
-      if (p < nvec) {
+      if (p < rp.npk) {
 #pragma unroll
-        for (int i = 0; i < W; ++i) mine[(size_t)p * W + i] = acc[k][i];
+        for (int i = 0; i < W; ++i)
+          if (i < rp.valid(p)) mine[(size_t)p * W + i] = acc[k][i];
       }
     }
   }
@@ -506,7 +556,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
 
 /* ------------------------------------------------------------------ shared-row reverse */
 
-/* Rows too long for one workgroup's registers, pack-aligned: the grid is S slices of C
+/* Rows too long for one workgroup's registers: the grid is S slices of C
  * consecutive workgroups. The C workgroups of a slice share every row of the slice
  * (rows slice, slice + S, ...): each keeps the dg sums of its chunk in registers for the whole
  * kernel and, per row, its chunk of x, dy and (from L2) the gain; the two row sums (x^2 and dy*g*x) are
@@ -523,7 +573,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
 template <class T> constexpr int norm_rev_cluster_nv() { return 2; }
 template <class T> constexpr int norm_rev_cluster_per_cu() { return sizeof(T) == 2 ? 1 : 2; }
 
-template <class T, int W, bool BLEND>
+template <class T, int W, bool BLEND, bool LOOSE>
 __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) void rmsnorm_rev_cluster(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha,
@@ -537,9 +587,9 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
   const int lane = threadIdx.x;
   const int rank = (int)(blockIdx.x % (unsigned)C);
   const size_t slice = blockIdx.x / (unsigned)C, S = gridDim.x / (unsigned)C;
-  const int nvec = (int)(n / W);
+  const RowPacks<T, W, LOOSE> rp(n);
   const int lo = rank * packs_per_block;
-  const int hi = lo + packs_per_block < nvec ? lo + packs_per_block : nvec;
+  const int hi = lo + packs_per_block < rp.npk ? lo + packs_per_block : rp.npk;
 
   P acc[NV][W];
 #pragma unroll
@@ -558,14 +608,17 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = lo + k * G + lane;
-      if (p < hi) {
-        xv[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(x + off + (size_t)p * W));
-        dv[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(dy + off + (size_t)p * W));
-        gv[k] = *reinterpret_cast<const V*>(gain + (size_t)p * W);
-      } else {
+      xv[k] = p < hi ? rp.template raw<true>(x + off, p) : V{};
+    }
 #pragma unroll
-        for (int i = 0; i < W; ++i) xv[k][i] = dv[k][i] = gv[k][i] = (T)0;
-      }
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * G + lane;
+      dv[k] = p < hi ? rp.template raw<true>(dy + off, p) : V{};
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * G + lane;
+      gv[k] = p < hi ? rp.template raw<false>(gain, p) : V{};
     }
     P ss = (P)0, c = (P)0;
 #pragma unroll
@@ -594,11 +647,11 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
       if (!complete) { /* gave up waiting: both sums over the whole row here, and no waiting for later rows */
         patience = 0;
         P s2 = (P)0, c2 = (P)0;
-        for (int p = lane; p < nvec; p += G) {
+        for (int p = lane; p < rp.npk; p += G) {
           P u[W], d[W], g[W];
-          load_pack<T, W>(x + off + (size_t)p * W, u);
-          load_pack<T, W>(dy + off + (size_t)p * W, d);
-          load_pack<T, W>(gain + (size_t)p * W, g);
+          rp.template load<false>(x + off, p, u);
+          rp.template load<false>(dy + off, p, d);
+          rp.template load<false>(gain, p, g);
 #pragma unroll
           for (int i = 0; i < W; ++i) {
             s2 += u[i] * u[i];
@@ -627,11 +680,11 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
         }
         if constexpr (BLEND) {
           P old[W];
-          load_pack<T, W>(dx + off + (size_t)p * W, old);
+          rp.template load<false>(dx + off, p, old);
 #pragma unroll
           for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
         }
-        store_pack_nt<T, W>(dx + off + (size_t)p * W, out);
+        rp.store(dx + off, p, out);
       }
     }
   }
@@ -642,16 +695,16 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
     const int p = lo + k * G + lane;
     if (p < hi) {
 #pragma unroll
-      for (int i = 0; i < W; ++i) mine[(size_t)p * W + i] = acc[k][i];
+      for (int i = 0; i < W; ++i)
+        if (i < rp.valid(p)) mine[(size_t)p * W + i] = acc[k][i];
     }
   }
 }
 
-/* Workgroups per row when the reverse shares rows (pack-aligned operands only); 0 when not. */
+/* Workgroups per row when the reverse shares rows; 0 when it does not. */
 template <class T> inline int rmsnorm_rev_cluster_size(size_t n) {
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  if (n % W != 0) return 0;
-  const size_t packs = n / W;
+  const size_t packs = (n + W - 1) / W;
   const int regime = row_regime_override();
   if (regime != REGIME_AUTO && regime != REGIME_CLUSTER) return 0;
   constexpr size_t resident = (size_t)NORM_BLOCK * max_nv_for<T>(16); /* what the resident reverse holds */
@@ -816,63 +869,62 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   MP_CHECK_LAUNCH();
 }
 
-template <class T, int W>
-inline void rmsnorm_reverse_w(const T* x, const T* gain, const T* dy, T* dx, T* dg, void* scratch,
-                              double eps, double alpha, size_t m, size_t n, hipStream_t stream) {
+template <class T, bool LOOSE>
+inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T* dg, void* scratch,
+                               double eps, double alpha, size_t m, size_t n, hipStream_t stream) {
   using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
   P* partials = static_cast<P*>(scratch);
   const size_t max_rows = rmsnorm_reverse_partial_rows(m);
+  const size_t packs = (n + W - 1) / W;
   const bool blend = alpha != 0.0;
   unsigned rows = 0;
-  /* four register arrays per thread (x, dy, gain, dg sums): 16 registers each when packed,
-   * 8 elements each on the element-wise path */
-  constexpr int MAXNV = W == 1 ? 8 : max_nv_for<T>(16);
-  /* shared rows: pack-aligned operands, dx distinct from x and dy (a workgroup that stops waiting
-   * re-reads the row), and rows beyond the resident kernel unless the regime is forced */
+  /* four register arrays per thread (x, dy, gain, dg sums): 16 registers each */
+  constexpr int MAXNV = max_nv_for<T>(16);
+  /* shared rows: dx distinct from x and dy (a workgroup that stops waiting re-reads the row), and
+   * rows beyond the resident kernel unless the regime is forced */
   const bool distinct = static_cast<const void*>(dx) != static_cast<const void*>(x) &&
                         static_cast<const void*>(dx) != static_cast<const void*>(dy);
-  const int C = W > 1 && distinct ? rmsnorm_rev_cluster_size<T>(n) : 0;
+  const int C = distinct ? rmsnorm_rev_cluster_size<T>(n) : 0;
   const bool force_shared = C >= 1 && row_regime_override() == REGIME_CLUSTER;
-  const RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row((n + W - 1) / W, MAXNV, 1, 8);
+  const RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row(packs, MAXNV, 1, 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     rows = (unsigned)(need < max_rows ? need : max_rows);
     const dim3 grid(rows), block(NORM_BLOCK);
-    if (blend) rmsnorm_rev_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
-    else rmsnorm_rev_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+    if (blend) rmsnorm_rev_resident<T, W, G, NV, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+    else rmsnorm_rev_resident<T, W, G, NV, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
   });
   bool shared = false;
-  if constexpr (W > 1) {
-    if (!resident && C >= 1) {
-      using Word = typename slot_word<P>::type;
-      size_t S = (size_t)compute_units() * norm_rev_cluster_per_cu<T>() / (size_t)C; /* every workgroup resident at once */
-      if (S > m) S = m;
-      if (S == 0) S = 1;
-      rows = (unsigned)S;
-      const int ppb = (int)((n / W + C - 1) / C);
-      require(ppb <= CLUSTER_THREADS * norm_rev_cluster_nv<T>(), "rmsnorm reverse: cluster chunk exceeds the register tile");
-      Word* slots = reinterpret_cast<Word*>(partials + rmsnorm_reverse_partial_rows(m) * n);
-      if (C > 1) {
-        const size_t words = m * (size_t)C * 2;
-        cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
-      }
-      const dim3 grid((unsigned)(S * C)), block(CLUSTER_THREADS);
-      if (blend) rmsnorm_rev_cluster<T, W, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
-      else rmsnorm_rev_cluster<T, W, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
-      shared = true;
+  if (!resident && C >= 1) {
+    using Word = typename slot_word<P>::type;
+    size_t S = (size_t)compute_units() * norm_rev_cluster_per_cu<T>() / (size_t)C; /* every workgroup resident at once */
+    if (S > m) S = m;
+    if (S == 0) S = 1;
+    rows = (unsigned)S;
+    const int ppb = (int)((packs + C - 1) / C);
+    require(ppb <= CLUSTER_THREADS * norm_rev_cluster_nv<T>(), "rmsnorm reverse: cluster chunk exceeds the register tile");
+    Word* slots = reinterpret_cast<Word*>(partials + rmsnorm_reverse_partial_rows(m) * n);
+    if (C > 1) {
+      const size_t words = m * (size_t)C * 2;
+      cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
     }
+    const dim3 grid((unsigned)(S * C)), block(CLUSTER_THREADS);
+    if (blend) rmsnorm_rev_cluster<T, W, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+    else rmsnorm_rev_cluster<T, W, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+    shared = true;
   }
   if (!resident && !shared) {
     rows = (unsigned)max_rows;
     const dim3 grid(rows), block(STREAM_THREADS);
-    constexpr int NA = W == 1 ? 16 : stream_acc_packs<T>();
-    const bool sums_fit = (n + W - 1) / W <= (size_t)STREAM_THREADS * NA;
+    constexpr int NA = stream_acc_packs<T>();
+    const bool sums_fit = packs <= (size_t)STREAM_THREADS * NA;
     if (sums_fit) {
-      if (blend) rmsnorm_rev_stream<T, W, NA, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
-      else rmsnorm_rev_stream<T, W, NA, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+      if (blend) rmsnorm_rev_stream<T, W, NA, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+      else rmsnorm_rev_stream<T, W, NA, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
     } else {
-      if (blend) rmsnorm_rev_stream<T, W, 0, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
-      else rmsnorm_rev_stream<T, W, 0, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+      if (blend) rmsnorm_rev_stream<T, W, 0, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+      else rmsnorm_rev_stream<T, W, 0, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
     }
   }
   MP_CHECK_LAUNCH();
@@ -887,8 +939,8 @@ inline void rmsnorm_reverse(const T* x, const T* gain, const T* dy, T* dx, T* dg
   require(n <= 0x40000000ull, "rmsnorm reverse: row length must not exceed 2^30");
   require(scratch != nullptr, "rmsnorm reverse: scratch must hold mpRmsnormReverseScratchBytes bytes");
   const bool packed = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gain) && (n % W) == 0;
-  if (packed) rmsnorm_reverse_w<T, W>(x, gain, dy, dx, dg, scratch, eps, alpha, m, n, stream);
-  else rmsnorm_reverse_w<T, 1>(x, gain, dy, dx, dg, scratch, eps, alpha, m, n, stream);
+  if (packed) rmsnorm_reverse_as<T, false>(x, gain, dy, dx, dg, scratch, eps, alpha, m, n, stream);
+  else rmsnorm_reverse_as<T, true>(x, gain, dy, dx, dg, scratch, eps, alpha, m, n, stream);
 }
 
 }  // namespace mp

@@ -646,13 +646,15 @@ def test_rmsnorm_reverse_cluster_path(dtype, packs, spin):
     G.set_regime(CLUSTER)
     G.set_cluster_tuning(packs, spin)
     eps = 1e-6
-    for (m, n) in [(3, 8), (5, 64), (4, 1000), (700, 2048), (33, 5000), (2, 50264), (3, 151936), (130, 776)]:
+    # the last four: rows that are not a whole number of packs, and operands shifted by one element
+    for (m, n, shift) in [(3, 8, 0), (5, 64, 0), (4, 1000, 0), (700, 2048, 0), (33, 5000, 0), (2, 50264, 0),
+                          (3, 151936, 0), (130, 776, 0), (4, 1001, 0), (3, 50257, 0), (2, 70001, 1), (33, 5000, 1)]:
         for alpha in (0.0, 1.0):
-            G.say(f"rmsnorm rev cluster dtype={dtype} packs={packs} spin={spin} shape=({m},{n}) alpha={alpha}")
-            x = G.dev(r.normal(0, 1, (m, n)), dtype)
-            g = G.dev(r.normal(1, 0.02, n), dtype)
-            dy = G.dev(r.normal(0, 1, (m, n)), dtype)
-            dx = G.dev(r.normal(0, 1, (m, n)), dtype)
+            G.say(f"rmsnorm rev cluster dtype={dtype} packs={packs} spin={spin} shape=({m},{n}) shift={shift} alpha={alpha}")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            g = G.dev(r.normal(1, 0.02, n), dtype, shift)
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            dx = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
             dg = G.dev(r.normal(0, 1, n), dtype)
             hdx, hdg = G.host(dx.t).copy(), G.host(dg.t).copy()
             scratch, nbytes = G.rmsnorm_scratch(dtype, m, n)
@@ -692,8 +694,8 @@ def test_rmsnorm_reverse_long_rows_in_place():
 def test_rmsnorm_reverse_unaligned(dtype):
     r = rng(61)
     eps = 1e-6
-    for (m, n) in [(5, 100), (3, 1027), (4, 4096)]:
-        for shifts in [(1, 0, 1, 1), (0, 1, 0, 0)]:
+    for (m, n) in [(5, 100), (3, 1027), (4, 4096), (700, 100), (300, 7), (130, 1003), (9, 9001)]:
+        for shifts in [(1, 0, 1, 1), (0, 1, 0, 0), (0, 0, 0, 0)]:
             G.say(f"rmsnorm rev unaligned dtype={dtype} shape=({m},{n}) shifts={shifts}")
             x = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[0])
             g = G.dev(r.normal(1, 0.02, n), dtype, shifts[1])
