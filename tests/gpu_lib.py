@@ -314,6 +314,15 @@ class BlasStream:
         utils.mpStreamSynchronize(self.sc)
         utils.mpDeinitStream(self.sc)
 
+    def enqueue(self, stem, dtype, *args):
+        """Any launcher on this stream, without waiting for it (sync() does)."""
+        kernels, _ = lib()
+        ffi.invoke(getattr(kernels, stem), KEY[dtype], *args, self.sc)
+
+    def sync(self):
+        _, utils = lib()
+        utils.mpStreamSynchronize(self.sc)
+
     def matrix_op(self, stem, src, dst, alpha, m, n):
         """reduce_ij_j and its like on this stream, whose context owns a workspace."""
         kernels, utils = lib()
