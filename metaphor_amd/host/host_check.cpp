@@ -376,6 +376,19 @@ int main(int argc, char** argv) {
   if (matrix_ops(stream)) return 1;
   printf("host_check: inner products, permutate, reduce / broadcast, checkpoint files ok\n");
 
+  { /* a group of streams: slots 1..3 beside the stream above, the same graph code on each of them */
+    auto group = mp::stream::Group<3>::init();
+    CHECK(group.items[0]->ID == 1 && group.items[2]->ID == 3);
+    for (mp::Stream s : group.items)
+      if (subgraphs_example(s)) return 1;
+    group.synchronize();
+    group.deinit();
+    mp::Stream again = mp::stream::init();
+    CHECK(again->ID == 1); /* released slots are handed out again */
+    mp::stream::deinit(again);
+  }
+  printf("host_check: stream group ok\n");
+
   mp::stream::sync(stream);
   mp::stream::deinit(stream);
   mp::device::check();

@@ -11,7 +11,7 @@
  *             inner_product_scaled, permutate}           src/metaphor.zig:44-56, src/ops/*.zig
  *   mp::ops::{selu, softmax, rmsnorm}                   new ops in the same shape
  *   mp::io::{save_tensor, load_tensor}, Graph::{save, load}   src/core/tensor_file.zig
- *   mp::algo::{fill, copy, sequence}, mp::util::{to_device, from_device}
+ *   mp::algo::{fill, copy, sequence}, mp::util::{to_device, from_device}, mp::stream::Group<N>
  * Errors follow the reference: an impossible request panics (prints and aborts), nothing returns
  * a status.
  *
@@ -73,6 +73,22 @@ namespace stream {
 Stream init();
 void deinit(Stream s);
 void sync(Stream s);
+/* N streams made, synchronised and released together (src/core/utils.zig:47-71). */
+template <size_t N> struct Group {
+  static_assert(N <= MAX_STREAMS, "Stream group is larger than max streams.");
+  Stream items[N];
+  static Group init() {
+    Group g;
+    for (size_t i = 0; i < N; ++i) g.items[i] = stream::init();
+    return g;
+  }
+  void synchronize() const {
+    for (size_t i = 0; i < N; ++i) stream::sync(items[i]);
+  }
+  void deinit() const {
+    for (size_t i = 0; i < N; ++i) stream::deinit(items[i]);
+  }
+};
 }  // namespace stream
 
 class Graph;
