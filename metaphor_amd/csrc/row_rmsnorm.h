@@ -342,11 +342,12 @@ template <class T, int W, bool LOOSE> struct RowPacks {
 template <class T, int W, int G, int NV, bool BLEND, bool LOOSE>
 __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
-    typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
+    typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n, unsigned by_xcd) {
   using P = typename precision<T>::type;
   constexpr int RPB = NORM_BLOCK / G;
   __shared__ P slots[2][2][G < WAVE ? 1 : RPB][G < WAVE ? 1 : G / WAVE];
   __shared__ P comb[RPB > 1 ? NORM_BLOCK * NV * W : 1]; /* one row of dg sums per group of the workgroup */
+  const unsigned block = by_xcd ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
 
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
   const RowPacks<T, W, LOOSE> rp(n);
@@ -361,7 +362,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
   }
 
   int parity = 0;
-  for (size_t base = (size_t)blockIdx.x * RPB; base < m; base += (size_t)gridDim.x * RPB, parity ^= 1) {
+  for (size_t base = (size_t)block * RPB; base < m; base += (size_t)gridDim.x * RPB, parity ^= 1) {
     const size_t row = base + sub;
     const bool live = row < m;
     const size_t off = (live ? row : 0) * n;
@@ -892,8 +893,8 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     rows = (unsigned)(need < max_rows ? need : max_rows);
     const dim3 grid(rows), block(NORM_BLOCK);
-    if (blend) rmsnorm_rev_resident<T, W, G, NV, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
-    else rmsnorm_rev_resident<T, W, G, NV, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+    if (blend) rmsnorm_rev_resident<T, W, G, NV, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, rows_share_lines<T>(n));
+    else rmsnorm_rev_resident<T, W, G, NV, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, rows_share_lines<T>(n));
   });
   bool shared = false;
   if (!resident && C >= 1) {

@@ -31,13 +31,14 @@ namespace mp {
 
 template <class T, int W, int G, int NV, bool RAGGED>
 __global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_fwd_resident(
-    const T* x, T* y, size_t m, size_t n) {
+    const T* x, T* y, size_t m, size_t n, unsigned by_xcd) {
   using P = typename precision<T>::type;
   constexpr int RPB = G < WAVE ? WAVE / G : 1; /* rows per workgroup: several only below a wave */
   __shared__ P slots[2][G < WAVE ? 1 : G / WAVE];
 
   const int lane = threadIdx.x % G;
-  const size_t row_at = (size_t)blockIdx.x * RPB + threadIdx.x / G;
+  const unsigned block = by_xcd ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+  const size_t row_at = (size_t)block * RPB + threadIdx.x / G;
   const bool live = row_at < m;            /* a dead part of a wave still runs the cross-lane steps */
   const size_t row = live ? row_at : m - 1;
 
@@ -64,13 +65,14 @@ __global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_fwd_resident(
 
 template <class T, int W, int G, int NV, bool RAGGED, bool BLEND>
 __global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_rev_resident(
-    const T* y, const T* dy, T* dx, typename precision<T>::type alpha, size_t m, size_t n) {
+    const T* y, const T* dy, T* dx, typename precision<T>::type alpha, size_t m, size_t n, unsigned by_xcd) {
   using P = typename precision<T>::type;
   constexpr int RPB = G < WAVE ? WAVE / G : 1;
   __shared__ P slots[G < WAVE ? 1 : G / WAVE];
 
   const int lane = threadIdx.x % G;
-  const size_t row_at = (size_t)blockIdx.x * RPB + threadIdx.x / G;
+  const unsigned block = by_xcd ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+  const size_t row_at = (size_t)block * RPB + threadIdx.x / G;
   const bool live = row_at < m;
   const size_t row = live ? row_at : m - 1;
 
@@ -681,8 +683,8 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, ragged ? 16 : 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
-    if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n);
-    else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n);
+    if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
+    else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
   });
   if (!resident)
     softmax_fwd_stream<T, W><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
@@ -749,11 +751,11 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) {
-      if (blend) softmax_rev_resident<T, W, G, NV, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
-      else softmax_rev_resident<T, W, G, NV, true, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+      if (blend) softmax_rev_resident<T, W, G, NV, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
+      else softmax_rev_resident<T, W, G, NV, true, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
     } else {
-      if (blend) softmax_rev_resident<T, W, G, NV, false, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
-      else softmax_rev_resident<T, W, G, NV, false, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+      if (blend) softmax_rev_resident<T, W, G, NV, false, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
+      else softmax_rev_resident<T, W, G, NV, false, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
     }
   });
   if (!resident) {
