@@ -7,9 +7,11 @@
  *   broadcast_j_ij  dst[i,j] = src[j] + alpha*dst[i,j]           src/cuda/nvcc_src/broadcast_j_ij.cu:9-57
  * The reference sums a row with one 32-lane warp in the storage type and mis-indexes the output
  * of the column sum (reduce_ij_j.cu:42-43, grid over m instead of n at :56); here sums run in
- * precision<T>, rows are folded with the wave64 all-reduce, and the column sum is a single
- * deterministic pass (each workgroup owns a strip of columns and walks all rows). alpha == 0
- * never reads dst.
+ * precision<T>, rows are folded with the wave64 all-reduce, and the column sum is deterministic:
+ * each workgroup owns a strip of columns and walks all rows, or, given a workspace, a chunk of
+ * the rows, whose partial sums a second kernel adds in a fixed order. Operands at any alignment
+ * and row length keep 128-bit accesses (packs that start at any element, see loose_vec_of).
+ * alpha == 0 never reads dst.
  */
 #ifndef MP_ROW_REDUCE_H
 #define MP_ROW_REDUCE_H
