@@ -140,3 +140,25 @@ def test_inner_product_at_size_is_linear_in_its_operands():
     scale = float((a1.float().abs().mean() + a2.float().abs().mean()) * b.float().abs().mean() * n)
     err = (c_sum.float() - c_acc.float()).abs().max().item()
     assert err <= 4e-3 * scale, (err, scale)
+
+
+def test_r16_vector_products_keep_subnormal_inputs():
+    """The r16 matrix-vector product multiplies packed halves (v_dot2_f32_f16); subnormal matrix
+    entries must still count: against a large vector they add up to ordinary values."""
+    f16 = torch.float16
+    m, n = 64, 4096
+    a = np.full((m, n), 3e-6)  # below the smallest normal r16 value (6.1e-5)
+    a[:, ::7] = 2.5e-7
+    A = G.dev(a, f16)
+    v, u = G.dev(np.full((n, 1), 2048.0), f16), G.dev(np.full((1, m), 2048.0), f16)
+    av, ua = G.Guarded((m, 1), f16), G.Guarded((1, n), f16)
+    with G.BlasStream() as stream:
+        G.say("A.v and u.A with subnormal r16 entries")
+        stream.inner_product("ij_jk_ik", A.t, v.t, 1.0, av.t, 0.0, m, n, 1)
+        stream.inner_product("ij_jk_ik", u.t, A.t, 1.0, ua.t, 0.0, 1, m, n)
+    ref_av, ref_ua = O.inner_product(G.host(A.t), G.host(v.t)), O.inner_product(G.host(u.t), G.host(A.t))
+    assert float(ref_av.min()) > 20.0 and float(ref_ua.min()) > 0.03
+    G.compare(av.t, ref_av, f16, "A.v with subnormal entries", rowwise=False)
+    G.compare(ua.t, ref_ua, f16, "u.A with subnormal entries", rowwise=False)
+    for gd in (A, v, u, av, ua):
+        gd.check("subnormal products")
