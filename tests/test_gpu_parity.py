@@ -766,3 +766,37 @@ def test_device_utils_roundtrip():
     utils.mpDeviceSynchronize()
     utils.mpCheckLastError()
     utils.mpDeinitStream(sc)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float16], ids=["r32", "r16"])
+@pytest.mark.parametrize("n", [96, 2048, 40000], ids=["short", "resident", "long"])
+def test_special_values_follow_the_closed_forms(dtype, n):
+    """NaN, +inf and all-zero rows: the kernels return what the closed forms (the oracle) return,
+    NaN where they are NaN, in every row regime; rows without special values are untouched."""
+    r = rng(91)
+    m = 6
+    x = r.normal(0, 1, (m, n))
+    x[1, n // 3] = np.inf          # softmax: exp(inf - inf) -> NaN row; rmsnorm: inf / inf -> NaN
+    x[2, n // 2] = np.nan          # NaN spreads over its row only
+    x[3, :] = 0.0                  # softmax: uniform 1/n; rmsnorm: 0 * rsqrt(eps) = 0
+    x[4, 5] = -np.inf              # softmax: exactly 0 there
+    eps = 1e-6
+    G.say(f"special values dtype={dtype} n={n}")
+    xd = G.dev(x, dtype)
+    g = G.dev(r.normal(1, 0.02, n), dtype)
+    p, y = G.Guarded((m, n), dtype), G.Guarded((m, n), dtype)
+    G.softmax(xd.t, p.t)
+    G.rmsnorm(xd.t, g.t, y.t, eps)
+    xh = G.host(xd.t)
+    with np.errstate(all="ignore"):
+        ref_p, ref_y = O.softmax_ij_j(xh), O.rmsnorm_ij_j(xh, G.host(g.t), eps)
+    G.compare(p.t, ref_p, dtype, "softmax with special values", atol=G.SOFTMAX_ATOL[dtype])
+    G.compare(y.t, ref_y, dtype, "rmsnorm with special values")
+    got_p, got_y = G.host(p.t).astype(np.float64), G.host(y.t).astype(np.float64)
+    assert np.array_equal(np.isnan(got_p), np.isnan(ref_p)), "softmax: NaN exactly where the closed form is NaN"
+    assert np.array_equal(np.isnan(got_y), np.isnan(ref_y)), "rmsnorm: NaN exactly where the closed form is NaN"
+    assert np.isnan(ref_p[1]).all() and np.isnan(ref_p[2]).all() and not np.isnan(ref_p[[0, 3, 4, 5]]).any()
+    assert got_p[4, 5] == 0.0 and np.allclose(got_p[3], 1.0 / n, rtol=2e-3)
+    assert (got_y[3] == 0.0).all()
+    for gd in (xd, g, p, y):
+        gd.check("special values")
