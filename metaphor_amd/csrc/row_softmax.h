@@ -247,11 +247,13 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
  * before it waits, so with in-order dispatch the wait is short; if spin_limit polls pass
  * anyway, the workgroup stops waiting and folds the whole row itself (one extra read of the row),
  * so every wave reaches the end whatever the scheduling. */
-/* packs per thread: 24 registers of row data, so that two workgroups fit a CU (64 registers) */
+/* packs per thread, so that two workgroups fit a CU (64 registers): 24 registers of widened row
+ * data for r32 and r64 (6 packs); r16 chunks stay in their storage type (four registers a
+ * pack) and are widened where they are used, at the price of a second exponential per element,
+ * which makes room for 7 packs: a 50257-wide r16 row then fits one workgroup and needs no
+ * exchange (5.2 -> 5.6 TB/s; 8 packs spill) */
 template <class T> constexpr int cluster_nv() {
-  /* r16 chunks stay in their storage type (four registers a pack) and are widened where they are
-   * used, at the price of a second exponential per element: 6 packs per thread like r32 */
-  if (sizeof(T) == 2) return 24 / 4;
+  if (sizeof(T) == 2) return 7;
   return 24 / ((PACK_BYTES / (int)sizeof(T)) * (int)(sizeof(typename precision<T>::type) / 4));
 }
 
