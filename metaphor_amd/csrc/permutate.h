@@ -15,6 +15,8 @@
  * sits in slot p ^ (r / W)), which keeps the 128-bit LDS writes aligned and spreads the transposed
  * reads over the banks. r16 tiles are gathered as 32-bit words (two neighbouring columns at
  * once) and separated in registers, so a thread issues W/2 LDS reads per output pack.
+ * The transposed reads still conflict (the counter shows conflicts in 11 % of the cycles), but they
+ * do not bound the kernel: with a conflict-free read pattern it measures the same 6.1 TB/s.
  * Operands whose rows are not 16-byte aligned (an odd row length, a shifted base) keep 128-bit
  * accesses, global and LDS: their packs simply start at any element. A misaligned 128-byte row
  * segment touches two cache lines, which costs this kernel more than it costs a copy (measured:
