@@ -603,19 +603,30 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
    * still publishes its sums first, so its partners are never held up by it). */
   unsigned patience = spin_limit;
   int parity = 0;
+  /* r16 runs one workgroup per CU, so nothing else on the CU fills the wait for the partners:
+   * the chunk of the next row is asked for before that wait (two-byte packs leave the registers) */
+  constexpr bool AHEAD = sizeof(T) == 2;
+  auto fetch = [&](size_t row, V (&xs)[NV], V (&ds)[NV]) {
+    const size_t off = row * n;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * G + lane;
+      xs[k] = p < hi ? rp.template raw<true>(x + off, p) : V{};
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * G + lane;
+      ds[k] = p < hi ? rp.template raw<true>(dy + off, p) : V{};
+    }
+  };
+  V xv[NV], dv[NV], xn[AHEAD ? NV : 1], dn[AHEAD ? NV : 1];
+  if constexpr (AHEAD) {
+    if (slice < m) fetch(slice, xv, dv);
+  }
   for (size_t row = slice; row < m; row += S, parity ^= 1) {
     const size_t off = row * n;
-    V xv[NV], dv[NV], gv[NV]; /* the gain chunk comes from L2 every row: registers go to the dg sums */
-#pragma unroll
-    for (int k = 0; k < NV; ++k) {
-      const int p = lo + k * G + lane;
-      xv[k] = p < hi ? rp.template raw<true>(x + off, p) : V{};
-    }
-#pragma unroll
-    for (int k = 0; k < NV; ++k) {
-      const int p = lo + k * G + lane;
-      dv[k] = p < hi ? rp.template raw<true>(dy + off, p) : V{};
-    }
+    V gv[NV]; /* the gain chunk comes from L2 every row: registers go to the dg sums */
+    if constexpr (!AHEAD) fetch(row, xv, dv);
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = lo + k * G + lane;
@@ -640,6 +651,9 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
       forget(gv[k]);
     }
 
+    if constexpr (AHEAD) {
+      if (row + S < m) fetch(row + S, xn, dn);
+    }
     if (C > 1) {
       P sums[2] = {ss, c};
       const bool complete = cluster_exchange_sums<2>(slots + row * (size_t)C * 2, C, rank, sums, patience, bc, lane);
@@ -686,6 +700,13 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
           for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
         }
         rp.store(dx + off, p, out);
+      }
+    }
+    if constexpr (AHEAD) {
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        xv[k] = xn[k];
+        dv[k] = dn[k];
       }
     }
   }
