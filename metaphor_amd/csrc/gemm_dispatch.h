@@ -88,10 +88,10 @@ inline void gemm_row_major(StreamContext ctx, bool a_transposed, bool b_transpos
     void* ws = blas ? blas->workspace : nullptr;
     const size_t ws_bytes = blas ? blas->workspace_bytes : 0;
     if (n == 1) outer_product<T>(A, B, C, alpha, beta, m, k, stream);
-    else if (k == 1 && !a_transposed) reduce_rows<T>(A, B, C, alpha, beta, m, n, stream);
+    else if (k == 1 && !a_transposed) reduce_rows<T>(A, B, C, alpha, beta, m, n, stream, ws, ws_bytes);
     else if (k == 1) reduce_cols<T>(A, B, C, ws, alpha, beta, n, m, stream, ws_bytes);
     else if (!b_transposed) reduce_cols<T>(B, A, C, ws, alpha, beta, n, k, stream, ws_bytes);
-    else reduce_rows<T>(B, A, C, alpha, beta, k, n, stream);
+    else reduce_rows<T>(B, A, C, alpha, beta, k, n, stream, ws, ws_bytes);
     return;
   }
   const rocblas_handle handle = get_handle(ctx);

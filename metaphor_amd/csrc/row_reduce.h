@@ -27,23 +27,29 @@ namespace mp {
 /* One group of G threads per row; groups of 16, 32 or 64 lanes share a 256-thread workgroup
  * (several rows per wavefront below 64), wider groups own one row per workgroup. */
 /* DOT: every element is multiplied by vec[column] first (a matrix-vector product, one dot
- * product per row). dst[row] = scale * sum + blend * dst[row]; blend == 0 never reads dst. */
-template <class T, int W, int G, bool DOT>
+ * product per row). dst[q] = scale * sum + blend * dst[q]; blend == 0 never reads dst.
+ * A row may be cut into `chunks` segments of chunk_len elements (the last one shorter): the
+ * kernel then sees rows * chunks logical rows and writes one sum per segment, which a second
+ * launch adds up; O is the type of those sums (the storage type, or precision<T> for partials). */
+template <class T, class O, int W, int G, bool DOT>
 __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
-    const T* src, const T* vec, T* dst, typename precision<T>::type scale, typename precision<T>::type blend,
-    size_t m, size_t n) {
+    const T* src, const T* vec, O* dst, typename precision<T>::type scale, typename precision<T>::type blend,
+    size_t segments, size_t n, unsigned chunks, size_t chunk_len) {
   using P = typename precision<T>::type;
   constexpr int BLOCK = G < 256 ? 256 : G, RPB = BLOCK / G, U = 4;
   __shared__ P slots[G < WAVE ? 1 : G / WAVE];
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
   const size_t want = (size_t)blockIdx.x * RPB + sub;
-  const bool live = want < m; /* a dead group of a live wavefront walks the last row and stores nothing */
-  const size_t row = live ? want : m - 1;
+  const bool live = want < segments; /* a dead group of a live wavefront walks the last segment and stores nothing */
+  const size_t q = live ? want : segments - 1;
+  const size_t row = q / chunks, first = (q % chunks) * chunk_len; /* chunks == 1: the whole row */
+  const size_t len = n - first < chunk_len ? n - first : chunk_len;
 
-  const T* r = src + row * n;
-  const RowGeom<T, W> g(r, n, true);
+  const T* r = src + row * n + first;
+  const T* v = vec + first; /* DOT only */
+  const RowGeom<T, W> g(r, len, true);
   const T* body = r + g.head;
-  const T* vbody = vec + g.head; /* DOT only: the vector entries of the packed columns */
+  const T* vbody = v + g.head; /* the vector entries of the packed columns */
   const bool vec_packed = DOT && (reinterpret_cast<uintptr_t>(vbody) & 15u) == 0;
   P s = (P)0;
   if constexpr (DOT && sizeof(T) == 2) {
@@ -96,27 +102,26 @@ __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
     size_t e = (size_t)-1;
     if (lane < g.head) e = (size_t)lane;
     else if (lane - g.head < g.tail) e = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
-    if (e != (size_t)-1) s += DOT ? (P)r[e] * (P)vec[e] : (P)r[e];
+    if (e != (size_t)-1) s += DOT ? (P)r[e] * (P)v[e] : (P)r[e];
   }
   s = group_allreduce<AddOP, G>(s, slots, lane);
-  if (live && lane == 0) dst[row] = (T)(blend != (P)0 ? scale * s + blend * (P)dst[row] : scale * s);
+  if (live && lane == 0) dst[q] = (O)(blend != (P)0 ? scale * s + blend * (P)dst[q] : scale * s);
 }
 
-/* dst[i] = scale * sum_j src[i,j] (* vec[j] when vec is given) + blend * dst[i] */
-template <class T>
-inline void reduce_rows(const T* src, const T* vec, T* dst, double scale, double blend, size_t m, size_t n,
-                        hipStream_t stream) {
-  if (m == 0) return;
-  using P = typename precision<T>::type;
-  constexpr int W = PACK_BYTES / (int)sizeof(T);
-  require(n <= 0x40000000ull, "row sums: row length must not exceed 2^30");
-  require(m < 0x7fffffffull, "row sums: too many rows for one grid");
-  const size_t packs = (n + W - 1) / W;
+/* One launch of the kernel above: `rows` rows of n elements of S, each cut into `chunks` segments. */
+template <class S, class O>
+inline void launch_reduce_rows(const S* src, const S* vec, O* dst, double scale, double blend, size_t rows, size_t n,
+                               size_t chunks, size_t chunk_len, hipStream_t stream) {
+  using P = typename precision<S>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(S);
+  const size_t segments = rows * chunks;
+  require(segments < 0x7fffffffull, "row sums: too many rows for one grid");
+  const size_t packs = (chunk_len + W - 1) / W;
 #define MP_ROWS_LAUNCH(G_)                                                                                          \
   do {                                                                                                              \
-    const dim3 grid((unsigned)((m + (G_ < 256 ? 256 / G_ : 1) - 1) / (G_ < 256 ? 256 / G_ : 1))), block(G_ < 256 ? 256 : G_); \
-    if (vec) reduce_rows_kernel<T, W, G_, true><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, m, n); \
-    else reduce_rows_kernel<T, W, G_, false><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, m, n);   \
+    const dim3 grid((unsigned)((segments + (G_ < 256 ? 256 / G_ : 1) - 1) / (G_ < 256 ? 256 / G_ : 1))), block(G_ < 256 ? 256 : G_); \
+    if (vec) reduce_rows_kernel<S, O, W, G_, true><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, segments, n, (unsigned)chunks, chunk_len); \
+    else reduce_rows_kernel<S, O, W, G_, false><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, segments, n, (unsigned)chunks, chunk_len);   \
   } while (0)
   if (packs <= 16) MP_ROWS_LAUNCH(16);
   else if (packs <= 32) MP_ROWS_LAUNCH(32);
@@ -127,9 +132,45 @@ inline void reduce_rows(const T* src, const T* vec, T* dst, double scale, double
   MP_CHECK_LAUNCH();
 }
 
+/* dst[i] = scale * sum_j src[i,j] (* vec[j] when vec is given) + blend * dst[i].
+ * workspace (optional, workspace_bytes of it): a few very long rows (the sum or the dot product
+ * of whole tensors) would otherwise keep one workgroup each busy; with it they are cut into
+ * segments whose sums, kept in precision<T>, a second launch adds in a fixed order
+ * (measured: r32 [1, 2^26] 0.06 TB/s without). */
 template <class T>
-inline void reduce_rows(const T* src, T* dst, double alpha, size_t m, size_t n, hipStream_t stream) {
-  reduce_rows<T>(src, nullptr, dst, 1.0, alpha, m, n, stream);
+inline void reduce_rows(const T* src, const T* vec, T* dst, double scale, double blend, size_t m, size_t n,
+                        hipStream_t stream, void* workspace = nullptr, size_t workspace_bytes = 0) {
+  if (m == 0) return;
+  using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  require(n <= 0x40000000ull, "row sums: row length must not exceed 2^30");
+  require(m < 0x7fffffffull, "row sums: too many rows for one grid");
+  constexpr size_t SHORTEST = 16384; /* elements of a segment: sixteen packs a thread of a 256-thread group for r32 */
+  const size_t want = (size_t)compute_units() * 16;
+  size_t chunks = 1;
+  if (workspace != nullptr && m < want && n >= 2 * SHORTEST) {
+    chunks = (want + m - 1) / m;
+    if (chunks > n / SHORTEST) chunks = n / SHORTEST;
+    const size_t fit = workspace_bytes / (m * sizeof(P));
+    if (chunks > fit) chunks = fit;
+    if (chunks > 4096) chunks = 4096;
+  }
+  if (chunks > 1) {
+    size_t chunk_len = (n + chunks - 1) / chunks;
+    chunk_len = (chunk_len + W - 1) / W * W; /* whole packs, so that aligned rows give aligned segments */
+    chunks = (n + chunk_len - 1) / chunk_len;
+    P* partials = static_cast<P*>(workspace);
+    launch_reduce_rows<T, P>(src, vec, partials, 1.0, 0.0, m, n, chunks, chunk_len, stream);
+    launch_reduce_rows<P, T>(partials, nullptr, dst, scale, blend, m, chunks, 1, chunks, stream);
+    return;
+  }
+  launch_reduce_rows<T, T>(src, vec, dst, scale, blend, m, n, 1, n, stream);
+}
+
+template <class T>
+inline void reduce_rows(const T* src, T* dst, double alpha, size_t m, size_t n, hipStream_t stream,
+                        void* workspace = nullptr, size_t workspace_bytes = 0) {
+  reduce_rows<T>(src, nullptr, dst, 1.0, alpha, m, n, stream, workspace, workspace_bytes);
 }
 
 /* ------------------------------------------------------------------ column sums */

@@ -162,3 +162,40 @@ def test_r16_vector_products_keep_subnormal_inputs():
     G.compare(ua.t, ref_ua, f16, "u.A with subnormal entries", rowwise=False)
     for gd in (A, v, u, av, ua):
         gd.check("subnormal products")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_sums_and_dot_products_of_few_long_rows(dtype):
+    """The sum or dot product of whole tensors: one to a few very long rows. On a stream made by
+    mpInitStream the rows are cut into segments through the stream's workspace (two launches,
+    fixed order); results must match the oracle like any other row sum."""
+    r = rng(36)
+    with G.BlasStream() as stream:
+        for (m, n, shift) in [(1, 100003, 0), (3, 250000, 0), (8, 70001, 1), (1, 1 << 21, 0), (40, 40000, 0)]:
+            for alpha in (0.0, -0.5):
+                G.say(f"long rows dtype={dtype} shape=({m},{n}) shift={shift} alpha={alpha}")
+                x = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+                v = G.dev(r.normal(0, 1, (n, 1)), dtype, shift)
+                s = G.dev(r.normal(0, 1, m), dtype)
+                d = G.dev(r.normal(0, 1, (m, 1)), dtype)
+                bs, bd = G.host(s.t).copy(), G.host(d.t).copy()
+                stream.matrix_op("reduce_ij_i", x.t, s.t, alpha, m, n)
+                stream.inner_product("ij_jk_ik", x.t, v.t, 1.0, d.t, alpha, m, n, 1)
+                xh = G.host(x.t)
+                mag = np.abs(xh.astype(np.float64)).sum(axis=1) + abs(alpha) * np.abs(bs.astype(np.float64))
+                G.compare(s.t, O.reduce_ij_i(xh, bs if alpha else None, alpha), dtype, f"row sums ({m},{n})",
+                          rowwise=False, scale=mag)
+                ref, scale = O.inner_product(xh, G.host(v.t), 1.0, bd if alpha else None, alpha, with_scale=True)
+                G.compare(d.t, ref, dtype, f"A.v ({m},{n})", rowwise=False, scale=scale)
+                # one row against a matrix stored [k, n]: k dot products of length n
+                k = 3
+                b = G.dev(r.normal(0, 1, (k, n)), dtype)
+                c = G.dev(r.normal(0, 1, (1, k)), dtype)
+                bc = G.host(c.t).copy()
+                row = G.dev(G.host(x.t)[:1].astype(np.float64), dtype)
+                stream.inner_product("ij_kj_ik", row.t, b.t, 0.5, c.t, alpha, 1, n, k)
+                ref, scale = O.inner_product(G.host(row.t), G.host(b.t), 0.5, bc if alpha else None, alpha, tb=True,
+                                             with_scale=True)
+                G.compare(c.t, ref, dtype, f"a.B^T ({k},{n})", rowwise=False, scale=scale)
+                for gd in (x, v, s, d, b, c, row):
+                    gd.check("long rows")
