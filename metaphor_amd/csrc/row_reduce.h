@@ -375,49 +375,14 @@ inline void outer_product(const T* a, const T* b, T* c, double scale, double ble
 
 /* ------------------------------------------------------------------ broadcasts */
 
-/* BY_ROW: dst[i,j] = src[i] + alpha*dst[i,j]; otherwise dst[i,j] = src[j] + alpha*dst[i,j].
- * One workgroup walks rows blockIdx.x, blockIdx.x + gridDim.x, ... */
-template <class T, int W, bool BY_ROW, bool BLEND>
-__global__ __launch_bounds__(256) void broadcast_kernel(
-    const T* src, T* dst, typename precision<T>::type alpha, size_t m, size_t n) {
-  using P = typename precision<T>::type;
-  const int lane = threadIdx.x;
-  for (size_t row = blockIdx.x; row < m; row += gridDim.x) {
-    T* r = dst + row * n;
-    const RowGeom<T, W> g(r, n, true);
-    T* body = r + g.head;
-    const P rv = BY_ROW ? (P)src[row] : (P)0;
-    for (int p = lane; p < g.nvec; p += 256) {
-      P out[W];
-#pragma unroll
-      for (int i = 0; i < W; ++i) out[i] = BY_ROW ? rv : (P)src[(size_t)g.head + (size_t)p * W + i];
-      if constexpr (BLEND) {
-        P old[W];
-        load_pack<T, W>(body + (size_t)p * W, old);
-#pragma unroll
-        for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
-      }
-      store_pack_nt<T, W>(body + (size_t)p * W, out);
-    }
-    if (W > 1) {
-      size_t e = (size_t)-1;
-      if (lane < g.head) e = (size_t)lane;
-      else if (lane - g.head < g.tail) e = (size_t)g.head + (size_t)g.nvec * W + (lane - g.head);
-      if (e != (size_t)-1) {
-        P out = BY_ROW ? rv : (P)src[e];
-        if constexpr (BLEND) out += alpha * (P)r[e];
-        r[e] = (T)out;
-      }
-    }
-  }
-}
+/* BY_ROW: dst[i,j] = src[i] + alpha*dst[i,j]; otherwise dst[i,j] = src[j] + alpha*dst[i,j]. */
 
 /* The destination as one flat array of m*n elements: one pack per thread in one-shot 256-thread
  * workgroups, the shape that writes fastest on this GPU, whatever the row length (short rows keep
  * every lane busy). ALIGNED: n % W == 0 and 16-byte aligned column values, so a pack lies inside
- * one row and its values are one aligned pack load; otherwise a pack may end in the next row
- * (n >= W, so in at most one): the column values are then a pack that starts at any element, or,
- * for the one pack per row that wraps, W single loads. DALIGNED: the destination base is 16-byte
+ * one row and its values are one aligned pack load; otherwise a pack may run over the end of its
+ * row (over several rows when n < W): the column values are then a pack that starts at any
+ * element, or, for a pack that wraps, W single loads. DALIGNED: the destination base is 16-byte
  * aligned; a destination that is not costs about 5 % (packs that start at any element). The last
  * workgroup also writes the m*n % W elements behind the last whole pack. */
 template <class T, int W, bool BY_ROW, bool BLEND, bool ALIGNED, bool DALIGNED>
@@ -433,23 +398,25 @@ __global__ __launch_bounds__(256) void broadcast_flat_kernel(
     const size_t row = row0 + off / n;
     const unsigned col = off % n;
     P out[W];
-    if constexpr (BY_ROW) {
+    if constexpr (BY_ROW && ALIGNED) {
       const P here = (P)src[row];
-      if constexpr (ALIGNED) {
 #pragma unroll
-        for (int i = 0; i < W; ++i) out[i] = here;
-      } else {
-        const P there = col + W > n ? (P)src[row + 1] : here; /* a wrapping pack is never in the last row */
-#pragma unroll
-        for (int i = 0; i < W; ++i) out[i] = col + i >= n ? there : here;
-      }
+      for (int i = 0; i < W; ++i) out[i] = here;
     } else if constexpr (ALIGNED) {
       load_pack<T, W>(src + col, out);
-    } else if (col + W <= n) {
+    } else if (!BY_ROW && col + W <= n) {
       load_pack_loose<T, W>(src + col, out);
-    } else {
+    } else { /* walk the pack's elements: the row advances whenever the column reaches n */
+      size_t r = row;
+      unsigned c = col;
 #pragma unroll
-      for (int i = 0; i < W; ++i) out[i] = (P)src[col + i >= n ? col + i - n : col + i];
+      for (int i = 0; i < W; ++i) {
+        out[i] = BY_ROW ? (P)src[r] : (P)src[c];
+        if (++c == n) {
+          c = 0;
+          ++r;
+        }
+      }
     }
     T* o = dst + idx * W;
     if constexpr (BLEND) {
@@ -478,28 +445,19 @@ inline void broadcast(const T* src, T* dst, double alpha, size_t m, size_t n, hi
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "broadcast: row length must not exceed 2^30");
-  if (n >= (size_t)W) {
-    const size_t total = m * n, blocks = (total / W + 255) / 256 + 1; /* + 1: the tail always has a workgroup */
-    require(blocks < 0x7fffffffull, "broadcast: too many elements for one grid");
-    const dim3 grid((unsigned)blocks), block(256);
-    const bool aligned = n % W == 0 && (BY_ROW || aligned16(src));
-    const bool blend = alpha != 0.0;
+  const size_t total = m * n, blocks = (total / W + 255) / 256 + 1; /* + 1: the tail always has a workgroup */
+  require(blocks < 0x7fffffffull, "broadcast: too many elements for one grid");
+  const dim3 grid((unsigned)blocks), block(256);
+  const bool aligned = n % W == 0 && (BY_ROW || aligned16(src));
+  const bool blend = alpha != 0.0;
 #define MP_FLAT_AS(BLEND_, ALIGNED_, DALIGNED_) \
   broadcast_flat_kernel<T, W, BY_ROW, BLEND_, ALIGNED_, DALIGNED_><<<grid, block, 0, stream>>>(src, dst, (P)alpha, total, (unsigned)n)
 #define MP_FLAT(BLEND_, ALIGNED_) \
   do { if (aligned16(dst)) MP_FLAT_AS(BLEND_, ALIGNED_, true); else MP_FLAT_AS(BLEND_, ALIGNED_, false); } while (0)
-    if (aligned) { if (blend) MP_FLAT(true, true); else MP_FLAT(false, true); }
-    else { if (blend) MP_FLAT(true, false); else MP_FLAT(false, false); }
+  if (aligned) { if (blend) MP_FLAT(true, true); else MP_FLAT(false, true); }
+  else { if (blend) MP_FLAT(true, false); else MP_FLAT(false, false); }
 #undef MP_FLAT
 #undef MP_FLAT_AS
-    MP_CHECK_LAUNCH();
-    return;
-  }
-  /* rows shorter than a pack */
-  const size_t cap = (size_t)compute_units() * 8;
-  const dim3 grid((unsigned)(m < cap ? m : cap)), block(256);
-  if (alpha != 0.0) broadcast_kernel<T, W, BY_ROW, true><<<grid, block, 0, stream>>>(src, dst, (P)alpha, m, n);
-  else broadcast_kernel<T, W, BY_ROW, false><<<grid, block, 0, stream>>>(src, dst, (P)alpha, m, n);
   MP_CHECK_LAUNCH();
 }
 
