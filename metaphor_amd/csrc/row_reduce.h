@@ -108,6 +108,42 @@ __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
   if (live && lane == 0) dst[q] = (O)(blend != (P)0 ? scale * s + blend * (P)dst[q] : scale * s);
 }
 
+/* Rows of up to sixteen packs: G = 1, 2, 4 or 8 lanes a row, each with up to SHORT_ROW_PACKS
+ * packs that start at any element (so no row needs lanes for a head and a tail); the pack that
+ * the end of the row cuts is read element by element. Groups as wide as the longer rows take
+ * would leave most lanes idle (measured on r32 [16M, 2]: 0.07 TB/s with sixteen lanes a row). */
+constexpr int SHORT_ROW_PACKS = 2;
+
+template <class T, class O, int W, int G, bool DOT>
+__global__ __launch_bounds__(256) void reduce_short_rows_kernel(
+    const T* src, const T* vec, O* dst, typename precision<T>::type scale, typename precision<T>::type blend,
+    size_t rows, unsigned n) {
+  using P = typename precision<T>::type;
+  const int lane = threadIdx.x % G;
+  const size_t want = ((size_t)blockIdx.x * 256 + threadIdx.x) / G;
+  const bool live = want < rows; /* a dead group of a live wavefront reads the last row and stores nothing */
+  const size_t row = live ? want : rows - 1;
+  const T* r = src + row * n;
+  P s = (P)0;
+#pragma unroll
+  for (int k = 0; k < SHORT_ROW_PACKS; ++k) {
+    const unsigned j = (unsigned)(lane + k * G) * W;
+    if (j + W <= n) {
+      P a[W], b[W];
+      load_pack_nt_loose<T, W>(r + j, a);
+      if constexpr (DOT) load_pack_loose<T, W>(vec + j, b);
+#pragma unroll
+      for (int i = 0; i < W; ++i) s += DOT ? a[i] * b[i] : a[i];
+    } else {
+#pragma unroll
+      for (int i = 0; i < W - 1; ++i)
+        if (j + i < n) s += DOT ? (P)r[j + i] * (P)vec[j + i] : (P)r[j + i];
+    }
+  }
+  s = fold_partials<AddOP, G>(s);
+  if (live && lane == 0) dst[row] = (O)(blend != (P)0 ? scale * s + blend * (P)dst[row] : scale * s);
+}
+
 /* One launch of the kernel above: `rows` rows of n elements of S, each cut into `chunks` segments. */
 template <class S, class O>
 inline void launch_reduce_rows(const S* src, const S* vec, O* dst, double scale, double blend, size_t rows, size_t n,
@@ -116,6 +152,22 @@ inline void launch_reduce_rows(const S* src, const S* vec, O* dst, double scale,
   constexpr int W = PACK_BYTES / (int)sizeof(S);
   const size_t segments = rows * chunks;
   require(segments < 0x7fffffffull, "row sums: too many rows for one grid");
+  if (chunks == 1 && n <= (size_t)(8 * SHORT_ROW_PACKS * W)) {
+    const size_t row_packs = (n + W - 1) / W;
+#define MP_SHORT_ROWS(G_)                                                                                           \
+  do {                                                                                                              \
+    const dim3 grid((unsigned)((rows * G_ + 255) / 256)), block(256);                                               \
+    if (vec) reduce_short_rows_kernel<S, O, W, G_, true><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, rows, (unsigned)n); \
+    else reduce_short_rows_kernel<S, O, W, G_, false><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, rows, (unsigned)n);   \
+  } while (0)
+    if (row_packs <= 1 * SHORT_ROW_PACKS) MP_SHORT_ROWS(1);
+    else if (row_packs <= 2 * SHORT_ROW_PACKS) MP_SHORT_ROWS(2);
+    else if (row_packs <= 4 * SHORT_ROW_PACKS) MP_SHORT_ROWS(4);
+    else MP_SHORT_ROWS(8);
+#undef MP_SHORT_ROWS
+    MP_CHECK_LAUNCH();
+    return;
+  }
   const size_t packs = (chunk_len + W - 1) / W;
 #define MP_ROWS_LAUNCH(G_)                                                                                          \
   do {                                                                                                              \
@@ -176,19 +228,25 @@ inline void reduce_rows(const T* src, T* dst, double alpha, size_t m, size_t n, 
 /* ------------------------------------------------------------------ column sums */
 
 /* A workgroup owns LANES*CW columns of the rows [blockIdx.y * chunk, (blockIdx.y + 1) * chunk); its
- * SLICES slices take every SLICES-th of those rows and are folded through LDS in slice order, so
- * the result does not depend on scheduling. The sums go to `out + blockIdx.y * n`: the destination
- * itself (O = T, one chunk holding every row, alpha blend) or a partial row of accumulators
- * (O = precision<T>, no blend) that sum_partial_rows adds up afterwards. WEIGHTED: row r counts
- * weight[r] times (a vector-matrix product). LOOSE: rows that are not 16-byte aligned (an odd row
- * length, a shifted base); the packs then start at any element, which a streaming read does not
- * feel, and the pack that the end of the row cuts is read element by element. */
+ * SLICES slices take every SLICES-th of those rows. The slices of a wavefront (64 / LANES of them)
+ * are folded with lane exchanges, the wavefronts through LDS in wavefront order, so the result
+ * does not depend on scheduling. LANES is the power of two that holds the packs of a row of a
+ * narrow matrix (every lane busy however narrow it is: LANES == 1 is a thread per row), else 8
+ * or 64.
+ * The sums go to `out + blockIdx.y * n`: the destination itself (O = T, one chunk holding every
+ * row, alpha blend) or a partial row of accumulators (O = precision<T>, no blend) that
+ * sum_partial_rows adds up afterwards. WEIGHTED: row r counts weight[r] times (a vector-matrix
+ * product). LOOSE: rows that are not 16-byte aligned (an odd row length, a shifted base); the
+ * packs then start at any element, which a streaming read does not feel, and the pack that the
+ * end of the row cuts is read element by element. */
 template <class T, class O, int CW, int LANES, int SLICES, bool WEIGHTED, bool LOOSE>
 __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
     const T* src, const T* weight, O* out, typename precision<T>::type scale, typename precision<T>::type blend,
     size_t m, size_t n, size_t chunk) {
   using P = typename precision<T>::type;
-  __shared__ P part[SLICES][LANES * CW + 1];
+  static_assert(LANES <= WAVE && (LANES & (LANES - 1)) == 0, "a wavefront holds whole slices");
+  constexpr int WAVES = LANES * SLICES / WAVE;
+  __shared__ P part[WAVES][LANES * CW + 1];
   const int c = threadIdx.x % LANES, slice = threadIdx.x / LANES;
   const size_t col = ((size_t)blockIdx.x * LANES + c) * CW;
   const size_t begin = (size_t)blockIdx.y * chunk, end = begin + chunk < m ? begin + chunk : m;
@@ -231,28 +289,52 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
     }
   }
 #pragma unroll
-  for (int i = 0; i < CW; ++i) part[slice][c * CW + i] = s[i];
+  for (int i = 0; i < CW; ++i) {
+#pragma unroll
+    for (int mask = LANES; mask < WAVE; mask <<= 1) s[i] += __shfl_xor(s[i], mask, WAVE);
+    if (threadIdx.x % WAVE < LANES) part[threadIdx.x / WAVE][c * CW + i] = s[i];
+  }
   __syncthreads();
   const int mine = threadIdx.x;
   const size_t at = (size_t)blockIdx.x * LANES * CW + mine;
   if (mine < LANES * CW && at < n) {
     P t = (P)0;
-    for (int i = 0; i < SLICES; ++i) t += part[i][mine];
+#pragma unroll
+    for (int i = 0; i < WAVES; ++i) t += part[i][mine];
     dst[at] = (O)(blend != (P)0 ? scale * t + blend * (P)dst[at] : scale * t);
   }
 }
 
+/* Lanes (packs) of a row per workgroup: as many as a narrow matrix has, so that no lane idles
+ * (measured on r32 [4M, 4]: 0.4 TB/s with 8 lanes); 8 lanes x one pack = 128 bytes, one cache
+ * line, of every aligned row (many strips, so narrow matrices still spread); a wavefront per
+ * kilobyte of a row for wide rows that are not aligned, because a misaligned 128-byte segment
+ * would touch two lines for the data of one (measured on r32 [20000, 50257]: 3.4 TB/s with 8
+ * lanes, one element per lane 4.3). */
+template <class T> inline size_t reduce_cols_lanes(size_t n, bool loose) {
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  const size_t packs = (n + W - 1) / W;
+  if (packs <= 1) return 1;
+  if (packs <= 2) return 2;
+  if (packs <= 4) return 4;
+  if (packs <= 8) return 8;
+  if (loose && packs <= 16) return 16;
+  if (loose && packs <= 32) return 32;
+  return loose ? 64 : 8;
+}
+
 /* Row chunks of the two-stage column sum: enough workgroups to fill the GPU when the matrix is
- * tall and narrow (a [262144, 1024] r32 matrix has 32 column strips), never chunks under 512
- * rows; 1 when the strips alone are enough or the matrix is short. */
+ * tall and narrow (a [262144, 1024] r32 matrix has 32 column strips), never chunks under four
+ * rows a slice (512 rows at 8 lanes); 1 when the strips alone are enough or the matrix is short. */
 template <class T> inline size_t reduce_cols_chunks(size_t m, size_t n) {
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  const size_t lanes = n % W == 0 ? 8 : 64; /* as reduce_cols picks them (a shifted base aside) */
+  const size_t lanes = reduce_cols_lanes<T>(n, n % W != 0); /* as reduce_cols picks them (a shifted base aside) */
   const size_t strips = ((n + W - 1) / W + lanes - 1) / lanes;
   const size_t want = (size_t)compute_units() * 4;
   if (strips >= want) return 1;
   size_t chunks = (want + strips - 1) / strips;
-  const size_t most = m / 512;
+  const size_t least = lanes >= 8 ? 512 : 4096 / lanes; /* rows */
+  const size_t most = m / least;
   if (chunks > most) chunks = most;
   if (chunks > 1024) chunks = 1024;
   return chunks > 1 ? chunks : 1;
@@ -280,14 +362,16 @@ inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, do
   } while (0)
 #define MP_COLS(O_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)                              \
   do {                                                                              \
-    if (loose) MP_COLS_AS(O_, 64, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);       \
+    if (lanes == 1) MP_COLS_AS(O_, 1, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);   \
+    else if (lanes == 2) MP_COLS_AS(O_, 2, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_); \
+    else if (lanes == 4) MP_COLS_AS(O_, 4, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_); \
+    else if (lanes == 16) MP_COLS_AS(O_, 16, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_); \
+    else if (lanes == 32) MP_COLS_AS(O_, 32, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_); \
+    else if (lanes == 64) MP_COLS_AS(O_, 64, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_); \
+    else if (loose) MP_COLS_AS(O_, 8, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);   \
     else MP_COLS_AS(O_, 8, false, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);             \
   } while (0)
-  /* aligned rows: 8 lanes x one pack = 128 bytes, one cache line, of every row per workgroup (many
-   * strips, so narrow matrices still spread); rows that are not: a wavefront per kilobyte of a
-   * row, because a misaligned 128-byte segment would touch two lines for the data of one
-   * (measured on r32 [20000, 50257]: 3.4 TB/s with 8 lanes, one element per lane 4.3) */
-  const size_t lanes = loose ? 64 : 8;
+  const size_t lanes = reduce_cols_lanes<T>(n, loose); /* under 8 lanes the kernel is always the loose one */
   const size_t blocks = ((n + W - 1) / W + lanes - 1) / lanes;
   require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
   size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;

@@ -199,3 +199,46 @@ def test_sums_and_dot_products_of_few_long_rows(dtype):
                 G.compare(c.t, ref, dtype, f"a.B^T ({k},{n})", rowwise=False, scale=scale)
                 for gd in (x, v, s, d, b, c, row):
                     gd.check("long rows")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_sums_and_products_of_tall_narrow_matrices(dtype):
+    """Rows of one element up to a few packs: row sums and A.v take a thread (or 2, 4, 8 lanes) per
+    row, column sums and v.A as many lanes per row as the row has packs, broadcasts the flat kernel."""
+    r = rng(37)
+    with G.BlasStream() as stream:
+        for (m, n, shift) in [(70001, 1, 0), (50003, 2, 1), (40001, 3, 0), (30011, 4, 0), (30011, 5, 1), (20001, 7, 0),
+                              (20000, 8, 0), (9001, 9, 1), (9001, 15, 0), (8192, 16, 0), (7001, 17, 0), (5003, 31, 1),
+                              (4096, 32, 0), (5003, 33, 0), (3001, 63, 0), (3001, 65, 1), (2049, 127, 0), (3, 5, 0)]:
+            for alpha in (0.0, 0.75):
+                G.say(f"narrow dtype={dtype} shape=({m},{n}) shift={shift} alpha={alpha}")
+                x = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+                xh = G.host(x.t)
+                si, sj = G.dev(r.normal(0, 1, m), dtype), G.dev(r.normal(0, 1, n), dtype, shift)
+                bi, bj = G.host(si.t).copy(), G.host(sj.t).copy()
+                stream.matrix_op("reduce_ij_i", x.t, si.t, alpha, m, n)
+                stream.matrix_op("reduce_ij_j", x.t, sj.t, alpha, m, n)
+                ax = np.abs(xh.astype(np.float64))
+                G.compare(si.t, O.reduce_ij_i(xh, bi if alpha else None, alpha), dtype, f"row sums ({m},{n})",
+                          rowwise=False, scale=ax.sum(axis=1) + abs(alpha) * np.abs(bi.astype(np.float64)))
+                G.compare(sj.t, O.reduce_ij_j(xh, bj if alpha else None, alpha), dtype, f"column sums ({m},{n})",
+                          rowwise=False, scale=ax.sum(axis=0) + abs(alpha) * np.abs(bj.astype(np.float64)))
+                # A.v: one dot product a row; u.A: the rows weighted and summed
+                v, d = G.dev(r.normal(0, 1, (n, 1)), dtype, shift), G.dev(r.normal(0, 1, (m, 1)), dtype)
+                u, e = G.dev(r.normal(0, 1, (1, m)), dtype), G.dev(r.normal(0, 1, (1, n)), dtype, shift)
+                bd, be = G.host(d.t).copy(), G.host(e.t).copy()
+                stream.inner_product("ij_jk_ik", x.t, v.t, 1.0, d.t, alpha, m, n, 1)
+                stream.inner_product("ij_jk_ik", u.t, x.t, -0.5, e.t, alpha, 1, m, n)
+                ref, scale = O.inner_product(xh, G.host(v.t), 1.0, bd if alpha else None, alpha, with_scale=True)
+                G.compare(d.t, ref, dtype, f"A.v ({m},{n})", rowwise=False, scale=scale)
+                ref, scale = O.inner_product(G.host(u.t), xh, -0.5, be if alpha else None, alpha, with_scale=True)
+                G.compare(e.t, ref, dtype, f"u.A ({m},{n})", rowwise=False, scale=scale)
+                # the reverses: both broadcasts into a copy of the matrix
+                for op, vec in (("broadcast_i_ij", si), ("broadcast_j_ij", sj)):
+                    y = G.dev(xh.astype(np.float64), dtype, shift)
+                    stream.matrix_op(op, vec.t, y.t, alpha, m, n)
+                    ref = getattr(O, op)(G.host(vec.t), m, n, xh if alpha else None, alpha)
+                    G.compare(y.t, ref, dtype, f"{op} ({m},{n})")
+                    y.check(op)
+                for gd in (x, si, sj, v, d, u, e):
+                    gd.check("narrow")
