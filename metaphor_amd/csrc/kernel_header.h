@@ -215,6 +215,57 @@ __device__ __forceinline__ void store_pack_nt_loose(T* p, const P (&in)[W]) {
   __builtin_nontemporal_store(v, reinterpret_cast<typename loose_vec_of<T, W>::type*>(p));
 }
 
+/* The first c < W elements of a pack that starts at any element, moved as pieces of W/2, W/4 ... 1
+ * elements picked by the bits of c: the end of a row that is not a whole number of packs long,
+ * without touching the row behind it. c = n % W is the same for every row, so the branches are
+ * uniform. The load sets the elements from c on to `fill`. */
+template <class T, int W, int OFF, int N, class P>
+__device__ __forceinline__ void load_cut_pack_from(const T* p, P (&out)[W], unsigned c) {
+  if constexpr (N >= 1) {
+    if (c & N) {
+      if constexpr (N == 1) {
+        out[OFF] = (P)p[OFF];
+      } else {
+        P piece[N];
+        load_pack_loose<T, N>(p + OFF, piece);
+#pragma unroll
+        for (int i = 0; i < N; ++i) out[OFF + i] = piece[i];
+      }
+      load_cut_pack_from<T, W, OFF + N, N / 2>(p, out, c);
+    } else {
+      load_cut_pack_from<T, W, OFF, N / 2>(p, out, c);
+    }
+  }
+}
+template <class T, int W, class P>
+__device__ __forceinline__ void load_cut_pack(const T* p, P (&out)[W], unsigned c, P fill) {
+#pragma unroll
+  for (int i = 0; i < W; ++i) out[i] = fill;
+  load_cut_pack_from<T, W, 0, W / 2>(p, out, c);
+}
+template <class T, int W, int OFF, int N, class P>
+__device__ __forceinline__ void store_cut_pack_from(T* p, const P (&in)[W], unsigned c) {
+  if constexpr (N >= 1) {
+    if (c & N) {
+      if constexpr (N == 1) {
+        p[OFF] = (T)in[OFF];
+      } else {
+        P piece[N];
+#pragma unroll
+        for (int i = 0; i < N; ++i) piece[i] = in[OFF + i];
+        store_pack_loose<T, N>(p + OFF, piece);
+      }
+      store_cut_pack_from<T, W, OFF + N, N / 2>(p, in, c);
+    } else {
+      store_cut_pack_from<T, W, OFF, N / 2>(p, in, c);
+    }
+  }
+}
+template <class T, int W, class P>
+__device__ __forceinline__ void store_cut_pack(T* p, const P (&in)[W], unsigned c) {
+  store_cut_pack_from<T, W, 0, W / 2>(p, in, c);
+}
+
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline unsigned misalign16(const void* p) { return (unsigned)(reinterpret_cast<uintptr_t>(p) & 15u); }
 

@@ -6,6 +6,8 @@
  * HBM once. HBM streams fastest here with many small waves each moving one or two packs, so
  * the plan takes the narrowest group that covers the row at a target NV (2 for softmax, 1 for
  * RMSNorm) and only lets NV grow once the group is 1024 threads wide:
+ *   short rows         up to 16 packs: 1, 2, 4, 8 or 16 lanes a row, a pack a lane, packs that
+ *                      start at the row's first element whatever its alignment (ShortRow);
  *   G = 8, 16, 32      several short rows per wavefront, DPP reductions inside 8-, 16- or
  *                      32-lane parts of the wave, so rows of a few hundred bytes keep all lanes busy
  *                      (8 lanes only for rows of at most eight packs, one pack a lane);
@@ -124,6 +126,69 @@ __device__ __forceinline__ unsigned xcd_contiguous_block(unsigned block, unsigne
   return xcd * per + (xcd < rem ? xcd : rem) + idx;
 }
 template <class T> inline unsigned rows_share_lines(size_t n) { return (n * sizeof(T)) % 128 != 0 ? 1u : 0u; }
+
+/* ---------------------------------------------------------------------------------------
+ * short rows: up to SHORT_MAX_PACKS packs, a pack a lane, 1, 2, 4, 8 or 16 lanes a row
+ * ------------------------------------------------------------------------------------- */
+
+constexpr int SHORT_MAX_PACKS = 16;
+constexpr int SHORT_THREADS = 256;
+
+inline unsigned short_row_grid(size_t m, int G) {
+  const size_t blocks = (m * (size_t)G + SHORT_THREADS - 1) / SHORT_THREADS;
+  require(blocks < 0x7fffffffull, "row launch: too many rows for one grid");
+  return (unsigned)blocks;
+}
+
+/* f.template operator()<G>() for the lanes a row of `packs` packs takes: the next power of two */
+template <class F> inline void for_short_row(size_t packs, F&& f) {
+  if (packs <= 1) f.template operator()<1>();
+  else if (packs <= 2) f.template operator()<2>();
+  else if (packs <= 4) f.template operator()<4>();
+  else if (packs <= 8) f.template operator()<8>();
+  else f.template operator()<16>();
+}
+
+/* A row of up to G packs in the registers of G lanes, a pack each, so that a wavefront's access
+ * is one contiguous kilobyte (two packs a lane over half the lanes: r32 n = 16 3.3 instead of
+ * 5.8 TB/s). Packs start at the row's first element whatever its alignment (one 128-bit access
+ * all the same), so rows of any length and base need no lanes for a head and a tail; the pack
+ * that the end of the row cuts moves in pieces (load_cut_pack). The groups wide rows take would
+ * leave most lanes idle here (measured, softmax r16 [4M, 8]: 1.1 TB/s at 8 lanes a row, 4.7 at
+ * one). */
+template <class T, int W, int G> struct ShortRow {
+  using P = typename precision<T>::type;
+  P v[W];
+
+  __device__ __forceinline__ void load(const T* row, unsigned n, int lane, P fill) {
+    const unsigned j = (unsigned)lane * W;
+    if (j + W <= n) load_pack_nt_loose<T, W>(row + j, v);
+    else if (j < n) load_cut_pack<T, W>(row + j, v, n - j, fill);
+    else
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[i] = fill;
+  }
+  __device__ __forceinline__ void store(T* row, unsigned n, int lane) const {
+    const unsigned j = (unsigned)lane * W;
+    if (j + W <= n) store_pack_nt_loose<T, W>(row + j, v);
+    else if (j < n) store_cut_pack<T, W>(row + j, v, n - j);
+  }
+};
+
+/* The row of this thread's group and whether it exists: a dead group of a live wavefront works
+ * on the last row, because the cross-lane steps need every lane, and stores nothing. Workgroups
+ * whose rows end inside a cache line are numbered so that neighbours share an L2. */
+template <int G> __device__ __forceinline__ size_t short_row_of(size_t m, unsigned by_xcd, bool& live) {
+  const unsigned block = by_xcd ? xcd_contiguous_block(blockIdx.x, gridDim.x) : blockIdx.x;
+  const size_t want = ((size_t)block * SHORT_THREADS + threadIdx.x) / G;
+  live = want < m;
+  return live ? want : m - 1;
+}
+
+/* whether the rows of one short-row workgroup end inside a cache line */
+template <class T> inline unsigned short_rows_share_lines(size_t n, int G) {
+  return ((size_t)(SHORT_THREADS / G) * n * sizeof(T)) % 128 != 0 ? 1u : 0u;
+}
 
 /* workgroups for m rows when a workgroup of max(G, 64) threads holds max(1, 64 / G) rows */
 inline unsigned row_grid(size_t m, int G) {

@@ -27,6 +27,64 @@
 
 namespace mp {
 
+/* ------------------------------------------------------------------ short rows */
+
+template <class T, int W, int G>
+__global__ __launch_bounds__(SHORT_THREADS) void softmax_fwd_short(const T* x, T* y, size_t m, unsigned n, unsigned by_xcd) {
+  using P = typename precision<T>::type;
+  const int lane = threadIdx.x % G;
+  bool live;
+  const size_t row = short_row_of<G>(m, by_xcd, live);
+  ShortRow<T, W, G> t;
+  t.load(x + row * n, n, lane, neg_inf<P>());
+
+  P mx = neg_inf<P>();
+#pragma unroll
+  for (int i = 0; i < W; ++i) mx = t.v[i] > mx ? t.v[i] : mx;
+  mx = fold_partials<MaxOP, G>(mx);
+
+  const P sh = shift_of(mx);
+  P s = (P)0;
+#pragma unroll
+  for (int i = 0; i < W; ++i) {
+    t.v[i] = exp_shifted(t.v[i], sh);
+    s += t.v[i];
+  }
+  s = fold_partials<AddOP, G>(s);
+
+  const P inv = (P)1 / s;
+#pragma unroll
+  for (int i = 0; i < W; ++i) t.v[i] *= inv;
+  if (live) t.store(y + row * n, n, lane);
+}
+
+template <class T, int W, int G, bool BLEND>
+__global__ __launch_bounds__(SHORT_THREADS) void softmax_rev_short(
+    const T* y, const T* dy, T* dx, typename precision<T>::type alpha, size_t m, unsigned n, unsigned by_xcd) {
+  using P = typename precision<T>::type;
+  const int lane = threadIdx.x % G;
+  bool live;
+  const size_t row = short_row_of<G>(m, by_xcd, live);
+  ShortRow<T, W, G> ty, tg;
+  ty.load(y + row * n, n, lane, (P)0);
+  tg.load(dy + row * n, n, lane, (P)0);
+
+  P dot = (P)0;
+#pragma unroll
+  for (int i = 0; i < W; ++i) dot += ty.v[i] * tg.v[i];
+  dot = fold_partials<AddOP, G>(dot);
+  if (!live) return; /* nothing below crosses lanes */
+
+#pragma unroll
+  for (int i = 0; i < W; ++i) ty.v[i] *= tg.v[i] - dot;
+  if constexpr (BLEND) {
+    tg.load(dx + row * n, n, lane, (P)0);
+#pragma unroll
+    for (int i = 0; i < W; ++i) ty.v[i] += alpha * tg.v[i];
+  }
+  ty.store(dx + row * n, n, lane);
+}
+
 /* ------------------------------------------------------------------ resident forward */
 
 template <class T, int W, int G, int NV, bool RAGGED>
@@ -653,12 +711,33 @@ inline unsigned stream_grid(size_t m) {
   return (unsigned)(m < cap ? m : cap);
 }
 
+/* Whether the short-row kernels take rows of n elements: up to four packs always, up to sixteen
+ * when no pack is cut (n % W == 0, whatever the base alignments) and up to eight for two-byte
+ * values; the other rows of five to sixteen packs that are not whole packs would leave lanes
+ * idle next to a cut pack, and the 16-lane groups with head and tail lanes are faster there
+ * (measured forward/reverse on [1M, 33] r32, nine packs: 3.6/4.3 TB/s there, 2.9/3.3 here; r16 n = 100,
+ * thirteen packs: 3.2/3.8 there, 3.1/2.9 here; but r16 n = 33, five packs: 1.6/1.8 there, 2.2/2.0 here). */
+template <class T> inline bool softmax_short_rows(size_t n) {
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  const size_t packs = (n + W - 1) / W;
+  if (row_regime_override() != REGIME_AUTO || packs > (size_t)SHORT_MAX_PACKS) return false;
+  return packs <= 4 || n % W == 0 || (sizeof(T) == 2 && packs <= 8);
+}
+
 template <class T>
 inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n, hipStream_t stream) {
   if (m == 0 || n == 0) return;
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "softmax: row length must not exceed 2^30");
+  if (softmax_short_rows<T>(n)) {
+    for_short_row((n + W - 1) / W, [&]<int G>() {
+      softmax_fwd_short<T, W, G><<<dim3(short_row_grid(m, G)), dim3(SHORT_THREADS), 0, stream>>>(
+          x, y, m, (unsigned)n, short_rows_share_lines<T>(n, G));
+    });
+    MP_CHECK_LAUNCH();
+    return;
+  }
   if (misalign16(x) != misalign16(y)) { /* rows of x and y peel differently: element-wise */
     softmax_fwd_stream<T, 1><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
     MP_CHECK_LAUNCH();
@@ -685,7 +764,7 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   }
   const bool ragged = !(aligned16(x) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(64);
-  RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, ragged ? 16 : 8);
+  RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, 16);
   if (row_regime_override() == REGIME_AUTO && sizeof(T) == 4 && packs > 2048 && packs <= 512 * 16)
     plan = RowPlan{packs <= 256 * 16 ? 256 : 512, 16}; /* see cluster_size */
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
@@ -726,6 +805,16 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   require(n <= 0x40000000ull, "softmax reverse: row length must not exceed 2^30");
   const P al = (P)alpha;
   const bool blend = alpha != 0.0;
+  if (softmax_short_rows<T>(n)) {
+    for_short_row((n + W - 1) / W, [&]<int G>() {
+      const dim3 grid(short_row_grid(m, G)), block(SHORT_THREADS);
+      const unsigned by_xcd = short_rows_share_lines<T>(n, G);
+      if (blend) softmax_rev_short<T, W, G, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, (unsigned)n, by_xcd);
+      else softmax_rev_short<T, W, G, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, (unsigned)n, by_xcd);
+    });
+    MP_CHECK_LAUNCH();
+    return;
+  }
   if (misalign16(y) != misalign16(dy) || misalign16(y) != misalign16(dx)) {
     const dim3 grid(stream_grid(m)), block(STREAM_THREADS);
     if (blend) softmax_rev_stream<T, 1, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
@@ -754,7 +843,7 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   }
   const bool ragged = !(aligned16(y) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, ragged ? 16 : 8);
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, 16);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) {

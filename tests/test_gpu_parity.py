@@ -526,6 +526,38 @@ def test_softmax_reverse_unaligned(dtype):
             dx.check("dx")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_softmax_short_rows_any_length_and_alignment(dtype):
+    """Rows of one element up to sixteen packs and a little beyond: 1 ... 16 lanes a row, packs
+    from the row's first element, cut packs in pieces; every length, bases shifted apart, in
+    place, with the reverse's alpha blend, and row counts that leave part of a wavefront dead."""
+    r = rng(43)
+    lengths = list(range(1, 36)) + [40, 47, 48, 56, 63, 64, 65, 72, 96, 100, 120, 127, 128, 129, 136]
+    for n in lengths:
+        for (m, shifts) in [(1001, (0, 0, 0)), (77, (1, 3, 2)), (3, (2, 2, 2))]:
+            G.say(f"softmax short dtype={dtype} shape=({m},{n}) shifts={shifts}")
+            x = G.dev(r.normal(0, 3, (m, n)), dtype, shifts[0])
+            y = G.Guarded((m, n), dtype, shifts[1])
+            G.softmax(x.t, y.t)
+            xh = G.host(x.t)
+            G.compare(y.t, O.softmax_ij_j(xh), dtype, f"softmax short ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
+            x.check("x")
+            y.check("y")
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[2])
+            yh, dyh = G.host(y.t), G.host(dy.t)
+            for alpha in (0.0, -0.5):
+                dx = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[0])
+                before = G.host(dx.t).copy()
+                G.softmax_reverse(y.t, dy.t, dx.t, alpha)
+                ref = O.softmax_ij_j_reverse(yh, dyh, before if alpha else None, alpha)
+                G.compare(dx.t, ref, dtype, f"softmax short reverse ({m},{n}) alpha={alpha}",
+                          scale=G.softmax_reverse_scale(yh, dyh, before if alpha else None, alpha))
+                dx.check("dx")
+            G.softmax(x.t, x.t)
+            G.compare(x.t, O.softmax_ij_j(xh), dtype, f"softmax short in place ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
+            x.check("in place")
+
+
 # ------------------------------------------------------------------ RMSNorm
 
 NORM_SHAPES = [(1, 1), (3, 7), (17, 64), (1031, 16), (259, 128), (33, 256), (64, 4096), (5, 1000), (300, 1024), (3, 50257),
