@@ -218,7 +218,7 @@ __device__ __forceinline__ void store_pack_nt_loose(T* p, const P (&in)[W]) {
 /* The first c < W elements of a pack that starts at any element, moved as pieces of W/2, W/4 ... 1
  * elements picked by the bits of c: the end of a row that is not a whole number of packs long,
  * without touching the row behind it. c = n % W is the same for every row, so the branches are
- * uniform. The load sets the elements from c on to `fill`. */
+ * uniform. The load leaves the elements from c on as they are. */
 template <class T, int W, int OFF, int N, class P>
 __device__ __forceinline__ void load_cut_pack_from(const T* p, P (&out)[W], unsigned c) {
   if constexpr (N >= 1) {
@@ -236,12 +236,6 @@ __device__ __forceinline__ void load_cut_pack_from(const T* p, P (&out)[W], unsi
       load_cut_pack_from<T, W, OFF, N / 2>(p, out, c);
     }
   }
-}
-template <class T, int W, class P>
-__device__ __forceinline__ void load_cut_pack(const T* p, P (&out)[W], unsigned c, P fill) {
-#pragma unroll
-  for (int i = 0; i < W; ++i) out[i] = fill;
-  load_cut_pack_from<T, W, 0, W / 2>(p, out, c);
 }
 template <class T, int W, int OFF, int N, class P>
 __device__ __forceinline__ void store_cut_pack_from(T* p, const P (&in)[W], unsigned c) {

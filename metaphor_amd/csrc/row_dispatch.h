@@ -140,38 +140,53 @@ inline unsigned short_row_grid(size_t m, int G) {
   return (unsigned)blocks;
 }
 
-/* f.template operator()<G>() for the lanes a row of `packs` packs takes: the next power of two */
-template <class F> inline void for_short_row(size_t packs, F&& f) {
-  if (packs <= 1) f.template operator()<1>();
-  else if (packs <= 2) f.template operator()<2>();
-  else if (packs <= 4) f.template operator()<4>();
-  else if (packs <= 8) f.template operator()<8>();
-  else f.template operator()<16>();
+/* f.template operator()<G, CUT>() for rows of n elements in packs of W: G, the lanes a row, is the
+ * next power of two from its packs; CUT says that the last pack is cut (code for it costs the
+ * rows of whole packs 10 % when compiled in: r16 n = 48 3.8 -> 4.2 TB/s without). */
+template <class F> inline void for_short_row(size_t n, int W, F&& f) {
+  const size_t packs = (n + W - 1) / W;
+#define MP_SHORT_LANES(CUT_)                          \
+  do {                                                \
+    if (packs <= 1) f.template operator()<1, CUT_>(); \
+    else if (packs <= 2) f.template operator()<2, CUT_>(); \
+    else if (packs <= 4) f.template operator()<4, CUT_>(); \
+    else if (packs <= 8) f.template operator()<8, CUT_>(); \
+    else f.template operator()<16, CUT_>();           \
+  } while (0)
+  if (n % W != 0) MP_SHORT_LANES(true);
+  else MP_SHORT_LANES(false);
+#undef MP_SHORT_LANES
 }
 
 /* A row of up to G packs in the registers of G lanes, a pack each, so that a wavefront's access
  * is one contiguous kilobyte (two packs a lane over half the lanes: r32 n = 16 3.3 instead of
  * 5.8 TB/s). Packs start at the row's first element whatever its alignment (one 128-bit access
  * all the same), so rows of any length and base need no lanes for a head and a tail; the pack
- * that the end of the row cuts moves in pieces (load_cut_pack). The groups wide rows take would
+ * that the end of the row cuts moves in pieces (load_cut_pack_from). The groups wide rows take would
  * leave most lanes idle here (measured, softmax r16 [4M, 8]: 1.1 TB/s at 8 lanes a row, 4.7 at
  * one). */
-template <class T, int W, int G> struct ShortRow {
+template <class T, int W, int G, bool CUT> struct ShortRow {
   using P = typename precision<T>::type;
   P v[W];
 
-  __device__ __forceinline__ void load(const T* row, unsigned n, int lane, P fill) {
+  /* NT: the row is read once (a streaming load); false for a vector that every row reuses */
+  template <bool NT = true> __device__ __forceinline__ void load(const T* row, unsigned n, int lane, P fill) {
     const unsigned j = (unsigned)lane * W;
-    if (j + W <= n) load_pack_nt_loose<T, W>(row + j, v);
-    else if (j < n) load_cut_pack<T, W>(row + j, v, n - j, fill);
-    else
+    if (j + W <= n) {
+      if constexpr (NT) load_pack_nt_loose<T, W>(row + j, v);
+      else load_pack_loose<T, W>(row + j, v);
+    } else {
 #pragma unroll
       for (int i = 0; i < W; ++i) v[i] = fill;
+      if constexpr (CUT)
+        if (j < n) load_cut_pack_from<T, W, 0, W / 2>(row + j, v, n - j);
+    }
   }
   __device__ __forceinline__ void store(T* row, unsigned n, int lane) const {
     const unsigned j = (unsigned)lane * W;
     if (j + W <= n) store_pack_nt_loose<T, W>(row + j, v);
-    else if (j < n) store_cut_pack<T, W>(row + j, v, n - j);
+    else if constexpr (CUT)
+      if (j < n) store_cut_pack<T, W>(row + j, v, n - j);
   }
 };
 

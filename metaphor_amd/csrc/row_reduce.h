@@ -108,37 +108,28 @@ __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
   if (live && lane == 0) dst[q] = (O)(blend != (P)0 ? scale * s + blend * (P)dst[q] : scale * s);
 }
 
-/* Rows of up to sixteen packs: G = 1, 2, 4 or 8 lanes a row, each with up to SHORT_ROW_PACKS
- * packs that start at any element (so no row needs lanes for a head and a tail); the pack that
- * the end of the row cuts is read element by element. Groups as wide as the longer rows take
- * would leave most lanes idle (measured on r32 [16M, 2]: 0.07 TB/s with sixteen lanes a row). */
-constexpr int SHORT_ROW_PACKS = 2;
-
-template <class T, class O, int W, int G, bool DOT>
-__global__ __launch_bounds__(256) void reduce_short_rows_kernel(
+/* Rows of up to sixteen packs: a pack a lane, 1 ... 16 lanes a row (ShortRow). Groups as wide as
+ * the longer rows take would leave most lanes idle (measured on r32 [16M, 2]: 0.07 TB/s with
+ * sixteen lanes a row). */
+template <class T, class O, int W, int G, bool CUT, bool DOT>
+__global__ __launch_bounds__(SHORT_THREADS) void reduce_short_rows_kernel(
     const T* src, const T* vec, O* dst, typename precision<T>::type scale, typename precision<T>::type blend,
     size_t rows, unsigned n) {
   using P = typename precision<T>::type;
   const int lane = threadIdx.x % G;
-  const size_t want = ((size_t)blockIdx.x * 256 + threadIdx.x) / G;
-  const bool live = want < rows; /* a dead group of a live wavefront reads the last row and stores nothing */
-  const size_t row = live ? want : rows - 1;
-  const T* r = src + row * n;
+  bool live;
+  const size_t row = short_row_of<G>(rows, 0, live);
+  ShortRow<T, W, G, CUT> a;
+  a.load(src + row * n, n, lane, (P)0);
   P s = (P)0;
+  if constexpr (DOT) {
+    ShortRow<T, W, G, CUT> b;
+    b.template load<false>(vec, n, lane, (P)0);
 #pragma unroll
-  for (int k = 0; k < SHORT_ROW_PACKS; ++k) {
-    const unsigned j = (unsigned)(lane + k * G) * W;
-    if (j + W <= n) {
-      P a[W], b[W];
-      load_pack_nt_loose<T, W>(r + j, a);
-      if constexpr (DOT) load_pack_loose<T, W>(vec + j, b);
+    for (int i = 0; i < W; ++i) s += a.v[i] * b.v[i];
+  } else {
 #pragma unroll
-      for (int i = 0; i < W; ++i) s += DOT ? a[i] * b[i] : a[i];
-    } else {
-#pragma unroll
-      for (int i = 0; i < W - 1; ++i)
-        if (j + i < n) s += DOT ? (P)r[j + i] * (P)vec[j + i] : (P)r[j + i];
-    }
+    for (int i = 0; i < W; ++i) s += a.v[i];
   }
   s = fold_partials<AddOP, G>(s);
   if (live && lane == 0) dst[row] = (O)(blend != (P)0 ? scale * s + blend * (P)dst[row] : scale * s);
@@ -152,19 +143,12 @@ inline void launch_reduce_rows(const S* src, const S* vec, O* dst, double scale,
   constexpr int W = PACK_BYTES / (int)sizeof(S);
   const size_t segments = rows * chunks;
   require(segments < 0x7fffffffull, "row sums: too many rows for one grid");
-  if (chunks == 1 && n <= (size_t)(8 * SHORT_ROW_PACKS * W)) {
-    const size_t row_packs = (n + W - 1) / W;
-#define MP_SHORT_ROWS(G_)                                                                                           \
-  do {                                                                                                              \
-    const dim3 grid((unsigned)((rows * G_ + 255) / 256)), block(256);                                               \
-    if (vec) reduce_short_rows_kernel<S, O, W, G_, true><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, rows, (unsigned)n); \
-    else reduce_short_rows_kernel<S, O, W, G_, false><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, rows, (unsigned)n);   \
-  } while (0)
-    if (row_packs <= 1 * SHORT_ROW_PACKS) MP_SHORT_ROWS(1);
-    else if (row_packs <= 2 * SHORT_ROW_PACKS) MP_SHORT_ROWS(2);
-    else if (row_packs <= 4 * SHORT_ROW_PACKS) MP_SHORT_ROWS(4);
-    else MP_SHORT_ROWS(8);
-#undef MP_SHORT_ROWS
+  if (chunks == 1 && n <= (size_t)(SHORT_MAX_PACKS * W)) {
+    for_short_row(n, W, [&]<int G, bool CUT>() {
+      const dim3 grid(short_row_grid(rows, G)), block(SHORT_THREADS);
+      if (vec) reduce_short_rows_kernel<S, O, W, G, CUT, true><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, rows, (unsigned)n);
+      else reduce_short_rows_kernel<S, O, W, G, CUT, false><<<grid, block, 0, stream>>>(src, vec, dst, (P)scale, (P)blend, rows, (unsigned)n);
+    });
     MP_CHECK_LAUNCH();
     return;
   }

@@ -29,13 +29,13 @@ namespace mp {
 
 /* ------------------------------------------------------------------ short rows */
 
-template <class T, int W, int G>
+template <class T, int W, int G, bool CUT>
 __global__ __launch_bounds__(SHORT_THREADS) void softmax_fwd_short(const T* x, T* y, size_t m, unsigned n, unsigned by_xcd) {
   using P = typename precision<T>::type;
   const int lane = threadIdx.x % G;
   bool live;
   const size_t row = short_row_of<G>(m, by_xcd, live);
-  ShortRow<T, W, G> t;
+  ShortRow<T, W, G, CUT> t;
   t.load(x + row * n, n, lane, neg_inf<P>());
 
   P mx = neg_inf<P>();
@@ -58,14 +58,14 @@ __global__ __launch_bounds__(SHORT_THREADS) void softmax_fwd_short(const T* x, T
   if (live) t.store(y + row * n, n, lane);
 }
 
-template <class T, int W, int G, bool BLEND>
+template <class T, int W, int G, bool CUT, bool BLEND>
 __global__ __launch_bounds__(SHORT_THREADS) void softmax_rev_short(
     const T* y, const T* dy, T* dx, typename precision<T>::type alpha, size_t m, unsigned n, unsigned by_xcd) {
   using P = typename precision<T>::type;
   const int lane = threadIdx.x % G;
   bool live;
   const size_t row = short_row_of<G>(m, by_xcd, live);
-  ShortRow<T, W, G> ty, tg;
+  ShortRow<T, W, G, CUT> ty, tg;
   ty.load(y + row * n, n, lane, (P)0);
   tg.load(dy + row * n, n, lane, (P)0);
 
@@ -715,8 +715,9 @@ inline unsigned stream_grid(size_t m) {
  * when no pack is cut (n % W == 0, whatever the base alignments) and up to eight for two-byte
  * values; the other rows of five to sixteen packs that are not whole packs would leave lanes
  * idle next to a cut pack, and the 16-lane groups with head and tail lanes are faster there
- * (measured forward/reverse on [1M, 33] r32, nine packs: 3.6/4.3 TB/s there, 2.9/3.3 here; r16 n = 100,
- * thirteen packs: 3.2/3.8 there, 3.1/2.9 here; but r16 n = 33, five packs: 1.6/1.8 there, 2.2/2.0 here). */
+ * (measured forward/reverse on [1M, 33] r32, nine packs: 3.5/4.2 TB/s there, 2.8/3.3 here; r32 n = 50: 4.6/4.6
+ * there, 4.2/4.4 here; r16 n = 100, thirteen packs: 3.2/3.7 there, 3.2/3.0 here; but r16 n = 33, five packs:
+ * 1.5/1.8 there, 2.2/2.1 here, and r16 n = 50: 2.0/2.3 there, 2.9/2.8 here). */
 template <class T> inline bool softmax_short_rows(size_t n) {
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   const size_t packs = (n + W - 1) / W;
@@ -731,8 +732,8 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "softmax: row length must not exceed 2^30");
   if (softmax_short_rows<T>(n)) {
-    for_short_row((n + W - 1) / W, [&]<int G>() {
-      softmax_fwd_short<T, W, G><<<dim3(short_row_grid(m, G)), dim3(SHORT_THREADS), 0, stream>>>(
+    for_short_row(n, W, [&]<int G, bool CUT>() {
+      softmax_fwd_short<T, W, G, CUT><<<dim3(short_row_grid(m, G)), dim3(SHORT_THREADS), 0, stream>>>(
           x, y, m, (unsigned)n, short_rows_share_lines<T>(n, G));
     });
     MP_CHECK_LAUNCH();
@@ -806,11 +807,11 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   const P al = (P)alpha;
   const bool blend = alpha != 0.0;
   if (softmax_short_rows<T>(n)) {
-    for_short_row((n + W - 1) / W, [&]<int G>() {
+    for_short_row(n, W, [&]<int G, bool CUT>() {
       const dim3 grid(short_row_grid(m, G)), block(SHORT_THREADS);
       const unsigned by_xcd = short_rows_share_lines<T>(n, G);
-      if (blend) softmax_rev_short<T, W, G, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, (unsigned)n, by_xcd);
-      else softmax_rev_short<T, W, G, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, (unsigned)n, by_xcd);
+      if (blend) softmax_rev_short<T, W, G, CUT, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, (unsigned)n, by_xcd);
+      else softmax_rev_short<T, W, G, CUT, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, (unsigned)n, by_xcd);
     });
     MP_CHECK_LAUNCH();
     return;
