@@ -198,16 +198,148 @@ __global__ __launch_bounds__(tp_threads<T>()) void permutate_kernel(
   }
 }
 
+/* ------------------------------------------------------------------ narrow matrices */
+
+/* A matrix with a short side of n <= TP_NARROW_MAX: [m, n] is an array of m records of n fields
+ * (AoS), its transpose [n, m] one array per field (SoA). The tall tile above would use n of its
+ * 8 packs of columns, or n of its 64 packs of rows (measured r32: [4M, 4] 2.5 TB/s, [4, 4M] 0.4).
+ * Here a workgroup moves a chunk of R records: the AoS side is one contiguous run of R * n
+ * elements, moved as linear packs, the SoA side n runs of R elements; in between the chunk lies in
+ * LDS in AoS order, one pad word after every 32 words so that the gathers and scatters with a stride
+ * of n elements spread over the banks. Packs on both sides start at any element. */
+constexpr size_t TP_NARROW_MAX = 64;
+constexpr int TP_NARROW_BYTES = 32768; /* of a chunk in LDS, pads aside */
+constexpr int TP_NARROW_THREADS = 256;
+
+/* records per chunk: what fits, in whole packs */
+template <class T> inline unsigned tp_narrow_records(size_t n) {
+  constexpr int W = pack_width<T>();
+  return (unsigned)(TP_NARROW_BYTES / sizeof(T) / n / W * W);
+}
+
+/* TO_SOA: src is [m, n] and dst [n, m]; otherwise src is [n, m] and dst [m, n]. */
+template <class T, bool TO_SOA, bool BLEND>
+__global__ __launch_bounds__(TP_NARROW_THREADS) void permutate_narrow_kernel(
+    const T* __restrict__ src, T* __restrict__ dst, typename precision<T>::type alpha, size_t m, unsigned n, unsigned R) {
+  using P = typename precision<T>::type;
+  constexpr int W = pack_width<T>(), THREADS = TP_NARROW_THREADS;
+  constexpr unsigned CAP = TP_NARROW_BYTES / sizeof(T);                   /* elements of a chunk */
+  constexpr unsigned BLOCK = 128 / sizeof(T);                             /* elements in 32 words */
+  constexpr unsigned PAD = sizeof(T) >= 4 ? 1 : 4 / sizeof(T);            /* elements of a pad: a word at least */
+  using V = typename vec_of<T, W>::type;
+  using VL = typename loose_vec_of<T, W>::type;
+  __shared__ T tile[CAP + CAP / BLOCK * PAD];
+  auto lds = [](unsigned e) -> unsigned { return e + e / BLOCK * PAD; };
+
+  const unsigned tid = threadIdx.x;
+  const size_t i0 = (size_t)blockIdx.x * R;
+  const unsigned here = m - i0 < (size_t)R ? (unsigned)(m - i0) : R; /* records of this chunk */
+  const unsigned count = here * n;                                   /* its elements */
+  const unsigned ppr = (here + W - 1) / W;                           /* packs of one SoA run, the last one maybe cut */
+  const T* aos_in = src + i0 * n;
+  T* aos_out = dst + i0 * n;
+  const T* soa_in = src + i0;
+  T* soa_out = dst + i0;
+
+  if constexpr (TO_SOA) {
+    for (unsigned e = tid * W; e < count; e += THREADS * W) {
+      if (e + W <= count) {
+        *reinterpret_cast<VL*>(&tile[lds(e)]) = __builtin_nontemporal_load(reinterpret_cast<const VL*>(aos_in + e));
+      } else {
+        for (unsigned k = e; k < count; ++k) tile[lds(k)] = aos_in[k];
+      }
+    }
+    __syncthreads();
+    for (unsigned q = tid; q < n * ppr; q += THREADS) {
+      const unsigned j = q / ppr, r0 = (q - j * ppr) * W;
+      const bool whole = r0 + W <= here;
+      V out;
+#pragma unroll
+      for (int r = 0; r < W; ++r) out[r] = r0 + r < here ? tile[lds((r0 + r) * n + j)] : (T)0;
+      T* to = soa_out + (size_t)j * m + r0;
+      if (whole) {
+        if constexpr (BLEND) {
+          const V old = *reinterpret_cast<const VL*>(to);
+#pragma unroll
+          for (int r = 0; r < W; ++r) out[r] = (T)((P)out[r] + alpha * (P)old[r]);
+        }
+        __builtin_nontemporal_store(out, reinterpret_cast<VL*>(to));
+      } else {
+#pragma unroll
+        for (int r = 0; r < W; ++r)
+          if (r0 + r < here) {
+            T x = out[r];
+            if constexpr (BLEND) x = (T)((P)x + alpha * (P)to[r]);
+            to[r] = x;
+          }
+      }
+    }
+  } else {
+    for (unsigned q = tid; q < n * ppr; q += THREADS) {
+      const unsigned j = q / ppr, r0 = (q - j * ppr) * W;
+      const T* from = soa_in + (size_t)j * m + r0;
+      V v;
+      if (r0 + W <= here) {
+        v = __builtin_nontemporal_load(reinterpret_cast<const VL*>(from));
+      } else {
+#pragma unroll
+        for (int r = 0; r < W; ++r) v[r] = r0 + r < here ? from[r] : (T)0;
+      }
+#pragma unroll
+      for (int r = 0; r < W; ++r)
+        if (r0 + r < here) tile[lds((r0 + r) * n + j)] = v[r];
+    }
+    __syncthreads();
+    for (unsigned e = tid * W; e < count; e += THREADS * W) {
+      T* to = aos_out + e;
+      if (e + W <= count) {
+        V out = *reinterpret_cast<const VL*>(&tile[lds(e)]);
+        if constexpr (BLEND) {
+          const V old = *reinterpret_cast<const VL*>(to);
+#pragma unroll
+          for (int r = 0; r < W; ++r) out[r] = (T)((P)out[r] + alpha * (P)old[r]);
+        }
+        __builtin_nontemporal_store(out, reinterpret_cast<VL*>(to));
+      } else {
+        for (unsigned k = e; k < count; ++k) {
+          T x = tile[lds(k)];
+          if constexpr (BLEND) x = (T)((P)x + alpha * (P)aos_out[k]);
+          aos_out[k] = x;
+        }
+      }
+    }
+  }
+}
+
 template <class T>
 inline void permutate(const T* src, T* dst, double alpha, size_t rows, size_t cols, hipStream_t stream) {
   if (rows == 0 || cols == 0) return;
   using P = typename precision<T>::type;
   constexpr int W = pack_width<T>(), TR = TP_ROW_PACKS * W, TC = TP_COL_PACKS * W;
   require(static_cast<const void*>(src) != static_cast<const void*>(dst), "permutate_ij_ji: source and destination must differ");
+  const bool blend = alpha != 0.0;
+  if (cols <= TP_NARROW_MAX || rows <= TP_NARROW_MAX) {
+    const bool to_soa = cols <= rows; /* the short side are the fields of a record */
+    const size_t m = to_soa ? rows : cols, n = to_soa ? cols : rows;
+    const unsigned R = tp_narrow_records<T>(n);
+    const size_t chunks = (m + R - 1) / R;
+    require(chunks < 0x7fffffffull, "permutate_ij_ji: too many chunks for one grid");
+    const dim3 grid((unsigned)chunks), block(TP_NARROW_THREADS);
+#define MP_TP_NARROW(TO_SOA)                                                                                      \
+  do {                                                                                                            \
+    if (blend) permutate_narrow_kernel<T, TO_SOA, true><<<grid, block, 0, stream>>>(src, dst, (P)alpha, m, (unsigned)n, R); \
+    else permutate_narrow_kernel<T, TO_SOA, false><<<grid, block, 0, stream>>>(src, dst, (P)alpha, m, (unsigned)n, R);      \
+  } while (0)
+    if (to_soa) MP_TP_NARROW(true);
+    else MP_TP_NARROW(false);
+#undef MP_TP_NARROW
+    MP_CHECK_LAUNCH();
+    return;
+  }
   const size_t tiles_r = (rows + TR - 1) / TR, tiles_c = (cols + TC - 1) / TC;
   require(tiles_r < 0x7fffffffull && tiles_c < 0x7fffffffull && tiles_r * tiles_c < 0x7fffffffull,
           "permutate_ij_ji: too many tiles for one grid");
-  const bool vin = aligned16(src) && cols % W == 0, vout = aligned16(dst) && rows % W == 0, blend = alpha != 0.0;
+  const bool vin = aligned16(src) && cols % W == 0, vout = aligned16(dst) && rows % W == 0;
   const dim3 grid((unsigned)(tiles_r * tiles_c)), block(tp_threads<T>());
   const unsigned tr = (unsigned)tiles_r; /* consecutive workgroups walk down a column band of the source */
 #define MP_TP_LAUNCH(VIN, VOUT)                                                                                  \

@@ -381,8 +381,12 @@ inline void reduce_cols(const T* src, T* dst, void* scratch, double alpha, size_
 }
 
 /* c[i,l] = scale * a[i] * b[l] + blend * c[i,l]: the product of a column and a row vector, written
- * like a broadcast (flat, one pack per thread) when c is pack-aligned. */
-template <class T, int W, bool BLEND>
+ * like a broadcast: c as one flat array, one pack per thread. ALIGNED: n % W == 0 and b 16-byte
+ * aligned, so a pack lies inside one row and its b values are one aligned pack; otherwise a pack
+ * may run over the end of its row (over several rows when n < W): the b values are then a pack
+ * that starts at any element, or, for a pack that wraps, single loads. DALIGNED: c is 16-byte
+ * aligned. The last workgroup also writes the m*n % W elements behind the last whole pack. */
+template <class T, int W, bool BLEND, bool ALIGNED, bool DALIGNED>
 __global__ __launch_bounds__(256) void outer_flat_kernel(
     const T* a, const T* b, T* c, typename precision<T>::type scale, typename precision<T>::type blend,
     size_t total, unsigned n) {
@@ -396,21 +400,36 @@ __global__ __launch_bounds__(256) void outer_flat_kernel(
     const size_t row = row0 + off / n;
     const unsigned col = off % n;
     P out[W];
+    if (ALIGNED || col + W <= n) {
+      if constexpr (ALIGNED) load_pack<T, W>(b + col, out);
+      else load_pack_loose<T, W>(b + col, out);
+      const P left = scale * (P)a[row];
 #pragma unroll
-    for (int i = 0; i < W; ++i) {
-      const bool next = col + i >= n; /* n >= W: a pack ends in the next row at most */
-      out[i] = scale * (P)a[row + (next ? 1 : 0)] * (P)b[next ? col + i - n : col + i];
+      for (int i = 0; i < W; ++i) out[i] *= left;
+    } else { /* walk the pack's elements: the row advances whenever the column reaches n */
+      size_t r = row;
+      unsigned l = col;
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        out[i] = scale * (P)a[r] * (P)b[l];
+        if (++l == n) {
+          l = 0;
+          ++r;
+        }
+      }
     }
     T* o = c + idx * W;
     if constexpr (BLEND) {
       P old[W];
-      load_pack_nt<T, W>(o, old);
+      if constexpr (DALIGNED) load_pack_nt<T, W>(o, old);
+      else load_pack_nt_loose<T, W>(o, old);
 #pragma unroll
       for (int i = 0; i < W; ++i) out[i] += blend * old[i];
     }
-    store_pack_nt<T, W>(o, out);
+    if constexpr (DALIGNED) store_pack_nt<T, W>(o, out);
+    else store_pack_nt_loose<T, W>(o, out);
   }
-  if (blockIdx.x == gridDim.x - 1) {
+  if (W > 1 && blockIdx.x == gridDim.x - 1) {
     const size_t e = packs * W + threadIdx.x;
     if (threadIdx.x < W && e < total) {
       P v = scale * (P)a[e / n] * (P)b[e % n];
@@ -424,20 +443,20 @@ template <class T>
 inline void outer_product(const T* a, const T* b, T* c, double scale, double blend, size_t m, size_t n, hipStream_t stream) {
   if (m == 0 || n == 0) return;
   using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "outer product: row length must not exceed 2^30");
-  const size_t total = m * n;
-  if (aligned16(c) && n >= (size_t)(PACK_BYTES / sizeof(T))) {
-    constexpr int W = PACK_BYTES / (int)sizeof(T);
-    const size_t blocks = (total / W + 255) / 256 + 1;
-    require(blocks < 0x7fffffffull, "outer product: too many elements for one grid");
-    if (blend != 0.0) outer_flat_kernel<T, W, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n);
-    else outer_flat_kernel<T, W, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n);
-  } else {
-    const size_t blocks = (total + 255) / 256 + 1;
-    require(blocks < 0x7fffffffull, "outer product: too many elements for one grid");
-    if (blend != 0.0) outer_flat_kernel<T, 1, true><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n);
-    else outer_flat_kernel<T, 1, false><<<dim3((unsigned)blocks), dim3(256), 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n);
-  }
+  const size_t total = m * n, blocks = (total / W + 255) / 256 + 1; /* + 1: the tail always has a workgroup */
+  require(blocks < 0x7fffffffull, "outer product: too many elements for one grid");
+  const dim3 grid((unsigned)blocks), block(256);
+  const bool aligned = n % W == 0 && aligned16(b);
+#define MP_OUTER_AS(BLEND_, ALIGNED_, DALIGNED_) \
+  outer_flat_kernel<T, W, BLEND_, ALIGNED_, DALIGNED_><<<grid, block, 0, stream>>>(a, b, c, (P)scale, (P)blend, total, (unsigned)n)
+#define MP_OUTER(BLEND_, ALIGNED_) \
+  do { if (aligned16(c)) MP_OUTER_AS(BLEND_, ALIGNED_, true); else MP_OUTER_AS(BLEND_, ALIGNED_, false); } while (0)
+  if (aligned) { if (blend != 0.0) MP_OUTER(true, true); else MP_OUTER(false, true); }
+  else { if (blend != 0.0) MP_OUTER(true, false); else MP_OUTER(false, false); }
+#undef MP_OUTER
+#undef MP_OUTER_AS
   MP_CHECK_LAUNCH();
 }
 

@@ -46,6 +46,30 @@ def test_permutate_forward_and_blend(dtype, shift):
             src.check("permutate src")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_permutate_narrow_matrices(dtype):
+    """A short side of up to 64: records to fields and back through the chunked kernel; chunk
+    boundaries (8192 / n records for r32), cut packs on either side, shifted bases, blend."""
+    r = rng(38)
+    for n in (1, 2, 3, 4, 5, 7, 8, 12, 16, 31, 33, 63, 64):
+        for (m, shifts) in ((1, (0, 0)), (6, (1, 0)), (1000, (0, 0)), (8193, (0, 1)), (40003, (1, 3))):
+            for (rows, cols) in ((m, n), (n, m)):
+                for alpha in (0.0, -0.5):
+                    G.say(f"permutate narrow dtype={dtype} shape=({rows},{cols}) alpha={alpha} shifts={shifts}")
+                    src = G.dev(r.normal(0, 1, (rows, cols)), dtype, shifts[0])
+                    dst = G.dev(r.normal(0, 1, (cols, rows)), dtype, shifts[1])
+                    before = G.host(dst.t).copy()
+                    G.permutate(src.t, dst.t, alpha)
+                    ref = O.permutate_ij_ji(G.host(src.t), before if alpha else None, alpha)
+                    if alpha == 0.0:
+                        assert np.array_equal(G.host(dst.t).astype(np.float64), ref), "transpose must move bits unchanged"
+                    else:
+                        G.compare(dst.t, ref, dtype, f"permutate ({rows},{cols}) alpha {alpha}", rowwise=False,
+                                  scale=np.abs(G.host(src.t).T.astype(np.float64)) + abs(alpha) * np.abs(before.astype(np.float64)))
+                    dst.check("permutate dst")
+                    src.check("permutate src")
+
+
 def test_permutate_mixed_alignment_and_empty():
     f32 = torch.float32
     r = rng(32)
@@ -233,12 +257,22 @@ def test_sums_and_products_of_tall_narrow_matrices(dtype):
                 G.compare(d.t, ref, dtype, f"A.v ({m},{n})", rowwise=False, scale=scale)
                 ref, scale = O.inner_product(G.host(u.t), xh, -0.5, be if alpha else None, alpha, with_scale=True)
                 G.compare(e.t, ref, dtype, f"u.A ({m},{n})", rowwise=False, scale=scale)
+                # the product of a column and a row vector, into a copy of the matrix
+                col, rowv = G.dev(r.normal(0, 1, (m, 1)), dtype), G.dev(r.normal(0, 1, (1, n)), dtype, shift)
+                c = G.dev(xh.astype(np.float64), dtype, shift)
+                stream.inner_product("ij_jk_ik", col.t, rowv.t, 0.5, c.t, alpha, m, 1, n)
+                ref, scale = O.inner_product(G.host(col.t), G.host(rowv.t), 0.5, xh if alpha else None, alpha, with_scale=True)
+                G.compare(c.t, ref, dtype, f"outer product ({m},{n})", rowwise=False, scale=scale)
+                for gd in (col, rowv, c):
+                    gd.check("outer product")
                 # the reverses: both broadcasts into a copy of the matrix
                 for op, vec in (("broadcast_i_ij", si), ("broadcast_j_ij", sj)):
                     y = G.dev(xh.astype(np.float64), dtype, shift)
                     stream.matrix_op(op, vec.t, y.t, alpha, m, n)
                     ref = getattr(O, op)(G.host(vec.t), m, n, xh if alpha else None, alpha)
-                    G.compare(y.t, ref, dtype, f"{op} ({m},{n})")
+                    vh = np.abs(G.host(vec.t).astype(np.float64))
+                    G.compare(y.t, ref, dtype, f"{op} ({m},{n})", rowwise=False,
+                              scale=(vh[:, None] if op == "broadcast_i_ij" else vh[None, :]) + abs(alpha) * ax)
                     y.check(op)
                 for gd in (x, si, sj, v, d, u, e):
                     gd.check("narrow")
