@@ -803,6 +803,114 @@ inline void sum_partial_rows(const typename precision<T>::type* partials, T* dst
   MP_CHECK_LAUNCH();
 }
 
+/* ------------------------------------------------------------------ short rows */
+
+/* Rows of up to sixteen packs (a norm over a head's few dozen values): a pack a lane, 1 ... 16
+ * lanes a row (ShortRow), one-shot workgroups of 256 threads. */
+template <class T, int W, int G, bool CUT>
+__global__ __launch_bounds__(SHORT_THREADS) void rmsnorm_fwd_short(
+    const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, unsigned n, unsigned by_xcd) {
+  using P = typename precision<T>::type;
+  const int lane = threadIdx.x % G;
+  bool live;
+  const size_t row = short_row_of<G>(m, by_xcd, live);
+  ShortRow<T, W, G, CUT> t, g;
+  t.load(x + row * n, n, lane, (P)0);
+  g.template load<false>(gain, n, lane, (P)0);
+  P ss = (P)0;
+#pragma unroll
+  for (int i = 0; i < W; ++i) ss += t.v[i] * t.v[i];
+  ss = fold_partials<AddOP, G>(ss);
+  const P r = rsqrt_of(ss / (P)n + eps);
+#pragma unroll
+  for (int i = 0; i < W; ++i) t.v[i] *= r * g.v[i];
+  if (live) t.store(y + row * n, n, lane);
+}
+
+/* The reverse walks the rows with gridDim.x workgroups of NORM_BLOCK threads, because every
+ * workgroup leaves one partial row of dg sums (partials holds gridDim.x rows of n values): the
+ * groups of a wavefront are folded with lane exchanges, the wavefronts through LDS in order. */
+template <class T, int W, int G, bool CUT, bool BLEND>
+__global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_short(
+    const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
+    typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, unsigned n) {
+  using P = typename precision<T>::type;
+  constexpr int RPB = NORM_BLOCK / G, WAVES = NORM_BLOCK / WAVE;
+  __shared__ P comb[WAVES][G * W];
+  const int lane = threadIdx.x % G, sub = threadIdx.x / G;
+  ShortRow<T, W, G, CUT> gv;
+  gv.template load<false>(gain, n, lane, (P)0);
+  P acc[W];
+#pragma unroll
+  for (int i = 0; i < W; ++i) acc[i] = (P)0;
+
+  for (size_t base = (size_t)blockIdx.x * RPB; base < m; base += (size_t)gridDim.x * RPB) {
+    const size_t want = base + sub;
+    const bool live = want < m; /* a dead group of a live wavefront reads the last row and keeps nothing */
+    const size_t off = (live ? want : m - 1) * n;
+    ShortRow<T, W, G, CUT> xv, dv;
+    xv.load(x + off, n, lane, (P)0);
+    dv.load(dy + off, n, lane, (P)0);
+    P ss = (P)0, c = (P)0;
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      ss += xv.v[i] * xv.v[i];
+      c += dv.v[i] * gv.v[i] * xv.v[i];
+    }
+    ss = fold_partials<AddOP, G>(ss);
+    c = fold_partials<AddOP, G>(c);
+    const P r = rsqrt_of(ss / (P)n + eps);
+    const P cc = c / (P)n * r * r;
+    if (live) {
+      ShortRow<T, W, G, CUT> out;
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        out.v[i] = r * (dv.v[i] * gv.v[i] - xv.v[i] * cc);
+        acc[i] += dv.v[i] * xv.v[i] * r;
+      }
+      if constexpr (BLEND) {
+        ShortRow<T, W, G, CUT> old;
+        old.template load<false>(dx + off, n, lane, (P)0);
+#pragma unroll
+        for (int i = 0; i < W; ++i) out.v[i] += alpha * old.v[i];
+      }
+      out.store(dx + off, n, lane);
+    }
+  }
+
+#pragma unroll
+  for (int i = 0; i < W; ++i) {
+#pragma unroll
+    for (int mask = G; mask < WAVE; mask <<= 1) acc[i] += __shfl_xor(acc[i], mask, WAVE);
+    if (threadIdx.x % WAVE < G) comb[threadIdx.x / WAVE][lane * W + i] = acc[i];
+  }
+  __syncthreads();
+  P* mine = partials + (size_t)blockIdx.x * n;
+  for (unsigned col = threadIdx.x; col < n; col += NORM_BLOCK) {
+    P t = (P)0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) t += comb[w][col];
+    mine[col] = t;
+  }
+}
+
+/* Whether the short-row kernels take rows of n elements. Up to four packs always (r32 [8M, 4]:
+ * 1.5/1.9 -> 5.7/5.2 TB/s forward/reverse, r16 [4M, 8]: 1.3/1.0 -> 4.3/4.3). From five to sixteen
+ * packs the groups of 8 and 16 lanes of the resident kernels are the same layout when the row
+ * fills them, and the measurements decide: r32 rows of whole packs gain forward (n = 64: 5.3 ->
+ * 5.6) and, below eight packs, in reverse (n = 24: 4.75 -> 4.87; n = 32 and 64 lose 6 %); r16 rows
+ * of whole packs gain in reverse (n = 64: 3.7 -> 4.5, n = 128: 4.4 -> 4.5) and lose 6 % forward; rows
+ * with a cut pack gain only forward in r16 up to eight packs (n = 33: 1.2 -> 1.7). */
+template <class T> inline bool rmsnorm_short_rows(size_t n, bool reverse) {
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  const size_t packs = (n + W - 1) / W;
+  const bool whole = n % W == 0;
+  if (row_regime_override() != REGIME_AUTO || packs > (size_t)SHORT_MAX_PACKS) return false;
+  if (packs <= 4) return true;
+  if (sizeof(T) == 2) return reverse ? whole : !whole && packs <= 8;
+  return whole && (!reverse || packs < 8);
+}
+
 /* ------------------------------------------------------------------ host dispatch */
 
 /* Partial rows the reverse may write: one per workgroup, at most two workgroups per CU. */
@@ -826,6 +934,14 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "rmsnorm: row length must not exceed 2^30");
   const size_t cap = (size_t)compute_units() * 2;
+  if (rmsnorm_short_rows<T>(n, false)) {
+    for_short_row(n, W, [&]<int G, bool CUT>() {
+      rmsnorm_fwd_short<T, W, G, CUT><<<dim3(short_row_grid(m, G)), dim3(SHORT_THREADS), 0, stream>>>(
+          x, gain, y, (P)eps, m, (unsigned)n, short_rows_share_lines<T>(n, G));
+    });
+    MP_CHECK_LAUNCH();
+    return;
+  }
   if (misalign16(x) != misalign16(y)) {
     const size_t grid = m < cap ? m : cap;
     rmsnorm_fwd_stream<T, 1><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
@@ -960,6 +1076,22 @@ inline void rmsnorm_reverse(const T* x, const T* gain, const T* dy, T* dx, T* dg
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   require(n <= 0x40000000ull, "rmsnorm reverse: row length must not exceed 2^30");
   require(scratch != nullptr, "rmsnorm reverse: scratch must hold mpRmsnormReverseScratchBytes bytes");
+  if (rmsnorm_short_rows<T>(n, true)) {
+    using P = typename precision<T>::type;
+    P* partials = static_cast<P*>(scratch);
+    const size_t max_rows = rmsnorm_reverse_partial_rows(m);
+    unsigned rows = 0;
+    for_short_row(n, W, [&]<int G, bool CUT>() {
+      const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
+      rows = (unsigned)(need < max_rows ? need : max_rows);
+      const dim3 grid(rows), block(NORM_BLOCK);
+      if (alpha != 0.0) rmsnorm_rev_short<T, W, G, CUT, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, (unsigned)n);
+      else rmsnorm_rev_short<T, W, G, CUT, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, (unsigned)n);
+    });
+    MP_CHECK_LAUNCH();
+    sum_partial_rows<T>(partials, dg, alpha, rows, n, stream);
+    return;
+  }
   const bool packed = aligned16(x) && aligned16(dy) && aligned16(dx) && aligned16(gain) && (n % W) == 0;
   if (packed) rmsnorm_reverse_as<T, false>(x, gain, dy, dx, dg, scratch, eps, alpha, m, n, stream);
   else rmsnorm_reverse_as<T, true>(x, gain, dy, dx, dg, scratch, eps, alpha, m, n, stream);

@@ -744,6 +744,42 @@ def test_rmsnorm_reverse_unaligned(dtype):
                 gd.check("rmsnorm rev unaligned")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rmsnorm_short_rows_any_length_and_alignment(dtype):
+    """Rows of one element up to sixteen packs and a little beyond, forward and reverse: 1 ... 16
+    lanes a row, packs from the row's first element, cut packs in pieces; bases shifted apart,
+    the alpha blend, in place, and row counts from three to more than the workgroups hold at once."""
+    r = rng(63)
+    eps = 1e-6
+    lengths = list(range(1, 20)) + [24, 31, 32, 33, 40, 47, 48, 63, 64, 65, 96, 100, 127, 128, 129, 136]
+    for n in lengths:
+        for (m, shifts) in [(3, (0, 0, 0, 0)), (1001, (1, 0, 3, 2)), (70001 if n <= 8 else 9001, (0, 1, 0, 0))]:
+            for alpha in (0.0, 0.5):
+                G.say(f"rmsnorm short dtype={dtype} shape=({m},{n}) shifts={shifts} alpha={alpha}")
+                x = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[0])
+                g = G.dev(r.normal(1, 0.02, n), dtype, shifts[1])
+                dy = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[2])
+                dx = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[3])
+                dg = G.dev(r.normal(0, 1, n), dtype)
+                y = G.Guarded((m, n), dtype, shifts[3])
+                xh, gh, dyh = G.host(x.t), G.host(g.t), G.host(dy.t)
+                hdx, hdg = G.host(dx.t).copy(), G.host(dg.t).copy()
+                G.rmsnorm(x.t, g.t, y.t, eps)
+                G.compare(y.t, O.rmsnorm_ij_j(xh, gh, eps), dtype, f"rmsnorm short ({m},{n})")
+                y.check("y")
+                scratch, _ = G.rmsnorm_scratch(dtype, m, n)
+                G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, eps, alpha)
+                rdx, rdg = O.rmsnorm_ij_j_reverse(xh, gh, dyh, eps, hdx if alpha else None, hdg if alpha else None, alpha)
+                sdx, sdg = G.rmsnorm_reverse_scales(xh, gh, dyh, eps, hdx if alpha else None, hdg if alpha else None, alpha)
+                G.compare(dx.t, rdx, dtype, f"rmsnorm short dx ({m},{n}) alpha {alpha}", scale=sdx)
+                G.compare(dg.t, rdg, dtype, f"rmsnorm short dg ({m},{n}) alpha {alpha}", rowwise=False, scale=sdg)
+                for gd in (x, g, dy, dx, dg, scratch):
+                    gd.check("rmsnorm short")
+            G.rmsnorm(x.t, g.t, x.t, eps)
+            G.compare(x.t, O.rmsnorm_ij_j(xh, gh, eps), dtype, f"rmsnorm short in place ({m},{n})")
+            x.check("in place")
+
+
 def test_rmsnorm_reverse_is_deterministic():
     r = rng(62)
     m, n = 2048, 4096
