@@ -27,9 +27,10 @@ namespace mp {
 /* One group of G threads per row; groups of 16, 32 or 64 lanes share a 256-thread workgroup
  * (several rows per wavefront below 64), wider groups own one row per workgroup. */
 /* DOT: every element is multiplied by vec[column] first (a matrix-vector product, one dot
- * product per row). dst[q] = scale * sum + blend * dst[q]; blend == 0 never reads dst.
+ * product per row). dst = scale * sum + blend * dst; blend == 0 never reads dst.
  * A row may be cut into `chunks` segments of chunk_len elements (the last one shorter): the
- * kernel then sees rows * chunks logical rows and writes one sum per segment, which a second
+ * kernel then sees rows * chunks logical rows and writes one sum per segment (dst[row * chunks +
+ * segment]), which a second
  * launch adds up; O is the type of those sums (the storage type, or precision<T> for partials). */
 template <class T, class O, int W, int G, bool DOT>
 __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
@@ -42,7 +43,23 @@ __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
   const size_t want = (size_t)blockIdx.x * RPB + sub;
   const bool live = want < segments; /* a dead group of a live wavefront walks the last segment and stores nothing */
   const size_t q = live ? want : segments - 1;
-  const size_t row = q / chunks, first = (q % chunks) * chunk_len; /* chunks == 1: the whole row */
+  /* Neighbouring workgroups take the same segment of neighbouring rows, so that every XCD reads a
+   * product's piece of the vector from HBM once for the rows / XCDS rows it sees of it. With few
+   * rows that is no reuse at all: then the workgroups that follow each other on one XCD (every
+   * XCDS-th) take the same segment instead (measured on r32 [8, 16M] A.v: 3.3 -> 5.3 TB/s; with
+   * many rows that order costs 10 %, [64, 2M]: 5.5 -> 4.8). */
+  const size_t rows = segments / chunks;
+  size_t row, piece;
+  if (DOT && RPB == 1 && chunks % XCDS == 0 && rows < 4 * XCDS) {
+    const size_t t = q / XCDS;
+    row = t % rows;
+    piece = t / rows * XCDS + q % XCDS;
+  } else {
+    row = q % rows;
+    piece = q / rows;
+  }
+  const size_t first = piece * chunk_len;
+  const size_t at = row * chunks + piece; /* chunks == 1: the whole row, at == q */
   const size_t len = n - first < chunk_len ? n - first : chunk_len;
 
   const T* r = src + row * n + first;
@@ -105,7 +122,7 @@ __global__ __launch_bounds__(G < 256 ? 256 : G) void reduce_rows_kernel(
     if (e != (size_t)-1) s += DOT ? (P)r[e] * (P)v[e] : (P)r[e];
   }
   s = group_allreduce<AddOP, G>(s, slots, lane);
-  if (live && lane == 0) dst[q] = (O)(blend != (P)0 ? scale * s + blend * (P)dst[q] : scale * s);
+  if (live && lane == 0) dst[at] = (O)(blend != (P)0 ? scale * s + blend * (P)dst[at] : scale * s);
 }
 
 /* Rows of up to sixteen packs: a pack a lane, 1 ... 16 lanes a row (ShortRow). Groups as wide as
@@ -279,15 +296,18 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
     if (threadIdx.x % WAVE < LANES) part[threadIdx.x / WAVE][c * CW + i] = s[i];
   }
   __syncthreads();
-  const int mine = threadIdx.x;
-  const size_t at = (size_t)blockIdx.x * LANES * CW + mine;
-  if (mine < LANES * CW && at < n) {
-    P t = (P)0;
+  for (int mine = threadIdx.x; mine < LANES * CW; mine += LANES * SLICES) { /* a small workgroup has fewer threads than columns */
+    const size_t at = (size_t)blockIdx.x * LANES * CW + mine;
+    if (at < n) {
+      P t = (P)0;
 #pragma unroll
-    for (int i = 0; i < WAVES; ++i) t += part[i][mine];
-    dst[at] = (O)(blend != (P)0 ? scale * t + blend * (P)dst[at] : scale * t);
+      for (int i = 0; i < WAVES; ++i) t += part[i][mine];
+      dst[at] = (O)(blend != (P)0 ? scale * t + blend * (P)dst[at] : scale * t);
+    }
   }
 }
+
+constexpr size_t SHORT_MATRIX_ROWS = 256; /* up to here the column sum takes four slices a workgroup */
 
 /* Lanes (packs) of a row per workgroup: as many as a narrow matrix has, so that no lane idles
  * (measured on r32 [4M, 4]: 0.4 TB/s with 8 lanes); 8 lanes x one pack = 128 bytes, one cache
@@ -339,11 +359,13 @@ inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, do
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   const bool loose = !(aligned16(src) && (n % W) == 0);
-#define MP_COLS_AS(O_, LANES_, LOOSE_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)                                                     \
+#define MP_COLS_SHAPE(O_, LANES_, SLICES_, LOOSE_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)                                         \
   do {                                                                                                                       \
-    if (weight) reduce_cols_kernel<T, O_, W, LANES_, 1024 / LANES_, true, LOOSE_><<<GRID_, dim3(1024), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_); \
-    else reduce_cols_kernel<T, O_, W, LANES_, 1024 / LANES_, false, LOOSE_><<<GRID_, dim3(1024), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_);       \
+    if (weight) reduce_cols_kernel<T, O_, W, LANES_, SLICES_, true, LOOSE_><<<GRID_, dim3(LANES_ * SLICES_), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_); \
+    else reduce_cols_kernel<T, O_, W, LANES_, SLICES_, false, LOOSE_><<<GRID_, dim3(LANES_ * SLICES_), 0, stream>>>(src, weight, OUT_, SCALE_, BLEND_, m, n, CHUNK_);       \
   } while (0)
+#define MP_COLS_AS(O_, LANES_, LOOSE_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_) \
+  MP_COLS_SHAPE(O_, LANES_, 1024 / LANES_, LOOSE_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)
 #define MP_COLS(O_, GRID_, OUT_, SCALE_, BLEND_, CHUNK_)                              \
   do {                                                                              \
     if (lanes == 1) MP_COLS_AS(O_, 1, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);   \
@@ -355,6 +377,19 @@ inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, do
     else if (loose) MP_COLS_AS(O_, 8, true, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);   \
     else MP_COLS_AS(O_, 8, false, GRID_, OUT_, SCALE_, BLEND_, CHUNK_);             \
   } while (0)
+  /* A few long rows (the sum of a handful of vectors): the 128 slices of an 8-lane workgroup
+   * would find eight rows to share (measured on r32 [8, 16M]: 0.34 TB/s, [256, 512K]: 4.1); a
+   * wavefront per kilobyte of the rows and four slices (fewer for one or two rows) keep every
+   * thread busy. */
+  if (m <= SHORT_MATRIX_ROWS && (n + W - 1) / W >= 64) {
+    const size_t wide = ((n + W - 1) / W + 63) / 64;
+    require(wide < 0x7fffffffull, "column sums: too many columns for one grid");
+    if (m == 1) MP_COLS_SHAPE(T, 64, 1, true, dim3((unsigned)wide), dst, (P)scale, (P)blend, m);
+    else if (m == 2) MP_COLS_SHAPE(T, 64, 2, true, dim3((unsigned)wide), dst, (P)scale, (P)blend, m);
+    else MP_COLS_SHAPE(T, 64, 4, true, dim3((unsigned)wide), dst, (P)scale, (P)blend, m);
+    MP_CHECK_LAUNCH();
+    return;
+  }
   const size_t lanes = reduce_cols_lanes<T>(n, loose); /* under 8 lanes the kernel is always the loose one */
   const size_t blocks = ((n + W - 1) / W + lanes - 1) / lanes;
   require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
@@ -370,6 +405,7 @@ inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, do
     return;
   }
   MP_COLS(T, dim3((unsigned)blocks), dst, (P)scale, (P)blend, m);
+#undef MP_COLS_SHAPE
 #undef MP_COLS_AS
 #undef MP_COLS
   MP_CHECK_LAUNCH();

@@ -43,7 +43,7 @@ def rows(total=1 << 28):
     print("|---|---|---|---|---|---|---|")
     for dt in (torch.float32, torch.float16):
         es = torch.empty(0, dtype=dt).element_size()
-        for n in (64, 256, 1000, 1024, 4096, 8192, 16384, 32768, 50257, 65536, 131072, 262144):
+        for n in (8, 16, 64, 256, 1000, 1024, 4096, 8192, 16384, 32768, 50257, 65536, 131072, 262144):
             m = total // n
             x = torch.randn(m, n, device="cuda", dtype=torch.float32).to(dt)
             dy = torch.randn(m, n, device="cuda", dtype=torch.float32).to(dt)
@@ -97,7 +97,7 @@ def matrix():
     kernels, _ = ffi.load()
     for dt in (torch.float32, torch.float16):
         es = torch.empty(0, dtype=dt).element_size()
-        for (m, n) in ((16384, 16384), (262144, 1024), (1024, 262144), (65536, 4096), (20000, 50257)):
+        for (m, n) in ((16384, 16384), (262144, 1024), (1024, 262144), (65536, 4096), (20000, 50257), (1 << 24, 8), (8, 1 << 24)):
             x = (torch.randn(m, n, device="cuda") * 0.1).to(dt)
             t = torch.empty(n, m, device="cuda", dtype=dt)
             vi, vj = torch.randn(m, device="cuda").to(dt), torch.randn(n, device="cuda").to(dt)

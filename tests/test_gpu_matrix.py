@@ -223,6 +223,26 @@ def test_sums_and_dot_products_of_few_long_rows(dtype):
                 G.compare(c.t, ref, dtype, f"a.B^T ({k},{n})", rowwise=False, scale=scale)
                 for gd in (x, v, s, d, b, c, row):
                     gd.check("long rows")
+        # the column sums of a few long rows (the sum of a handful of vectors) and u.A
+        for (m, n, shift) in [(1, 100003, 0), (2, 5000, 1), (3, 250000, 0), (8, 70001, 1), (40, 40000, 0), (65, 3000, 0),
+                              (256, 2049, 0), (257, 2049, 1), (5, 511, 0)]:
+            for alpha in (0.0, -0.5):
+                G.say(f"short matrix dtype={dtype} shape=({m},{n}) shift={shift} alpha={alpha}")
+                x = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+                xh = G.host(x.t)
+                sj = G.dev(r.normal(0, 1, n), dtype, shift)
+                bj = G.host(sj.t).copy()
+                stream.matrix_op("reduce_ij_j", x.t, sj.t, alpha, m, n)
+                ax = np.abs(xh.astype(np.float64))
+                G.compare(sj.t, O.reduce_ij_j(xh, bj if alpha else None, alpha), dtype, f"column sums ({m},{n})",
+                          rowwise=False, scale=ax.sum(axis=0) + abs(alpha) * np.abs(bj.astype(np.float64)))
+                u, e = G.dev(r.normal(0, 1, (1, m)), dtype), G.dev(r.normal(0, 1, (1, n)), dtype, shift)
+                be = G.host(e.t).copy()
+                stream.inner_product("ij_jk_ik", u.t, x.t, -0.5, e.t, alpha, 1, m, n)
+                ref, scale = O.inner_product(G.host(u.t), xh, -0.5, be if alpha else None, alpha, with_scale=True)
+                G.compare(e.t, ref, dtype, f"u.A ({m},{n})", rowwise=False, scale=scale)
+                for gd in (x, sj, u, e):
+                    gd.check("short matrix")
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
