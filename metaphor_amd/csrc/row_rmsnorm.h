@@ -45,9 +45,62 @@ __device__ __forceinline__ void group_allreduce_sum2(P& a, P& b, P* slots_a, P* 
   }
 }
 
+/* A row as packs counted from its first element: npk = ceil(n / W) packs,
+ * the last of which holds `last` elements (W when n is a multiple of W). A thread owns the same
+ * columns in every row (their gain, and in the reverse their dg sums, stay in registers),
+ * whatever the alignment:
+ * LOOSE = false: every operand 16-byte aligned and n % W == 0, so every pack is whole and aligned;
+ * LOOSE = true: packs start at any element (see loose_vec_of; free for these streaming reads,
+ * about 5 % on the stores) and the cut pack of a row moves element by element, zero-filled. */
+template <class T, int W, bool LOOSE> struct RowPacks {
+  using P = typename precision<T>::type;
+  using V = typename vec_of<T, W>::type;
+  using VL = typename std::conditional<LOOSE, typename loose_vec_of<T, W>::type, V>::type;
+  int npk, last;
+  __device__ __forceinline__ explicit RowPacks(size_t n)
+      : npk(LOOSE ? (int)((n + W - 1) / W) : (int)(n / W)),
+        last(LOOSE ? (int)(n - (size_t)((int)((n + W - 1) / W) - 1) * W) : W) {}
+  /* elements of pack p that exist (p < npk) */
+  __device__ __forceinline__ int valid(int p) const { return LOOSE && p == npk - 1 ? last : W; }
+  /* pack p < npk of the row at `row`, in the storage type */
+  template <bool NT> __device__ __forceinline__ V raw(const T* row, int p) const {
+    const T* at = row + (size_t)(unsigned)p * W;
+    if (!LOOSE || valid(p) == W) {
+      if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const VL*>(at));
+      else return *reinterpret_cast<const VL*>(at);
+    }
+    V v;
+#pragma unroll
+    for (int i = 0; i < W; ++i) v[i] = i < last ? at[i] : (T)0;
+    return v;
+  }
+  template <bool NT> __device__ __forceinline__ void load(const T* row, int p, P (&out)[W]) const {
+    const V v = raw<NT>(row, p);
+#pragma unroll
+    for (int i = 0; i < W; ++i) out[i] = (P)v[i];
+  }
+  __device__ __forceinline__ void store(T* row, int p, const P (&in)[W]) const {
+    T* at = row + (size_t)(unsigned)p * W;
+    if (!LOOSE || valid(p) == W) {
+      V v;
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[i] = (T)in[i];
+      __builtin_nontemporal_store(v, reinterpret_cast<VL*>(at));
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i)
+        if (i < last) at[i] = (T)in[i];
+    }
+  }
+};
+
 /* ------------------------------------------------------------------ resident forward */
 
-template <class T, int W, int G, int NV, bool RAGGED, int BLOCK = NORM_BLOCK>
+/* LOOSE = false: x, gain and y 16-byte aligned and n % W == 0. LOOSE = true: any alignment of the
+ * three and any n; the packs start at the row's first element (see RowPacks), so a thread's
+ * columns, and with them its gain, are the same in every row (gain read element by element for
+ * rows that each peel differently: r32 n = 257 3.3 TB/s). */
+template <class T, int W, int G, int NV, bool LOOSE, int BLOCK = NORM_BLOCK>
 __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
   using P = typename precision<T>::type;
@@ -55,20 +108,15 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
   __shared__ P slots[2][G < WAVE ? 1 : RPB][G < WAVE ? 1 : G / WAVE];
 
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
+  const RowPacks<T, W, LOOSE> rp(n);
 
   P gv[NV][W];
-  if constexpr (!RAGGED) { /* aligned rows: a thread's columns are the same in every row */
-    const int nvec = (int)(n / W);
 #pragma unroll
-    for (int k = 0; k < NV; ++k) {
-      const int p = k * G + lane;
-      if (p < nvec) {
-        load_pack<T, W>(gain + (size_t)p * W, gv[k]);
-      } else {
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
 #pragma unroll
-        for (int i = 0; i < W; ++i) gv[k][i] = (P)0;
-      }
-    }
+    for (int i = 0; i < W; ++i) gv[k][i] = (P)0;
+    if (p < rp.npk) rp.template load<false>(gain, p, gv[k]);
   }
 
   int parity = 0;
@@ -76,37 +124,40 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
     const size_t row = base + sub;
     const bool live = row < m; /* uniform per wave; dead groups still meet the barrier */
     const T* xr = x + (live ? row : 0) * n;
-    const RowGeom<T, W> g(xr, n, RAGGED);
-    RowTile<T, W, G, NV, RAGGED> t;
-    t.load(xr, g, live ? lane : 0x3fffffff, (P)0);
+    P xv[NV][W];
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      if (live && p < rp.npk) {
+        rp.template load<true>(xr, p, xv[k]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) xv[k][i] = (P)0;
+      }
+    }
 
     P ss = (P)0;
-    t.each([&](P& e) { ss += e * e; });
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int i = 0; i < W; ++i) ss += xv[k][i] * xv[k][i];
     ss = group_allreduce<AddOP, G>(ss, slots[parity][G < WAVE ? 0 : sub], lane);
     const P r = rsqrt_of(ss / (P)n + eps);
 
     if (live) {
-      if constexpr (!RAGGED) {
+      T* yr = y + row * n;
 #pragma unroll
-        for (int k = 0; k < NV; ++k)
+      for (int k = 0; k < NV; ++k) {
+        const int p = k * G + lane;
+        if (p < rp.npk) {
 #pragma unroll
-          for (int i = 0; i < W; ++i) t.v[k][i] *= r * gv[k][i];
-      } else {
-#pragma unroll
-        for (int k = 0; k < NV; ++k) {
-          const int p = k * G + lane;
-          if (p < g.nvec) {
-#pragma unroll
-            for (int i = 0; i < W; ++i) t.v[k][i] *= r * (P)gain[(size_t)g.head + (size_t)p * W + i];
-          }
+          for (int i = 0; i < W; ++i) xv[k][i] *= r * gv[k][i];
+          rp.store(yr, p, xv[k]);
         }
-        if (lane < g.head) t.edge *= r * (P)gain[lane];
-        else if (lane - g.head < g.tail) t.edge *= r * (P)gain[(size_t)g.head + (size_t)g.nvec * W + (lane - g.head)];
       }
-      t.store(y + row * n, g, lane);
     }
     if constexpr (G <= WAVE && BLOCK > WAVE) { /* keep the waves of a persistent workgroup on neighbouring rows */
-      if (n / W >= (size_t)G) __syncthreads();
+      if (rp.npk >= G) __syncthreads();
     }
   }
 }
@@ -288,55 +339,6 @@ template <class T> inline size_t rmsnorm_scratch_bytes(size_t m, size_t n) {
 }
 
 /* ------------------------------------------------------------------ resident reverse */
-
-/* A row of the reverse kernels as packs counted from its first element: npk = ceil(n / W) packs,
- * the last of which holds `last` elements (W when n is a multiple of W). A thread owns the same
- * columns in every row and keeps their dg sums in registers, whatever the alignment:
- * LOOSE = false: every operand 16-byte aligned and n % W == 0, so every pack is whole and aligned;
- * LOOSE = true: packs start at any element (see loose_vec_of; free for these streaming reads,
- * about 5 % on the stores) and the cut pack of a row moves element by element, zero-filled. */
-template <class T, int W, bool LOOSE> struct RowPacks {
-  using P = typename precision<T>::type;
-  using V = typename vec_of<T, W>::type;
-  using VL = typename std::conditional<LOOSE, typename loose_vec_of<T, W>::type, V>::type;
-  int npk, last;
-  __device__ __forceinline__ explicit RowPacks(size_t n)
-      : npk(LOOSE ? (int)((n + W - 1) / W) : (int)(n / W)),
-        last(LOOSE ? (int)(n - (size_t)((int)((n + W - 1) / W) - 1) * W) : W) {}
-  /* elements of pack p that exist (p < npk) */
-  __device__ __forceinline__ int valid(int p) const { return LOOSE && p == npk - 1 ? last : W; }
-  /* pack p < npk of the row at `row`, in the storage type */
-  template <bool NT> __device__ __forceinline__ V raw(const T* row, int p) const {
-    const T* at = row + (size_t)(unsigned)p * W;
-    if (!LOOSE || valid(p) == W) {
-      if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const VL*>(at));
-      else return *reinterpret_cast<const VL*>(at);
-    }
-    V v;
-#pragma unroll
-    for (int i = 0; i < W; ++i) v[i] = i < last ? at[i] : (T)0;
-    return v;
-  }
-  template <bool NT> __device__ __forceinline__ void load(const T* row, int p, P (&out)[W]) const {
-    const V v = raw<NT>(row, p);
-#pragma unroll
-    for (int i = 0; i < W; ++i) out[i] = (P)v[i];
-  }
-  __device__ __forceinline__ void store(T* row, int p, const P (&in)[W]) const {
-    T* at = row + (size_t)(unsigned)p * W;
-    if (!LOOSE || valid(p) == W) {
-      V v;
-#pragma unroll
-      for (int i = 0; i < W; ++i) v[i] = (T)in[i];
-      __builtin_nontemporal_store(v, reinterpret_cast<VL*>(at));
-    } else {
-#pragma unroll
-      for (int i = 0; i < W; ++i)
-        if (i < last) at[i] = (T)in[i];
-    }
-  }
-};
-
 
 /* partials holds gridDim.x rows of n values of precision<T>. */
 template <class T, int W, int G, int NV, bool BLEND, bool LOOSE>
@@ -942,15 +944,12 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
     MP_CHECK_LAUNCH();
     return;
   }
-  if (misalign16(x) != misalign16(y)) {
-    const size_t grid = m < cap ? m : cap;
-    rmsnorm_fwd_stream<T, 1><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
-    MP_CHECK_LAUNCH();
-    return;
-  }
-  const bool ragged = !(aligned16(x) && aligned16(gain) && (n % W) == 0);
+  /* rows of x and y that peel differently: the kernels that hold a row in registers take them (their
+   * packs start at the row's first element), the others go element by element */
+  const bool mismatch = misalign16(x) != misalign16(y);
+  const bool loose = !(aligned16(x) && aligned16(y) && aligned16(gain) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  {
+  if (!mismatch) {
     const int C = rmsnorm_cluster_size<T>((n + W - 1) / W);
     const bool shareable = scratch != nullptr && static_cast<const void*>(x) != static_cast<const void*>(y);
     if (C >= 1 && (C == 1 || shareable) && m * (size_t)C < 0x7fffffffull) {
@@ -975,7 +974,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
    * nothing beats the persistent kernel below 32 packs a row. Measured on the MI355X. */
   constexpr int ONESHOT = 256;
   const int nv_target = sizeof(T) == 2 ? 2 : 1;
-  const RowPlan shot = plan_row(packs, MAXNV, nv_target, ragged ? 16 : 8);
+  const RowPlan shot = plan_row(packs, MAXNV, nv_target, 8);
   const bool take_shot = row_regime_override() == REGIME_AUTO && shot.G > 0 && shot.G <= ONESHOT &&
                          (sizeof(T) != 2 || packs >= 32);
   if (take_shot) {
@@ -984,7 +983,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
         const size_t need = (m + ONESHOT / G - 1) / (ONESHOT / G);
         require(need < 0x7fffffffull, "rmsnorm: too many rows for one grid");
         const dim3 grid((unsigned)need), block(ONESHOT);
-        if (ragged) rmsnorm_fwd_resident<T, W, G, NV, true, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+        if (loose) rmsnorm_fwd_resident<T, W, G, NV, true, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
         else rmsnorm_fwd_resident<T, W, G, NV, false, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
       }
     });
@@ -993,16 +992,17 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
       return;
     }
   }
-  const RowPlan plan = plan_row(packs, MAXNV, 1, ragged ? 16 : 8);
+  const RowPlan plan = plan_row(packs, MAXNV, 1, 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
-    if (ragged) rmsnorm_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+    if (loose) rmsnorm_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
     else rmsnorm_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
   });
   if (!resident) {
     const size_t grid = m < cap ? m : cap;
-    rmsnorm_fwd_stream<T, W><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
+    if (mismatch) rmsnorm_fwd_stream<T, 1><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
+    else rmsnorm_fwd_stream<T, W><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
   }
   MP_CHECK_LAUNCH();
 }
