@@ -51,7 +51,9 @@ __device__ __forceinline__ void group_allreduce_sum2(P& a, P& b, P* slots_a, P* 
  * whatever the alignment:
  * LOOSE = false: every operand 16-byte aligned and n % W == 0, so every pack is whole and aligned;
  * LOOSE = true: packs start at any element (see loose_vec_of; free for these streaming reads,
- * about 5 % on the stores) and the cut pack of a row moves element by element, zero-filled. */
+ * about 5 % on the stores) and the cut pack of a row moves element by element, zero-filled
+ * (predicated single accesses in line; moved in pieces behind branches, as the short rows do,
+ * these kernels lose 10-25 %: r16 n = 2047 forward 4.6 -> 3.4 TB/s). */
 template <class T, int W, bool LOOSE> struct RowPacks {
   using P = typename precision<T>::type;
   using V = typename vec_of<T, W>::type;
@@ -973,7 +975,9 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
    * two packs per thread for the same effect (n = 1024: 5.6 -> 6.1) and
    * nothing beats the persistent kernel below 32 packs a row. Measured on the MI355X. */
   constexpr int ONESHOT = 256;
-  const int nv_target = sizeof(T) == 2 ? 2 : 1;
+  /* rows whose packs start at any element: two packs a thread, so that a row one pack over a power
+   * of two does not idle half of a group twice as wide (r32 n = 257: 4.1 -> 5.1 TB/s, n = 130: 3.8 -> 4.9) */
+  const int nv_target = sizeof(T) == 2 || loose ? 2 : 1;
   const RowPlan shot = plan_row(packs, MAXNV, nv_target, 8);
   const bool take_shot = row_regime_override() == REGIME_AUTO && shot.G > 0 && shot.G <= ONESHOT &&
                          (sizeof(T) != 2 || packs >= 32);
@@ -992,7 +996,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
       return;
     }
   }
-  const RowPlan plan = plan_row(packs, MAXNV, 1, 8);
+  const RowPlan plan = plan_row(packs, MAXNV, loose ? 2 : 1, 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
