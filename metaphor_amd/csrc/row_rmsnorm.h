@@ -107,10 +107,17 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
   using P = typename precision<T>::type;
   constexpr int RPB = BLOCK / G;
+  static_assert(G >= W, "the first lanes of a group hold the elements behind the last whole pack");
   __shared__ P slots[2][G < WAVE ? 1 : RPB][G < WAVE ? 1 : G / WAVE];
 
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
-  const RowPacks<T, W, LOOSE> rp(n);
+  /* the whole packs of a row; the n % W elements behind them go one to a lane (a single lane
+   * moving them with W predicated accesses costs every wavefront those instructions: r16 n = 100
+   * 3.2 -> 4.4 TB/s, r32 n = 257 5.0 -> 5.5; the reverse kernel, shorter of registers, loses by
+   * the same change and keeps the cut pack on one lane) */
+  const size_t body = n / W * W;
+  const RowPacks<T, W, LOOSE> rp(body);
+  const bool edged = LOOSE && (size_t)lane < n - body;
 
   P gv[NV][W];
 #pragma unroll
@@ -120,6 +127,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
     for (int i = 0; i < W; ++i) gv[k][i] = (P)0;
     if (p < rp.npk) rp.template load<false>(gain, p, gv[k]);
   }
+  const P ge = edged ? (P)gain[body + lane] : (P)0;
 
   int parity = 0;
   for (size_t base = (size_t)blockIdx.x * RPB; base < m; base += (size_t)gridDim.x * RPB, parity ^= 1) {
@@ -137,8 +145,11 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
         for (int i = 0; i < W; ++i) xv[k][i] = (P)0;
       }
     }
+    P xe = (P)0;
+    if constexpr (LOOSE)
+      if (edged && live) xe = (P)xr[body + lane];
 
-    P ss = (P)0;
+    P ss = xe * xe;
 #pragma unroll
     for (int k = 0; k < NV; ++k)
 #pragma unroll
@@ -157,6 +168,8 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
           rp.store(yr, p, xv[k]);
         }
       }
+      if constexpr (LOOSE)
+        if (edged) yr[body + lane] = (T)(xe * r * ge);
     }
     if constexpr (G <= WAVE && BLOCK > WAVE) { /* keep the waves of a persistent workgroup on neighbouring rows */
       if (rp.npk >= G) __syncthreads();
