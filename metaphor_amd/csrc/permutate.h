@@ -200,14 +200,18 @@ __global__ __launch_bounds__(tp_threads<T>()) void permutate_kernel(
 
 /* ------------------------------------------------------------------ narrow matrices */
 
-/* A matrix with a short side of n <= TP_NARROW_MAX: [m, n] is an array of m records of n fields
+/* A matrix with a short side of n: [m, n] is an array of m records of n fields
  * (AoS), its transpose [n, m] one array per field (SoA). The tall tile above would use n of its
  * 8 packs of columns, or n of its 64 packs of rows (measured r32: [4M, 4] 2.5 TB/s, [4, 4M] 0.4).
  * Here a workgroup moves a chunk of R records: the AoS side is one contiguous run of R * n
  * elements, moved as linear packs, the SoA side n runs of R elements; in between the chunk lies in
  * LDS in AoS order, one pad word after every 32 words so that the gathers and scatters with a stride
- * of n elements spread over the banks. Packs on both sides start at any element. */
-constexpr size_t TP_NARROW_MAX = 64;
+ * of n elements spread over the banks. Packs on both sides start at any element. The more fields,
+ * the fewer records fit a chunk and the shorter its runs on the field side: reads stand that
+ * better than writes (measured against the tall tile, r32 fields to records n = 130: 3.9 -> 4.3 TB/s,
+ * r16 n = 128: 3.6 -> 4.9; records to fields n = 96: 5.0 -> 3.4), hence the two limits. */
+constexpr size_t TP_NARROW_MAX = 64;      /* records of up to this many fields are split into fields this way */
+constexpr size_t TP_NARROW_MAX_BACK = 160; /* and fields are gathered into records of up to this many */
 constexpr int TP_NARROW_BYTES = 32768; /* of a chunk in LDS, pads aside */
 constexpr int TP_NARROW_THREADS = 256;
 
@@ -318,8 +322,8 @@ inline void permutate(const T* src, T* dst, double alpha, size_t rows, size_t co
   constexpr int W = pack_width<T>(), TR = TP_ROW_PACKS * W, TC = TP_COL_PACKS * W;
   require(static_cast<const void*>(src) != static_cast<const void*>(dst), "permutate_ij_ji: source and destination must differ");
   const bool blend = alpha != 0.0;
-  if (cols <= TP_NARROW_MAX || rows <= TP_NARROW_MAX) {
-    const bool to_soa = cols <= rows; /* the short side are the fields of a record */
+  const bool to_soa = cols <= rows; /* the short side are the fields of a record */
+  if (to_soa ? cols <= TP_NARROW_MAX : rows <= TP_NARROW_MAX_BACK) {
     const size_t m = to_soa ? rows : cols, n = to_soa ? cols : rows;
     const unsigned R = tp_narrow_records<T>(n);
     const size_t chunks = (m + R - 1) / R;

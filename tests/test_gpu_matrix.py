@@ -48,10 +48,10 @@ def test_permutate_forward_and_blend(dtype, shift):
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 def test_permutate_narrow_matrices(dtype):
-    """A short side of up to 64: records to fields and back through the chunked kernel; chunk
+    """A short side of up to 64 (160 when fields are gathered into records): records to fields and back through the chunked kernel; chunk
     boundaries (8192 / n records for r32), cut packs on either side, shifted bases, blend."""
     r = rng(38)
-    for n in (1, 2, 3, 4, 5, 7, 8, 12, 16, 31, 33, 63, 64):
+    for n in (1, 2, 3, 4, 5, 7, 8, 12, 16, 31, 33, 63, 64, 65, 130, 160, 161):
         for (m, shifts) in ((1, (0, 0)), (6, (1, 0)), (1000, (0, 0)), (8193, (0, 1)), (40003, (1, 3))):
             for (rows, cols) in ((m, n), (n, m)):
                 for alpha in (0.0, -0.5):
