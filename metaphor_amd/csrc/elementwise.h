@@ -40,12 +40,24 @@ constexpr int EW_BLOCK = 64;
  * everything that also reads is fastest with single-wave workgroups. */
 template <int NIN> constexpr int ew_block() { return NIN == 0 ? 256 : EW_BLOCK; }
 
-/* F::apply(const P (&in)[NIN], P (&out)[NOUT]) computes one element. */
-template <class T, int W, int NIN, int NOUT, int UNROLL, class F>
-__global__ __launch_bounds__(ew_block<NIN>()) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, size_t n, F f) {
+/* How the operands of a launch lie in memory: all at the same place, other than its start, of a
+ * 128-byte cache line, so that after the first `head` elements every
+ * wavefront's kilobyte starts on a line again (a kilobyte that straddles lines costs 15 %,
+ * whether its packs are 16-byte aligned or not: r32 with all operands shifted by one element 5.4
+ * against 6.4 TB/s); all 16-byte aligned; or anything else, and the packs then start at any element (see loose_vec_of),
+ * which costs a streaming kernel 5-15 % where one-element accesses cost half (r32) or three
+ * quarters (r16) of the bandwidth. */
+enum EwLayout { EW_ALIGNED, EW_PEELED, EW_LOOSE };
+
+/* F::apply(const P (&in)[NIN], P (&out)[NOUT]) computes one element. head: the elements before the
+ * first pack (EW_PEELED only, less than a cache line of them). */
+template <class T, int W, int LAYOUT, int NIN, int NOUT, int UNROLL, class F>
+__global__ __launch_bounds__(ew_block<NIN>()) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, size_t n, unsigned head_arg, F f) {
   using P = typename precision<T>::type;
   constexpr int NA = NIN > 0 ? NIN : 1, EW_BLOCK = ew_block<NIN>();
-  const size_t npacks = n / W;
+  constexpr bool LOOSE = LAYOUT == EW_LOOSE;
+  const size_t head = LAYOUT == EW_PEELED ? head_arg : 0;
+  const size_t npacks = (n - head) / W;
   const size_t base = (size_t)blockIdx.x * (EW_BLOCK * UNROLL) + threadIdx.x;
 
   P in[UNROLL][NA][W];
@@ -54,8 +66,10 @@ __global__ __launch_bounds__(ew_block<NIN>()) void ew_kernel(EwPtrs<NIN, NOUT> p
     const size_t p = base + (size_t)u * EW_BLOCK;
     if (p < npacks) {
 #pragma unroll
-      for (int s = 0; s < NIN; ++s)
-        load_pack_nt<T, W>(static_cast<const T*>(ptrs.in[s]) + p * W, in[u][s]);
+      for (int s = 0; s < NIN; ++s) {
+        if constexpr (LOOSE) load_pack_nt_loose<T, W>(static_cast<const T*>(ptrs.in[s]) + head + p * W, in[u][s]);
+        else load_pack_nt<T, W>(static_cast<const T*>(ptrs.in[s]) + head + p * W, in[u][s]);
+      }
     }
   }
 #pragma unroll
@@ -68,52 +82,66 @@ __global__ __launch_bounds__(ew_block<NIN>()) void ew_kernel(EwPtrs<NIN, NOUT> p
         P a[NA], r[NOUT];
 #pragma unroll
         for (int s = 0; s < NIN; ++s) a[s] = in[u][s][i];
-        ew_apply<F, P, NIN, NOUT>(f, a, r, p * W + i);
+        ew_apply<F, P, NIN, NOUT>(f, a, r, head + p * W + i);
 #pragma unroll
         for (int s = 0; s < NOUT; ++s) out[s][i] = r[s];
       }
 #pragma unroll
-      for (int s = 0; s < NOUT; ++s)
-        store_pack_nt<T, W>(static_cast<T*>(ptrs.out[s]) + p * W, out[s]);
+      for (int s = 0; s < NOUT; ++s) {
+        if constexpr (LOOSE) store_pack_nt_loose<T, W>(static_cast<T*>(ptrs.out[s]) + head + p * W, out[s]);
+        else store_pack_nt<T, W>(static_cast<T*>(ptrs.out[s]) + head + p * W, out[s]);
+      }
     }
   }
 
-  /* the n % W elements after the last whole pack */
+  /* the elements before the first pack and after the last whole one */
   if (W > 1 && blockIdx.x == 0) {
-    const size_t e = npacks * W + threadIdx.x;
-    if (e < n) {
+    auto single = [&](size_t e) {
       P a[NA], r[NOUT];
 #pragma unroll
       for (int s = 0; s < NIN; ++s) a[s] = (P) static_cast<const T*>(ptrs.in[s])[e];
       ew_apply<F, P, NIN, NOUT>(f, a, r, e);
 #pragma unroll
       for (int s = 0; s < NOUT; ++s) static_cast<T*>(ptrs.out[s])[e] = (T)r[s];
-    }
+    };
+    const size_t after = head + npacks * W + threadIdx.x;
+    if (after < n) single(after);
+    if constexpr (LAYOUT == EW_PEELED)
+      if (threadIdx.x < head) single(threadIdx.x); /* head < 128 / sizeof(T) <= 64 threads */
   }
 }
 
-/* Enqueue f over n elements. Operands that are all 16-byte aligned take the packed path;
- * anything else takes the same kernel with one-element packs. n == 0 enqueues nothing. */
+/* Enqueue f over n elements: one pack per stream per lane, laid out as EwLayout says.
+ * n == 0 enqueues nothing. */
 template <class T, int NIN, int NOUT, int UNROLL, class F>
 inline void ew_launch(const EwPtrs<NIN, NOUT>& ptrs, size_t n, F f, hipStream_t stream) {
   if (n == 0) return;
   constexpr int EW_BLOCK = ew_block<NIN>();
   require(n / EW_BLOCK < 0x7fffffffull, "elementwise launch: too many elements for one grid");
-  bool packed = true;
-  for (int s = 0; s < NIN; ++s) packed = packed && aligned16(ptrs.in[s]);
-  for (int s = 0; s < NOUT; ++s) packed = packed && aligned16(ptrs.out[s]);
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  if (packed) {
-    const size_t npacks = n / W;
-    const size_t per_block = (size_t)EW_BLOCK * UNROLL;
-    size_t blocks = (npacks + per_block - 1) / per_block;
-    if (blocks == 0) blocks = 1; /* only a scalar tail */
-    ew_kernel<T, W, NIN, NOUT, UNROLL, F><<<dim3((unsigned)blocks), dim3(EW_BLOCK), 0, stream>>>(ptrs, n, f);
-  } else {
-    const size_t per_block = (size_t)EW_BLOCK * UNROLL;
-    const size_t blocks = (n + per_block - 1) / per_block;
-    ew_kernel<T, 1, NIN, NOUT, UNROLL, F><<<dim3((unsigned)blocks), dim3(EW_BLOCK), 0, stream>>>(ptrs, n, f);
+  /* the place in a cache line that the operands share, or ~0u when they differ */
+  auto in_line = [](const void* p) { return (unsigned)(reinterpret_cast<uintptr_t>(p) & 127u); };
+  unsigned mis = NIN > 0 ? in_line(ptrs.in[0]) : in_line(ptrs.out[0]);
+  bool packed = true;
+  for (int s = 0; s < NIN; ++s) {
+    mis = in_line(ptrs.in[s]) == mis ? mis : ~0u;
+    packed = packed && aligned16(ptrs.in[s]);
   }
+  for (int s = 0; s < NOUT; ++s) {
+    mis = in_line(ptrs.out[s]) == mis ? mis : ~0u;
+    packed = packed && aligned16(ptrs.out[s]);
+  }
+  static_assert(128 / sizeof(T) <= 64, "the first workgroup's threads cover the head");
+  const bool peel = mis != 0 && mis != ~0u && mis % sizeof(T) == 0 && n >= (size_t)(128 / sizeof(T)) + W;
+  const unsigned head = peel ? (unsigned)((128 - mis) / sizeof(T)) : 0;
+  const size_t npacks = (n - head) / W;
+  const size_t per_block = (size_t)EW_BLOCK * UNROLL;
+  size_t blocks = (npacks + per_block - 1) / per_block;
+  if (blocks == 0) blocks = 1; /* only single elements */
+  const dim3 grid((unsigned)blocks), block(EW_BLOCK);
+  if (peel) ew_kernel<T, W, EW_PEELED, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, head, f);
+  else if (packed) ew_kernel<T, W, EW_ALIGNED, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
+  else ew_kernel<T, W, EW_LOOSE, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
   MP_CHECK_LAUNCH();
 }
 

@@ -95,6 +95,26 @@ def test_remaining_elementwise_launchers(dtype, shift):
             g.check(f"remaining elementwise n={n}")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_elementwise_operand_layouts(dtype):
+    """Operands at the start of a cache line, all at the same other place of one (the first elements
+    are peeled off), 16-byte aligned at different places, and at places that differ by single
+    elements (packs that start anywhere); lengths around the peeled head and the pack width."""
+    r = rng(24)
+    for n in (1, 5, 17, 31, 32, 33, 40, 63, 64, 65, 71, 100, 1000, 4099, 70001):
+        for shifts in ((0, 0, 0), (1, 1, 1), (5, 5, 5), (4, 4, 4), (8, 8, 8), (4, 8, 0), (1, 0, 0), (0, 0, 3), (1, 2, 3), (31, 31, 31)):
+            G.say(f"elementwise layouts dtype={dtype} n={n} shifts={shifts}")
+            a = G.dev(r.normal(0, 1, n), dtype, shifts[0])
+            b = G.dev(r.normal(0, 1, n), dtype, shifts[1])
+            c = G.Guarded((n,), dtype, shifts[2])
+            G.addition(a.t, b.t, c.t)
+            assert torch.equal(c.t, a.t + b.t), f"addition n={n} shifts={shifts}"
+            G.hadamard(a.t, b.t, c.t)
+            assert torch.equal(c.t, a.t * b.t), f"hadamard n={n} shifts={shifts}"
+            for gd in (a, b, c):
+                gd.check("elementwise layouts")
+
+
 def test_reference_example_all_ones_through_relu_add():
     # src/examples/subgraphs.zig:34-45: x = w1 = w2 = 1; z4 = relu(relu(x + w1) + w2) == 3
     f32 = torch.float32
