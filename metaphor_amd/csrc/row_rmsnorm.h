@@ -45,57 +45,6 @@ __device__ __forceinline__ void group_allreduce_sum2(P& a, P& b, P* slots_a, P* 
   }
 }
 
-/* A row as packs counted from its first element: npk = ceil(n / W) packs,
- * the last of which holds `last` elements (W when n is a multiple of W). A thread owns the same
- * columns in every row (their gain, and in the reverse their dg sums, stay in registers),
- * whatever the alignment:
- * LOOSE = false: every operand 16-byte aligned and n % W == 0, so every pack is whole and aligned;
- * LOOSE = true: packs start at any element (see loose_vec_of; free for these streaming reads,
- * about 5 % on the stores) and the cut pack of a row moves element by element, zero-filled
- * (predicated single accesses in line; moved in pieces behind branches, as the short rows do,
- * these kernels lose 10-25 %: r16 n = 2047 forward 4.6 -> 3.4 TB/s). */
-template <class T, int W, bool LOOSE> struct RowPacks {
-  using P = typename precision<T>::type;
-  using V = typename vec_of<T, W>::type;
-  using VL = typename std::conditional<LOOSE, typename loose_vec_of<T, W>::type, V>::type;
-  int npk, last;
-  __device__ __forceinline__ explicit RowPacks(size_t n)
-      : npk(LOOSE ? (int)((n + W - 1) / W) : (int)(n / W)),
-        last(LOOSE ? (int)(n - (size_t)((int)((n + W - 1) / W) - 1) * W) : W) {}
-  /* elements of pack p that exist (p < npk) */
-  __device__ __forceinline__ int valid(int p) const { return LOOSE && p == npk - 1 ? last : W; }
-  /* pack p < npk of the row at `row`, in the storage type */
-  template <bool NT> __device__ __forceinline__ V raw(const T* row, int p) const {
-    const T* at = row + (size_t)(unsigned)p * W;
-    if (!LOOSE || valid(p) == W) {
-      if constexpr (NT) return __builtin_nontemporal_load(reinterpret_cast<const VL*>(at));
-      else return *reinterpret_cast<const VL*>(at);
-    }
-    V v;
-#pragma unroll
-    for (int i = 0; i < W; ++i) v[i] = i < last ? at[i] : (T)0;
-    return v;
-  }
-  template <bool NT> __device__ __forceinline__ void load(const T* row, int p, P (&out)[W]) const {
-    const V v = raw<NT>(row, p);
-#pragma unroll
-    for (int i = 0; i < W; ++i) out[i] = (P)v[i];
-  }
-  __device__ __forceinline__ void store(T* row, int p, const P (&in)[W]) const {
-    T* at = row + (size_t)(unsigned)p * W;
-    if (!LOOSE || valid(p) == W) {
-      V v;
-#pragma unroll
-      for (int i = 0; i < W; ++i) v[i] = (T)in[i];
-      __builtin_nontemporal_store(v, reinterpret_cast<VL*>(at));
-    } else {
-#pragma unroll
-      for (int i = 0; i < W; ++i)
-        if (i < last) at[i] = (T)in[i];
-    }
-  }
-};
-
 /* ------------------------------------------------------------------ resident forward */
 
 /* LOOSE = false: x, gain and y 16-byte aligned and n % W == 0. LOOSE = true: any alignment of the

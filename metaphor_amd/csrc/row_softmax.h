@@ -180,6 +180,111 @@ __global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_rev_resident(
   }
 }
 
+/* ------------------------------------------------------------------ rows shifted apart */
+
+/* The resident kernels for operands whose rows do not peel alike (x 16-byte aligned and y not, a
+ * gradient at another offset than its output): packs counted from each row's first element
+ * (RowPacks), at whatever alignment each operand has. Element by element these rows ran at
+ * 0.3-1.7 TB/s. */
+template <class T, int W, int G, int NV>
+__global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_fwd_loose(const T* x, T* y, size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  constexpr int RPB = G < WAVE ? WAVE / G : 1;
+  __shared__ P slots[2][G < WAVE ? 1 : G / WAVE];
+  const int lane = threadIdx.x % G;
+  const size_t row_at = (size_t)blockIdx.x * RPB + threadIdx.x / G;
+  const bool live = row_at < m; /* a dead part of a wave still runs the cross-lane steps */
+  const size_t row = live ? row_at : m - 1;
+  const RowPacks<T, W, true> rp(n);
+
+  P v[NV][W];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
+    if (p < rp.npk) rp.template load<true>(x + row * n, p, v[k]);
+#pragma unroll
+    for (int i = 0; i < W; ++i)
+      if (p >= rp.npk || i >= rp.valid(p)) v[k][i] = neg_inf<P>();
+  }
+  P mx = neg_inf<P>();
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) mx = v[k][i] > mx ? v[k][i] : mx;
+  mx = group_allreduce<MaxOP, G>(mx, slots[0], lane);
+
+  const P sh = shift_of(mx);
+  P s = (P)0;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      v[k][i] = exp_shifted(v[k][i], sh);
+      s += v[k][i];
+    }
+  s = group_allreduce<AddOP, G>(s, slots[1], lane);
+
+  const P inv = (P)1 / s;
+  if (!live) return;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
+    if (p < rp.npk) {
+#pragma unroll
+      for (int i = 0; i < W; ++i) v[k][i] *= inv;
+      rp.store(y + row * n, p, v[k]);
+    }
+  }
+}
+
+template <class T, int W, int G, int NV, bool BLEND>
+__global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_rev_loose(
+    const T* y, const T* dy, T* dx, typename precision<T>::type alpha, size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  constexpr int RPB = G < WAVE ? WAVE / G : 1;
+  __shared__ P slots[G < WAVE ? 1 : G / WAVE];
+  const int lane = threadIdx.x % G;
+  const size_t row_at = (size_t)blockIdx.x * RPB + threadIdx.x / G;
+  const bool live = row_at < m;
+  const size_t row = live ? row_at : m - 1;
+  const RowPacks<T, W, true> rp(n);
+
+  P yv[NV][W], gv[NV][W];
+  P dot = (P)0;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
+    if (p < rp.npk) {
+      rp.template load<true>(y + row * n, p, yv[k]);
+      rp.template load<true>(dy + row * n, p, gv[k]);
+    } else {
+#pragma unroll
+      for (int i = 0; i < W; ++i) yv[k][i] = gv[k][i] = (P)0;
+    }
+#pragma unroll
+    for (int i = 0; i < W; ++i) dot += yv[k][i] * gv[k][i];
+  }
+  dot = group_allreduce<AddOP, G>(dot, slots, lane);
+  if (!live) return; /* nothing below crosses lanes */
+
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
+    if (p < rp.npk) {
+      P out[W];
+#pragma unroll
+      for (int i = 0; i < W; ++i) out[i] = yv[k][i] * (gv[k][i] - dot);
+      if constexpr (BLEND) {
+        P old[W];
+        rp.template load<false>(dx + row * n, p, old);
+#pragma unroll
+        for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+      }
+      rp.store(dx + row * n, p, out);
+    }
+  }
+}
+
 /* ------------------------------------------------------------------ streaming forward */
 
 /* Folds one value into a lane's running (max, sum of exp(x - max)). */
@@ -739,8 +844,13 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
     MP_CHECK_LAUNCH();
     return;
   }
-  if (misalign16(x) != misalign16(y)) { /* rows of x and y peel differently: element-wise */
-    softmax_fwd_stream<T, 1><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
+  if (misalign16(x) != misalign16(y)) { /* rows of x and y peel differently */
+    constexpr int MAXNV = max_nv_for<T>(64);
+    const bool resident = for_row_plan<MAXNV, true>(plan_row((n + W - 1) / W, MAXNV, 2, 16), [&]<int G, int NV>() {
+      softmax_fwd_loose<T, W, G, NV><<<dim3(row_grid(m, G)), dim3(G < WAVE ? WAVE : G), 0, stream>>>(x, y, m, n);
+    });
+    if (!resident) /* rows beyond the registers of a workgroup: element by element */
+      softmax_fwd_stream<T, 1><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
     MP_CHECK_LAUNCH();
     return;
   }
@@ -816,10 +926,18 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
     MP_CHECK_LAUNCH();
     return;
   }
-  if (misalign16(y) != misalign16(dy) || misalign16(y) != misalign16(dx)) {
-    const dim3 grid(stream_grid(m)), block(STREAM_THREADS);
-    if (blend) softmax_rev_stream<T, 1, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
-    else softmax_rev_stream<T, 1, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+  if (misalign16(y) != misalign16(dy) || misalign16(y) != misalign16(dx)) { /* rows that peel differently */
+    constexpr int MAXNV = max_nv_for<T>(32);
+    const bool resident = for_row_plan<MAXNV, true>(plan_row((n + W - 1) / W, MAXNV, 2, 16), [&]<int G, int NV>() {
+      const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
+      if (blend) softmax_rev_loose<T, W, G, NV, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+      else softmax_rev_loose<T, W, G, NV, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+    });
+    if (!resident) { /* rows beyond the registers of a workgroup: element by element */
+      const dim3 grid(stream_grid(m)), block(STREAM_THREADS);
+      if (blend) softmax_rev_stream<T, 1, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+      else softmax_rev_stream<T, 1, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+    }
     MP_CHECK_LAUNCH();
     return;
   }
