@@ -128,7 +128,9 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
 
 /* ------------------------------------------------------------------ streaming forward */
 
-template <class T, int W>
+/* The packs of a row start where x's alignment puts them; the gain's, and with APART (y not
+ * aligned like x) y's, start at any element. */
+template <class T, int W, bool APART = false>
 __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_fwd_stream(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
   using P = typename precision<T>::type;
@@ -172,11 +174,13 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_fwd_stream(
     const P r = rsqrt_of(ss / (P)n + eps);
 
     for (int p = lane; p < g.nvec; p += G) {
-      P buf[W];
+      P buf[W], gv[W];
       load_pack_nt<T, W>(body + (size_t)p * W, buf);
+      load_pack_loose<T, W>(gain + (size_t)g.head + (size_t)p * W, gv);
 #pragma unroll
-      for (int i = 0; i < W; ++i) buf[i] *= r * (P)gain[(size_t)g.head + (size_t)p * W + i];
-      store_pack_nt<T, W>(ybody + (size_t)p * W, buf);
+      for (int i = 0; i < W; ++i) buf[i] *= r * gv[i];
+      if constexpr (APART) store_pack_nt_loose<T, W>(ybody + (size_t)p * W, buf);
+      else store_pack_nt<T, W>(ybody + (size_t)p * W, buf);
     }
     if (W > 1 && edge != (size_t)-1) yr[edge] = (T)((P)xr[edge] * r * (P)gain[edge]);
   }
@@ -967,7 +971,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   });
   if (!resident) {
     const size_t grid = m < cap ? m : cap;
-    if (mismatch) rmsnorm_fwd_stream<T, 1><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
+    if (mismatch) rmsnorm_fwd_stream<T, W, true><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
     else rmsnorm_fwd_stream<T, W><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
   }
   MP_CHECK_LAUNCH();

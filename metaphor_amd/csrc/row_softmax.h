@@ -341,7 +341,9 @@ __device__ __forceinline__ void row_online_max_sum(const T* xr, const RowGeom<T,
   }
 }
 
-template <class T, int W>
+/* APART: y is not aligned like x (whose alignment sets where the packs of a row start): its
+ * packs then start at any element. */
+template <class T, int W, bool APART = false>
 __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
     const T* x, T* y, size_t m, size_t n) {
   using P = typename precision<T>::type;
@@ -381,7 +383,8 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
         if (p < g.nvec) {
 #pragma unroll
           for (int i = 0; i < W; ++i) buf[u][i] = exp_shifted(buf[u][i], sh) * inv;
-          store_pack_nt<T, W>(ybody + (size_t)p * W, buf[u]);
+          if constexpr (APART) store_pack_nt_loose<T, W>(ybody + (size_t)p * W, buf[u]);
+          else store_pack_nt<T, W>(ybody + (size_t)p * W, buf[u]);
         }
       }
     }
@@ -606,7 +609,9 @@ template <class T> inline size_t softmax_scratch_bytes(size_t m, size_t n) {
 
 /* ------------------------------------------------------------------ streaming reverse */
 
-template <class T, int W, bool BLEND>
+/* APART: dy or dx is not aligned like y (whose alignment sets where the packs of a row start):
+ * their packs then start at any element. */
+template <class T, int W, bool BLEND, bool APART = false>
 __global__ __launch_bounds__(STREAM_THREADS) void softmax_rev_stream(
     const T* y, const T* dy, T* dx, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
@@ -632,7 +637,8 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_rev_stream(
         const int p = p0 + u * G;
         if (p < g.nvec) {
           load_pack<T, W>(ybody + (size_t)p * W, a[u]);
-          load_pack<T, W>(gbody + (size_t)p * W, b[u]);
+          if constexpr (APART) load_pack_loose<T, W>(gbody + (size_t)p * W, b[u]);
+          else load_pack<T, W>(gbody + (size_t)p * W, b[u]);
         } else {
 #pragma unroll
           for (int i = 0; i < W; ++i) a[u][i] = b[u][i] = (P)0;
@@ -658,7 +664,8 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_rev_stream(
         const int p = p0 + u * G;
         if (p < g.nvec) {
           load_pack_nt<T, W>(ybody + (size_t)p * W, a[u]);
-          load_pack_nt<T, W>(gbody + (size_t)p * W, b[u]);
+          if constexpr (APART) load_pack_nt_loose<T, W>(gbody + (size_t)p * W, b[u]);
+          else load_pack_nt<T, W>(gbody + (size_t)p * W, b[u]);
         }
       }
 #pragma unroll
@@ -670,11 +677,13 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_rev_stream(
           for (int i = 0; i < W; ++i) out[i] = a[u][i] * (b[u][i] - dot);
           if constexpr (BLEND) {
             P old[W];
-            load_pack<T, W>(dbody + (size_t)p * W, old);
+            if constexpr (APART) load_pack_loose<T, W>(dbody + (size_t)p * W, old);
+            else load_pack<T, W>(dbody + (size_t)p * W, old);
 #pragma unroll
             for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
           }
-          store_pack_nt<T, W>(dbody + (size_t)p * W, out);
+          if constexpr (APART) store_pack_nt_loose<T, W>(dbody + (size_t)p * W, out);
+          else store_pack_nt<T, W>(dbody + (size_t)p * W, out);
         }
       }
     }
@@ -849,8 +858,8 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
     const bool resident = for_row_plan<MAXNV, true>(plan_row((n + W - 1) / W, MAXNV, 2, 16), [&]<int G, int NV>() {
       softmax_fwd_loose<T, W, G, NV><<<dim3(row_grid(m, G)), dim3(G < WAVE ? WAVE : G), 0, stream>>>(x, y, m, n);
     });
-    if (!resident) /* rows beyond the registers of a workgroup: element by element */
-      softmax_fwd_stream<T, 1><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
+    if (!resident) /* rows beyond the registers of a workgroup */
+      softmax_fwd_stream<T, W, true><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
     MP_CHECK_LAUNCH();
     return;
   }
@@ -933,10 +942,10 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
       if (blend) softmax_rev_loose<T, W, G, NV, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
       else softmax_rev_loose<T, W, G, NV, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
     });
-    if (!resident) { /* rows beyond the registers of a workgroup: element by element */
+    if (!resident) { /* rows beyond the registers of a workgroup */
       const dim3 grid(stream_grid(m)), block(STREAM_THREADS);
-      if (blend) softmax_rev_stream<T, 1, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
-      else softmax_rev_stream<T, 1, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+      if (blend) softmax_rev_stream<T, W, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
+      else softmax_rev_stream<T, W, false, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
     }
     MP_CHECK_LAUNCH();
     return;

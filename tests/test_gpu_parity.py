@@ -601,9 +601,11 @@ def test_rmsnorm_forward_all_regimes(dtype, regime):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
-def test_rmsnorm_forward_unaligned_and_in_place(dtype):
+@pytest.mark.parametrize("regime", [0, 6])
+def test_rmsnorm_forward_unaligned_and_in_place(dtype, regime):
     r = rng(51)
     eps = 1e-6
+    G.set_regime(regime)
     for (m, n) in [(5, 100), (3, 1027), (2, 50257), (4, 4096)]:
         for sx, sg, sy in [(1, 0, 1), (1, 1, 0), (0, 1, 0)]:
             G.say(f"rmsnorm unaligned dtype={dtype} shape=({m},{n}) shifts=({sx},{sg},{sy})")
