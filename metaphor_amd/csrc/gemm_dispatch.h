@@ -69,6 +69,133 @@ template <> struct gemm_types<r16> { static constexpr rocblas_datatype data = ro
 template <> struct gemm_types<r32> { static constexpr rocblas_datatype data = rocblas_datatype_f32_r, compute = rocblas_datatype_f32_r; };
 template <> struct gemm_types<r64> { static constexpr rocblas_datatype data = rocblas_datatype_f64_r, compute = rocblas_datatype_f64_r; };
 
+/* ------------------------------------------------------------------ few outputs, long contraction */
+
+/* C[m,k] with m, k <= R (4 or 8) and a long contraction n: up to 64 dot products over operands that
+ * are read once, an HBM-bound pass that the library's GEMM runs on a single workgroup (measured
+ * through it, r32 [4, 1M] x [1M, 4]: 30 ms, 1 GB/s). Here a thread takes W contraction steps at a
+ * time and keeps all m*k sums in registers; the workgroups walk the contraction, each leaves one
+ * partial C (scaled by alpha) in the stream's workspace and sum_partial_rows adds them in a fixed
+ * order with the beta blend.
+ * An operand is LONG when the contraction index is its contiguous one (A as [m,n], B as [k,n]):
+ * a step is then one pack of each of its rows; otherwise (A as [n,m], B as [n,k]) a step is W rows
+ * of up to R elements, each read as one R-element vector from the row's first element (which
+ * reads past a row shorter than R: the main loop stops R steps before the end, and the last
+ * elements go one by one). */
+constexpr size_t SMALL_PRODUCT_MIN_N = 8192; /* shorter contractions stay with the library */
+constexpr int SMALL_PRODUCT_THREADS = 256;
+
+template <class T, int W, int R, bool LONG>
+__device__ __forceinline__ void small_product_step(const T* x, unsigned r, size_t n, size_t j0,
+                                                   typename precision<T>::type (&out)[R][W]) {
+  using P = typename precision<T>::type;
+  if constexpr (LONG) {
+#pragma unroll
+    for (int i = 0; i < R; ++i) {
+      if (i < (int)r) {
+        load_pack_nt_loose<T, W>(x + (size_t)i * n + j0, out[i]);
+      } else {
+#pragma unroll
+        for (int w = 0; w < W; ++w) out[i][w] = (P)0;
+      }
+    }
+  } else {
+#pragma unroll
+    for (int w = 0; w < W; ++w) {
+      P row[R];
+      load_pack_nt_loose<T, R>(x + (j0 + w) * r, row);
+#pragma unroll
+      for (int i = 0; i < R; ++i) out[i][w] = i < (int)r ? row[i] : (P)0;
+    }
+  }
+}
+
+template <class T, int W, int R, bool A_LONG, bool B_LONG>
+__global__ __launch_bounds__(SMALL_PRODUCT_THREADS) void small_product_kernel(
+    const T* a, const T* b, typename precision<T>::type* partials, typename precision<T>::type scale,
+    unsigned m, unsigned k, size_t n, size_t steps) {
+  using P = typename precision<T>::type;
+  constexpr int THREADS = SMALL_PRODUCT_THREADS, WAVES = THREADS / WAVE;
+  __shared__ P part[WAVES][R * R];
+  P acc[R][R];
+#pragma unroll
+  for (int i = 0; i < R; ++i)
+#pragma unroll
+    for (int l = 0; l < R; ++l) acc[i][l] = (P)0;
+
+  for (size_t s = (size_t)blockIdx.x * THREADS + threadIdx.x; s < steps; s += (size_t)gridDim.x * THREADS) {
+    P av[R][W], bv[R][W];
+    small_product_step<T, W, R, A_LONG>(a, m, n, s * W, av);
+    small_product_step<T, W, R, B_LONG>(b, k, n, s * W, bv);
+#pragma unroll
+    for (int i = 0; i < R; ++i)
+#pragma unroll
+      for (int l = 0; l < R; ++l)
+#pragma unroll
+        for (int w = 0; w < W; ++w) acc[i][l] += av[i][w] * bv[l][w];
+  }
+
+#pragma unroll
+  for (int i = 0; i < R; ++i)
+#pragma unroll
+    for (int l = 0; l < R; ++l) {
+      const P v = wave_allreduce<AddOP>(acc[i][l]);
+      if (threadIdx.x % WAVE == 0) part[threadIdx.x / WAVE][i * R + l] = v;
+    }
+  __syncthreads();
+  const unsigned i = threadIdx.x / R, l = threadIdx.x % R;
+  if (threadIdx.x < R * R && i < m && l < k) {
+    P t = (P)0;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) t += part[w][threadIdx.x];
+    if (blockIdx.x == 0) { /* the contraction steps behind the last whole one */
+      for (size_t j = steps * W; j < n; ++j) {
+        const P x = (P)(A_LONG ? a[(size_t)i * n + j] : a[j * m + i]);
+        const P y = (P)(B_LONG ? b[(size_t)l * n + j] : b[j * k + l]);
+        t += x * y;
+      }
+    }
+    partials[(size_t)blockIdx.x * (m * k) + i * k + l] = scale * t;
+  }
+}
+
+/* Whether the product goes to the kernel above, and with how many workgroups (0: no). */
+template <class T> inline unsigned small_product_blocks(size_t m, size_t n, size_t k, size_t workspace_bytes) {
+  using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  if (m > 8 || k > 8 || n < SMALL_PRODUCT_MIN_N) return 0;
+  const size_t steps = (n - 8) / W;
+  size_t blocks = (steps + SMALL_PRODUCT_THREADS - 1) / SMALL_PRODUCT_THREADS; /* a step a thread at least */
+  const size_t most = (size_t)compute_units() * 4, fit = workspace_bytes / (m * k * sizeof(P));
+  if (blocks > most) blocks = most;
+  if (blocks > fit) blocks = fit;
+  return (unsigned)blocks;
+}
+
+template <class T>
+inline void small_product(const T* a, const T* b, T* c, bool a_transposed, bool b_transposed, double alpha, double beta,
+                          size_t m, size_t n, size_t k, unsigned blocks, void* workspace, hipStream_t stream) {
+  using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  P* partials = static_cast<P*>(workspace);
+  const dim3 grid(blocks), block(SMALL_PRODUCT_THREADS);
+#define MP_SMALL_PRODUCT(R_, AL_, BL_) \
+  small_product_kernel<T, W, R_, AL_, BL_><<<grid, block, 0, stream>>>(a, b, partials, (P)alpha, (unsigned)m, (unsigned)k, n, (n - R_) / W)
+#define MP_SMALL_PRODUCT_R(R_)                                   \
+  do {                                                           \
+    if (!a_transposed && b_transposed) MP_SMALL_PRODUCT(R_, true, true);        \
+    else if (!a_transposed) MP_SMALL_PRODUCT(R_, true, false);   \
+    else if (b_transposed) MP_SMALL_PRODUCT(R_, false, true);    \
+    else MP_SMALL_PRODUCT(R_, false, false);                     \
+  } while (0)
+  if (m <= 4 && k <= 4) MP_SMALL_PRODUCT_R(4);
+  else MP_SMALL_PRODUCT_R(8);
+#undef MP_SMALL_PRODUCT_R
+#undef MP_SMALL_PRODUCT
+  MP_CHECK_LAUNCH();
+  sum_partial_rows<T>(partials, c, beta, blocks, m * k, stream);
+}
+
 /* A is [m,n] (or [n,m] when a_transposed), B is [n,k] (or [k,n] when b_transposed), C is [m,k];
  * all row-major and dense. In column-major terms C^T[k,m] = op(B)^T * op(A)^T, which is one
  * library call with the operands exchanged. */
@@ -93,6 +220,13 @@ inline void gemm_row_major(StreamContext ctx, bool a_transposed, bool b_transpos
     else if (!b_transposed) reduce_cols<T>(B, A, C, ws, alpha, beta, n, k, stream, ws_bytes);
     else reduce_rows<T>(B, A, C, alpha, beta, k, n, stream, ws, ws_bytes);
     return;
+  }
+  if (MpBlasContext* blas = get_blas(ctx)) {
+    if (const unsigned blocks = small_product_blocks<T>(m, n, k, blas->workspace ? blas->workspace_bytes : 0)) {
+      small_product<T>(static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), a_transposed, b_transposed,
+                       alpha, beta, m, n, k, blocks, blas->workspace, get_stream(ctx));
+      return;
+    }
   }
   const rocblas_handle handle = get_handle(ctx);
   require(handle != nullptr, "inner_product: the stream context carries no BLAS handle (create the stream with mpInitStream)");

@@ -126,6 +126,31 @@ def test_inner_product_every_operand_form(dtype):
                     c.check("inner product c")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_inner_product_of_few_outputs_and_a_long_contraction(dtype):
+    """C of at most 8 x 8 over a contraction of thousands to a million: the kernel that keeps every sum
+    in registers and splits the contraction over workgroups, every operand form, shifted bases,
+    contraction lengths around whole steps."""
+    r = rng(39)
+    with G.BlasStream() as bs:
+        for (m, n, k) in [(4, 8192, 4), (2, 8193, 3), (8, 8200, 8), (5, 100003, 7), (3, 20011, 2), (4, 1 << 20, 4),
+                          (8, 300007, 5), (2, 9000, 2), (7, 8191, 7)]:
+            for form, ta, tb in FORMS:
+                for (alpha, beta, shift) in ((1.0, 0.0, 0), (-0.5, 0.75, 1)):
+                    G.say(f"few outputs {form} dtype={dtype} m,n,k=({m},{n},{k}) alpha={alpha} beta={beta} shift={shift}")
+                    a = G.dev(r.normal(0, 1, (n, m) if ta else (m, n)), dtype, shift)
+                    b = G.dev(r.normal(0, 1, (k, n) if tb else (n, k)), dtype, shift)
+                    c = G.dev(r.normal(0, 1, (m, k)), dtype, shift)
+                    before = G.host(c.t).copy()
+                    bs.inner_product(form, a.t, b.t, alpha, c.t, beta, m, n, k)
+                    ref, scale = O.inner_product(G.host(a.t), G.host(b.t), alpha, before if beta else None, beta,
+                                                 ta=ta, tb=tb, with_scale=True)
+                    G.compare(c.t, ref, dtype, f"few outputs {form} ({m},{n},{k}) {alpha},{beta}", rowwise=False,
+                              scale=scale)
+                    for gd in (a, b, c):
+                        gd.check("few outputs")
+
+
 def test_inner_product_reference_example():
     # src/examples/experimental.zig:19-34,51-62: z = x.y, then the reverse with a seed of ones
     f32 = torch.float32
