@@ -196,6 +196,99 @@ inline void small_product(const T* a, const T* b, T* c, bool a_transposed, bool 
   sum_partial_rows<T>(partials, c, beta, blocks, m * k, stream);
 }
 
+/* ------------------------------------------------------------------ many rows through a tiny matrix */
+
+/* C[m,k] = alpha * op(A)[m,n] * op(B)[n,k] + beta * C with n, k <= R (4 or 8) and many rows: every
+ * row of C is a few values made from a few values, an HBM-bound pass over A and C that the
+ * library's GEMM runs at 0.2 TB/s (r32 [4M, 4] x [4, 4]). A thread takes one row: B sits in
+ * registers (its loads are uniform), the row of A comes as one R-element vector from the row's first
+ * element (past the row's end when n < R, so the last rows of the matrix go element by element),
+ * or, for A stored [n, m], as n coalesced loads; the row of C leaves as one vector when k == R and
+ * in pieces otherwise (store_cut_pack). */
+constexpr size_t TINY_MAP_MIN_ROWS = 1024; /* fewer rows stay with the library */
+
+template <class T, int R, bool A_T, bool B_T, bool BLEND>
+__global__ __launch_bounds__(256) void tiny_map_kernel(
+    const T* a, const T* b, T* c, typename precision<T>::type alpha, typename precision<T>::type beta,
+    size_t m, unsigned n, unsigned k) {
+  using P = typename precision<T>::type;
+  P bm[R][R];
+#pragma unroll
+  for (int j = 0; j < R; ++j)
+#pragma unroll
+    for (int l = 0; l < R; ++l)
+      bm[j][l] = j < (int)n && l < (int)k ? (P)(B_T ? b[(size_t)l * n + j] : b[(size_t)j * k + l]) : (P)0;
+
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= m) return;
+  /* whether R elements from this row's start stay inside A, inside C */
+  const bool inside_a = i * n + R <= m * n, inside_c = i * k + R <= m * k;
+
+  P x[R];
+  if constexpr (A_T) {
+#pragma unroll
+    for (int j = 0; j < R; ++j) x[j] = j < (int)n ? (P)__builtin_nontemporal_load(a + (size_t)j * m + i) : (P)0;
+  } else {
+    if (inside_a) {
+      load_pack_nt_loose<T, R>(a + i * n, x);
+    } else {
+#pragma unroll
+      for (int j = 0; j < R; ++j) x[j] = j < (int)n ? (P)a[i * n + j] : (P)0;
+    }
+#pragma unroll
+    for (int j = 0; j < R; ++j) x[j] = j < (int)n ? x[j] : (P)0;
+  }
+
+  P y[R];
+#pragma unroll
+  for (int l = 0; l < R; ++l) {
+    P t = (P)0;
+#pragma unroll
+    for (int j = 0; j < R; ++j) t += x[j] * bm[j][l];
+    y[l] = alpha * t;
+  }
+  T* out = c + i * k;
+  if constexpr (BLEND) {
+    P old[R];
+    if (inside_c) {
+      load_pack_nt_loose<T, R>(out, old);
+    } else {
+#pragma unroll
+      for (int l = 0; l < R; ++l) old[l] = l < (int)k ? (P)out[l] : (P)0;
+    }
+#pragma unroll
+    for (int l = 0; l < R; ++l) y[l] += beta * (l < (int)k ? old[l] : (P)0);
+  }
+  if (k == R) store_pack_nt_loose<T, R>(out, y);
+  else store_cut_pack<T, R>(out, y, k);
+}
+
+template <class T>
+inline void tiny_map(const T* a, const T* b, T* c, bool a_transposed, bool b_transposed, double alpha, double beta,
+                     size_t m, size_t n, size_t k, hipStream_t stream) {
+  using P = typename precision<T>::type;
+  const size_t blocks = (m + 255) / 256;
+  require(blocks < 0x7fffffffull, "inner_product: too many rows for one grid");
+  const dim3 grid((unsigned)blocks), block(256);
+#define MP_TINY_MAP(R_, AT_, BT_)                                                                                              \
+  do {                                                                                                                         \
+    if (beta != 0.0) tiny_map_kernel<T, R_, AT_, BT_, true><<<grid, block, 0, stream>>>(a, b, c, (P)alpha, (P)beta, m, (unsigned)n, (unsigned)k); \
+    else tiny_map_kernel<T, R_, AT_, BT_, false><<<grid, block, 0, stream>>>(a, b, c, (P)alpha, (P)beta, m, (unsigned)n, (unsigned)k);         \
+  } while (0)
+#define MP_TINY_MAP_R(R_)                                     \
+  do {                                                        \
+    if (a_transposed && b_transposed) MP_TINY_MAP(R_, true, true);   \
+    else if (a_transposed) MP_TINY_MAP(R_, true, false);      \
+    else if (b_transposed) MP_TINY_MAP(R_, false, true);      \
+    else MP_TINY_MAP(R_, false, false);                       \
+  } while (0)
+  if (n <= 4 && k <= 4) MP_TINY_MAP_R(4);
+  else MP_TINY_MAP_R(8);
+#undef MP_TINY_MAP_R
+#undef MP_TINY_MAP
+  MP_CHECK_LAUNCH();
+}
+
 /* A is [m,n] (or [n,m] when a_transposed), B is [n,k] (or [k,n] when b_transposed), C is [m,k];
  * all row-major and dense. In column-major terms C^T[k,m] = op(B)^T * op(A)^T, which is one
  * library call with the operands exchanged. */
@@ -219,6 +312,11 @@ inline void gemm_row_major(StreamContext ctx, bool a_transposed, bool b_transpos
     else if (k == 1) reduce_cols<T>(A, B, C, ws, alpha, beta, n, m, stream, ws_bytes);
     else if (!b_transposed) reduce_cols<T>(B, A, C, ws, alpha, beta, n, k, stream, ws_bytes);
     else reduce_rows<T>(B, A, C, alpha, beta, k, n, stream, ws, ws_bytes);
+    return;
+  }
+  if (n <= 8 && k <= 8 && m >= TINY_MAP_MIN_ROWS) {
+    tiny_map<T>(static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), a_transposed, b_transposed, alpha,
+                beta, m, n, k, get_stream(ctx));
     return;
   }
   if (MpBlasContext* blas = get_blas(ctx)) {

@@ -151,6 +151,31 @@ def test_inner_product_of_few_outputs_and_a_long_contraction(dtype):
                         gd.check("few outputs")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_inner_product_of_many_rows_through_a_tiny_matrix(dtype):
+    """C[m, k] with n, k <= 8 and a thousand rows or more: the kernel that gives a thread one row, every
+    operand form, row lengths on and off the 4- and 8-element packs, shifted bases, and row counts
+    whose last rows cannot be read as whole packs."""
+    r = rng(41)
+    with G.BlasStream() as bs:
+        for (m, n, k) in [(4096, 4, 4), (1024, 8, 8), (70001, 3, 4), (50003, 4, 3), (33333, 2, 2), (20001, 5, 8),
+                          (20001, 8, 5), (10007, 7, 7), (9001, 2, 8), (9001, 8, 2), (1025, 6, 3), (1 << 18, 4, 4)]:
+            for form, ta, tb in FORMS:
+                for (alpha, beta, shift) in ((1.0, 0.0, 0), (-0.5, 0.75, 1)):
+                    G.say(f"tiny matrix {form} dtype={dtype} m,n,k=({m},{n},{k}) alpha={alpha} beta={beta} shift={shift}")
+                    a = G.dev(r.normal(0, 1, (n, m) if ta else (m, n)), dtype, shift)
+                    b = G.dev(r.normal(0, 1, (k, n) if tb else (n, k)), dtype, shift)
+                    c = G.dev(r.normal(0, 1, (m, k)), dtype, shift)
+                    before = G.host(c.t).copy()
+                    bs.inner_product(form, a.t, b.t, alpha, c.t, beta, m, n, k)
+                    ref, scale = O.inner_product(G.host(a.t), G.host(b.t), alpha, before if beta else None, beta,
+                                                 ta=ta, tb=tb, with_scale=True)
+                    G.compare(c.t, ref, dtype, f"tiny matrix {form} ({m},{n},{k}) {alpha},{beta}", rowwise=False,
+                              scale=scale)
+                    for gd in (a, b, c):
+                        gd.check("tiny matrix")
+
+
 def test_inner_product_reference_example():
     # src/examples/experimental.zig:19-34,51-62: z = x.y, then the reverse with a seed of ones
     f32 = torch.float32
