@@ -289,6 +289,168 @@ inline void tiny_map(const T* a, const T* b, T* c, bool a_transposed, bool b_tra
   MP_CHECK_LAUNCH();
 }
 
+/* ------------------------------------------------------------------ a few dot products per row */
+
+/* C[m,k] = alpha * A[m,n] * op(B) + beta * C with 2 <= k <= 8 outputs per row and many rows of any
+ * length (a router's logits over a few experts, a head with a few classes): one HBM-bound read of
+ * A, which the library's GEMM runs at 0.7 - 2.4 TB/s for r32. A group of G threads takes ROWS
+ * consecutive rows at once, so that every pack of the k vectors it loads (from L2; Bt is [k,n],
+ * contiguous along the contraction) meets ROWS packs of A: vector traffic k / ROWS of the matrix
+ * traffic. Packs count from each row's first element at whatever alignment it has (element-aligned
+ * 128-bit accesses), so a pack column is the same in every row and in every vector; the n % W
+ * elements behind the last whole pack go one to a lane. The ROWS * k sums are folded across the
+ * group in a fixed order (lanes, then wavefronts through LDS behind one barrier) and leave as one
+ * contiguous run of ROWS * k values. */
+constexpr int FEW_DOTS_ROWS = 4; /* rows a group walks at once (8 measured slower for k = 8: the folds and the stores weigh more than the vector loads) */
+constexpr size_t FEW_DOTS_MIN_ROWS = 1024;       /* fewer rows, or a smaller matrix, stay with the library */
+constexpr size_t FEW_DOTS_MIN_ELEMENTS = 1u << 21;
+
+template <class T>
+__global__ __launch_bounds__(256) void few_dots_transpose_kernel(const T* b, T* bt, size_t n, unsigned k) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; /* index into Bt[k,n] */
+  if (i < n * k) bt[i] = b[(i % n) * k + i / n];
+}
+
+template <class T, int W, int G, int K, int R, bool BLEND>
+__global__ __launch_bounds__(G < 256 ? 256 : G) void few_dots_kernel(
+    const T* a, const T* bt, T* c, typename precision<T>::type alpha, typename precision<T>::type beta, size_t m,
+    size_t n, unsigned k) {
+  using P = typename precision<T>::type;
+  constexpr int BLOCK = G < 256 ? 256 : G, RPB = BLOCK / G, NW = G < WAVE ? 1 : G / WAVE;
+  __shared__ P slots[G > WAVE ? R * K : 1][NW];
+  const int sub = threadIdx.x / G, lane = threadIdx.x % G;
+  const size_t group = (size_t)blockIdx.x * RPB + sub;
+  const bool live = group * R < m; /* a dead group of a live workgroup walks the first rows and stores nothing */
+  const size_t row0 = live ? group * R : 0;
+
+  const T* rows[R];
+#pragma unroll
+  for (int r = 0; r < R; ++r) rows[r] = a + (row0 + r < m ? row0 + r : m - 1) * n;
+  const T* vecs[K];
+#pragma unroll
+  for (int j = 0; j < K; ++j) vecs[j] = bt + (size_t)(j < (int)k ? j : 0) * n; /* vectors past k repeat the first */
+
+  P s[R][K];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int j = 0; j < K; ++j) s[r][j] = (P)0;
+
+  const size_t packs = n / W;
+  if constexpr (sizeof(T) == 2) {
+    /* v_dot2_f32_f16 on the packs as loaded: two exact half products added to an fp32 sum per
+     * instruction, instead of two conversions and a multiply-add per element */
+    using V = typename vec_of<T, W>::type;
+    using LV = typename loose_vec_of<T, W>::type;
+    typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+    for (size_t p = lane; p < packs; p += G) {
+      V av[R];
+#pragma unroll
+      for (int r = 0; r < R; ++r) av[r] = __builtin_nontemporal_load(reinterpret_cast<const LV*>(rows[r] + p * W));
+#pragma unroll
+      for (int j = 0; j < K; ++j) {
+        const V bv = *reinterpret_cast<const LV*>(vecs[j] + p * W);
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+#pragma unroll
+          for (int i = 0; i < W; i += 2)
+            s[r][j] = __builtin_amdgcn_fdot2(half2_t{av[r][i], av[r][i + 1]}, half2_t{bv[i], bv[i + 1]}, s[r][j], false);
+      }
+    }
+  } else
+  for (size_t p = lane; p < packs; p += G) {
+    P av[R][W];
+#pragma unroll
+    for (int r = 0; r < R; ++r) load_pack_nt_loose<T, W>(rows[r] + p * W, av[r]);
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      P bv[W];
+      load_pack_loose<T, W>(vecs[j] + p * W, bv);
+#pragma unroll
+      for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int i = 0; i < W; ++i) s[r][j] += av[r][i] * bv[i];
+    }
+  }
+  if (W > 1 && (size_t)lane < n - packs * W) {
+    const size_t e = packs * W + lane;
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      const P bv = (P)vecs[j][e];
+#pragma unroll
+      for (int r = 0; r < R; ++r) s[r][j] += (P)rows[r][e] * bv;
+    }
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int j = 0; j < K; ++j) {
+      if constexpr (G <= WAVE) {
+        s[r][j] = lanes_allreduce<AddOP, G>(s[r][j]);
+      } else {
+        s[r][j] = wave_allreduce<AddOP>(s[r][j]);
+        if ((lane & (WAVE - 1)) == 0) slots[r * K + j][lane / WAVE] = s[r][j];
+      }
+    }
+  if constexpr (G > WAVE) {
+    __syncthreads();
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int j = 0; j < K; ++j) s[r][j] = fold_partials<AddOP, NW>(slots[r * K + j][lane & (NW - 1)]);
+  }
+
+  /* lane o of the group writes the o-th of the group's values, C[row0 * k + o] */
+  const size_t left = m - row0 < (size_t)R ? m - row0 : (size_t)R;
+  const unsigned count = live ? (unsigned)left * k : 0;
+#pragma unroll
+  for (int base = 0; base < R * K; base += G) {
+    const unsigned o = (unsigned)(base + lane);
+    P val = (P)0;
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int j = 0; j < K; ++j)
+        if (j < (int)k && o == (unsigned)r * k + (unsigned)j) val = s[r][j];
+    if (o < count) {
+      T* out = c + row0 * k + o;
+      val *= alpha;
+      if constexpr (BLEND) val += beta * (P)*out;
+      *out = (T)val;
+    }
+  }
+}
+
+/* Bt: the k vectors, each n long. */
+template <class T>
+inline void few_dots(const T* a, const T* bt, T* c, double alpha, double beta, size_t m, size_t n, size_t k,
+                     hipStream_t stream) {
+  using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  constexpr size_t R = FEW_DOTS_ROWS;
+  const size_t packs = n / W, groups = (m + R - 1) / R;
+  require(groups < 0x7fffffffull, "inner_product: too many rows for one grid");
+#define MP_FEW_DOTS(G_, K_, R_)                                                                                   \
+  do {                                                                                                         \
+    const dim3 grid((unsigned)((groups + (G_ < 256 ? 256 / G_ : 1) - 1) / (G_ < 256 ? 256 / G_ : 1))), block(G_ < 256 ? 256 : G_); \
+    if (beta != 0.0) few_dots_kernel<T, W, G_, K_, R_, true><<<grid, block, 0, stream>>>(a, bt, c, (P)alpha, (P)beta, m, n, (unsigned)k); \
+    else few_dots_kernel<T, W, G_, K_, R_, false><<<grid, block, 0, stream>>>(a, bt, c, (P)alpha, (P)beta, m, n, (unsigned)k);          \
+  } while (0)
+#define MP_FEW_DOTS_K(G_)              \
+  do {                                 \
+    if (k <= 2) MP_FEW_DOTS(G_, 2, FEW_DOTS_ROWS);    \
+    else if (k <= 4) MP_FEW_DOTS(G_, 4, FEW_DOTS_ROWS); \
+    else MP_FEW_DOTS(G_, 8, FEW_DOTS_ROWS);           \
+  } while (0)
+  if (packs <= 64) MP_FEW_DOTS_K(16);
+  else if (packs <= 512) MP_FEW_DOTS_K(64);
+  else MP_FEW_DOTS_K(256);
+#undef MP_FEW_DOTS_K
+#undef MP_FEW_DOTS
+  MP_CHECK_LAUNCH();
+}
+
 /* A is [m,n] (or [n,m] when a_transposed), B is [n,k] (or [k,n] when b_transposed), C is [m,k];
  * all row-major and dense. In column-major terms C^T[k,m] = op(B)^T * op(A)^T, which is one
  * library call with the operands exchanged. */
@@ -318,6 +480,24 @@ inline void gemm_row_major(StreamContext ctx, bool a_transposed, bool b_transpos
     tiny_map<T>(static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), a_transposed, b_transposed, alpha,
                 beta, m, n, k, get_stream(ctx));
     return;
+  }
+  if (!a_transposed && k >= 2 && k <= 8 && n > 8 && m >= FEW_DOTS_MIN_ROWS && m * n >= FEW_DOTS_MIN_ELEMENTS) {
+    const T* A = static_cast<const T*>(a);
+    const T* B = static_cast<const T*>(b);
+    T* C = static_cast<T*>(c);
+    hipStream_t stream = get_stream(ctx);
+    if (b_transposed) {
+      few_dots<T>(A, B, C, alpha, beta, m, n, k, stream);
+      return;
+    }
+    /* B stored [n,k]: its k columns are laid out as vectors in the stream's workspace first */
+    MpBlasContext* blas = get_blas(ctx);
+    if (blas && blas->workspace && n * k * sizeof(T) <= blas->workspace_bytes) {
+      T* bt = static_cast<T*>(blas->workspace);
+      few_dots_transpose_kernel<T><<<dim3((unsigned)((n * k + 255) / 256)), dim3(256), 0, stream>>>(B, bt, n, (unsigned)k);
+      few_dots<T>(A, bt, C, alpha, beta, m, n, k, stream);
+      return;
+    }
   }
   if (MpBlasContext* blas = get_blas(ctx)) {
     if (const unsigned blocks = small_product_blocks<T>(m, n, k, blas->workspace ? blas->workspace_bytes : 0)) {

@@ -176,6 +176,32 @@ def test_inner_product_of_many_rows_through_a_tiny_matrix(dtype):
                         gd.check("tiny matrix")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_inner_product_of_many_rows_with_a_few_vectors(dtype):
+    """C[m, k] with 2 <= k <= 8 and thousands of rows of any length: the kernel that walks four rows at a
+    time against the k vectors, for B stored as the vectors and as their transpose, row lengths around
+    whole packs and around the group widths, shifted bases, row counts that leave a group short of rows."""
+    r = rng(43)
+    with G.BlasStream() as bs:
+        for (m, n, k) in [(4096, 512, 2), (2048, 1024, 8), (1025, 2049, 3), (70001, 33, 5), (300001, 9, 8),
+                          (5003, 4099, 7), (1024, 2048, 4), (40002, 64, 8), (9001, 257, 6), (3001, 1000, 2),
+                          (1027, 8200, 8)]:
+            for form, ta, tb in FORMS[:2]:
+                for (alpha, beta, shift) in ((1.0, 0.0, 0), (-0.5, 0.75, 1)):
+                    G.say(f"few vectors {form} dtype={dtype} m,n,k=({m},{n},{k}) alpha={alpha} beta={beta} shift={shift}")
+                    a = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+                    b = G.dev(r.normal(0, 1, (k, n) if tb else (n, k)), dtype, shift)
+                    c = G.dev(r.normal(0, 1, (m, k)), dtype, shift)
+                    before = G.host(c.t).copy()
+                    bs.inner_product(form, a.t, b.t, alpha, c.t, beta, m, n, k)
+                    ref, scale = O.inner_product(G.host(a.t), G.host(b.t), alpha, before if beta else None, beta,
+                                                 ta=ta, tb=tb, with_scale=True)
+                    G.compare(c.t, ref, dtype, f"few vectors {form} ({m},{n},{k}) {alpha},{beta}", rowwise=False,
+                              scale=scale)
+                    for gd in (a, b, c):
+                        gd.check("few vectors")
+
+
 def test_inner_product_reference_example():
     # src/examples/experimental.zig:19-34,51-62: z = x.y, then the reverse with a seed of ones
     f32 = torch.float32
