@@ -451,6 +451,138 @@ inline void few_dots(const T* a, const T* bt, T* c, double alpha, double beta, s
   MP_CHECK_LAUNCH();
 }
 
+/* ------------------------------------------------------------------ rows made of a few terms */
+
+/* C[m,k] = alpha * A[m,n] * op(B) + beta * C with a contraction of 2 <= n <= 8 and long rows of C
+ * (the gradient that a layer with a few outputs sends back to its input: every row of C is a
+ * combination of the n rows of B): one HBM-bound write of C, which the library's GEMM runs at
+ * 1.3 TB/s for r32 [1M, 8] x [8, 64]. A thread owns one pack column of C for FEW_TERMS_ROWS
+ * consecutive rows: its n x W piece of B sits in registers (read once per FEW_TERMS_ROWS packs
+ * written), a row of A comes as one 8-element vector from the row's first element (the last rows
+ * of the matrix, where that would pass the end, element by element), packs count from each row's
+ * first element at whatever alignment it has, and the pack that the row's end cuts leaves in
+ * pieces. Measured 2.2 - 3.4 TB/s for r32 (rows of C of 16 and 64 elements: 0.5 and 1.3 through
+ * the GEMM, which wins from rows of about a thousand on), and lower with fewer rows a
+ * thread: the limit is the vector memory pipeline, through which every lane of a row asks for
+ * the same 32 bytes of A and every thread for its piece of B, not HBM. */
+constexpr int FEW_TERMS_ROWS = 4;
+constexpr size_t FEW_TERMS_MIN_ELEMENTS = 1u << 21; /* a smaller C stays with the library */
+constexpr size_t FEW_TERMS_MAX_ROW = 128;           /* and so do longer rows of C: r32 k = 1024: 5.9 TB/s there, 3.4 here */
+
+template <class T, int W, bool B_T, bool BLEND>
+__global__ __launch_bounds__(256) void few_terms_kernel(
+    const T* a, const T* b, T* c, typename precision<T>::type alpha, typename precision<T>::type beta, size_t m,
+    unsigned n, size_t k, size_t packs_per_row, size_t row_groups) {
+  using P = typename precision<T>::type;
+  constexpr int R = FEW_TERMS_ROWS, N = 8;
+  const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (t >= row_groups * packs_per_row) return;
+  size_t group, col;
+  if (row_groups * packs_per_row <= 0xffffffffull) { /* the common case without a 64-bit division */
+    const unsigned q = (unsigned)t / (unsigned)packs_per_row;
+    group = q;
+    col = (size_t)((unsigned)t - q * (unsigned)packs_per_row) * W;
+  } else {
+    group = t / packs_per_row;
+    col = (t % packs_per_row) * W;
+  }
+  const unsigned width = k - col < (size_t)W ? (unsigned)(k - col) : (unsigned)W;
+
+  P bm[N][W];
+#pragma unroll
+  for (int j = 0; j < N; ++j)
+#pragma unroll
+    for (int i = 0; i < W; ++i) bm[j][i] = (P)0;
+  if constexpr (!B_T) {
+#pragma unroll
+    for (int j = 0; j < N; ++j)
+      if (j < (int)n) {
+        const T* src = b + (size_t)j * k + col;
+        if (width == W) {
+          load_pack_loose<T, W>(src, bm[j]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < W; ++i)
+            if (i < (int)width) bm[j][i] = (P)src[i];
+        }
+      }
+  } else {
+#pragma unroll
+    for (int i = 0; i < W; ++i)
+      if (i < (int)width) {
+        const T* src = b + (col + i) * n;
+        if ((col + i) * n + N <= k * n) {
+          P piece[N];
+          load_pack_loose<T, N>(src, piece);
+#pragma unroll
+          for (int j = 0; j < N; ++j) bm[j][i] = j < (int)n ? piece[j] : (P)0;
+        } else {
+#pragma unroll
+          for (int j = 0; j < N; ++j)
+            if (j < (int)n) bm[j][i] = (P)src[j];
+        }
+      }
+  }
+
+#pragma unroll
+  for (int r = 0; r < R; ++r) {
+    const size_t row = group * R + r;
+    if (row >= m) break;
+    P x[N];
+    if (row * n + N <= m * n) {
+      load_pack_nt_loose<T, N>(a + row * n, x);
+#pragma unroll
+      for (int j = 0; j < N; ++j) x[j] = j < (int)n ? x[j] : (P)0;
+    } else {
+#pragma unroll
+      for (int j = 0; j < N; ++j) x[j] = j < (int)n ? (P)a[row * n + j] : (P)0;
+    }
+    P y[W];
+#pragma unroll
+    for (int i = 0; i < W; ++i) {
+      P sum = (P)0;
+#pragma unroll
+      for (int j = 0; j < N; ++j) sum += x[j] * bm[j][i];
+      y[i] = alpha * sum;
+    }
+    T* out = c + row * k + col;
+    if constexpr (BLEND) {
+      if (width == W) {
+        P old[W];
+        load_pack_nt_loose<T, W>(out, old);
+#pragma unroll
+        for (int i = 0; i < W; ++i) y[i] += beta * old[i];
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i)
+          if (i < (int)width) y[i] += beta * (P)out[i];
+      }
+    }
+    if (width == W) store_pack_nt_loose<T, W>(out, y);
+    else store_cut_pack<T, W>(out, y, width);
+  }
+}
+
+template <class T>
+inline void few_terms(const T* a, const T* b, T* c, bool b_transposed, double alpha, double beta, size_t m, size_t n,
+                      size_t k, hipStream_t stream) {
+  using P = typename precision<T>::type;
+  constexpr int W = PACK_BYTES / (int)sizeof(T);
+  const size_t packs_per_row = (k + W - 1) / W, row_groups = (m + FEW_TERMS_ROWS - 1) / FEW_TERMS_ROWS;
+  const size_t blocks = (row_groups * packs_per_row + 255) / 256;
+  require(blocks < 0x7fffffffull, "inner_product: too many outputs for one grid");
+  const dim3 grid((unsigned)blocks), block(256);
+#define MP_FEW_TERMS(BT_)                                                                                           \
+  do {                                                                                                              \
+    if (beta != 0.0) few_terms_kernel<T, W, BT_, true><<<grid, block, 0, stream>>>(a, b, c, (P)alpha, (P)beta, m, (unsigned)n, k, packs_per_row, row_groups); \
+    else few_terms_kernel<T, W, BT_, false><<<grid, block, 0, stream>>>(a, b, c, (P)alpha, (P)beta, m, (unsigned)n, k, packs_per_row, row_groups);          \
+  } while (0)
+  if (b_transposed) MP_FEW_TERMS(true);
+  else MP_FEW_TERMS(false);
+#undef MP_FEW_TERMS
+  MP_CHECK_LAUNCH();
+}
+
 /* A is [m,n] (or [n,m] when a_transposed), B is [n,k] (or [k,n] when b_transposed), C is [m,k];
  * all row-major and dense. In column-major terms C^T[k,m] = op(B)^T * op(A)^T, which is one
  * library call with the operands exchanged. */
@@ -479,6 +611,11 @@ inline void gemm_row_major(StreamContext ctx, bool a_transposed, bool b_transpos
   if (n <= 8 && k <= 8 && m >= TINY_MAP_MIN_ROWS) {
     tiny_map<T>(static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), a_transposed, b_transposed, alpha,
                 beta, m, n, k, get_stream(ctx));
+    return;
+  }
+  if (!a_transposed && n >= 2 && n <= 8 && k > 8 && k <= FEW_TERMS_MAX_ROW && m * k >= FEW_TERMS_MIN_ELEMENTS) {
+    few_terms<T>(static_cast<const T*>(a), static_cast<const T*>(b), static_cast<T*>(c), b_transposed, alpha, beta, m, n, k,
+                 get_stream(ctx));
     return;
   }
   if (!a_transposed && k >= 2 && k <= 8 && n > 8 && m >= FEW_DOTS_MIN_ROWS && m * n >= FEW_DOTS_MIN_ELEMENTS) {

@@ -202,6 +202,32 @@ def test_inner_product_of_many_rows_with_a_few_vectors(dtype):
                         gd.check("few vectors")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_inner_product_of_long_rows_from_a_few_terms(dtype):
+    """C[m, k] over a contraction of 2 to 8 with rows of C longer than that: the kernel that keeps a
+    piece of B in registers and writes a pack column of four rows a thread, for B stored either way,
+    row lengths around whole packs, shifted bases, row counts that leave the last threads short of
+    rows; the last shape has rows long enough to stay with the library."""
+    r = rng(47)
+    with G.BlasStream() as bs:
+        for (m, n, k) in [(1 << 15, 8, 64), (70001, 3, 33), (300001, 5, 9), (40000, 4, 100), (20001, 7, 127),
+                          (16385, 2, 128), (150001, 8, 17), (262147, 6, 12), (5003, 7, 4099)]:
+            for form, ta, tb in FORMS[:2]:
+                for (alpha, beta, shift) in ((1.0, 0.0, 0), (-0.5, 0.75, 1)):
+                    G.say(f"few terms {form} dtype={dtype} m,n,k=({m},{n},{k}) alpha={alpha} beta={beta} shift={shift}")
+                    a = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+                    b = G.dev(r.normal(0, 1, (k, n) if tb else (n, k)), dtype, shift)
+                    c = G.dev(r.normal(0, 1, (m, k)), dtype, shift)
+                    before = G.host(c.t).copy()
+                    bs.inner_product(form, a.t, b.t, alpha, c.t, beta, m, n, k)
+                    ref, scale = O.inner_product(G.host(a.t), G.host(b.t), alpha, before if beta else None, beta,
+                                                 ta=ta, tb=tb, with_scale=True)
+                    G.compare(c.t, ref, dtype, f"few terms {form} ({m},{n},{k}) {alpha},{beta}", rowwise=False,
+                              scale=scale)
+                    for gd in (a, b, c):
+                        gd.check("few terms")
+
+
 def test_inner_product_reference_example():
     # src/examples/experimental.zig:19-34,51-62: z = x.y, then the reverse with a seed of ones
     f32 = torch.float32
