@@ -458,7 +458,7 @@ inline void few_dots(const T* a, const T* bt, T* c, double alpha, double beta, s
  * combination of the n rows of B): one HBM-bound write of C, which the library's GEMM runs at
  * 1.3 TB/s for r32 [1M, 8] x [8, 64]. A thread owns one pack column of C for FEW_TERMS_ROWS
  * consecutive rows: its n x W piece of B sits in registers (read once per FEW_TERMS_ROWS packs
- * written), a row of A comes as one 8-element vector from the row's first element (the last rows
+ * written), a row of A comes as one 4- or 8-element vector from the row's first element (the last rows
  * of the matrix, where that would pass the end, element by element), packs count from each row's
  * first element at whatever alignment it has, and the pack that the row's end cuts leaves in
  * pieces. Measured 2.2 - 3.4 TB/s for r32 (rows of C of 16 and 64 elements: 0.5 and 1.3 through
@@ -469,12 +469,12 @@ constexpr int FEW_TERMS_ROWS = 4;
 constexpr size_t FEW_TERMS_MIN_ELEMENTS = 1u << 21; /* a smaller C stays with the library */
 constexpr size_t FEW_TERMS_MAX_ROW = 128;           /* and so do longer rows of C: r32 k = 1024: 5.9 TB/s there, 3.4 here */
 
-template <class T, int W, bool B_T, bool BLEND>
+template <class T, int W, int N, bool B_T, bool BLEND>
 __global__ __launch_bounds__(256) void few_terms_kernel(
     const T* a, const T* b, T* c, typename precision<T>::type alpha, typename precision<T>::type beta, size_t m,
     unsigned n, size_t k, size_t packs_per_row, size_t row_groups) {
   using P = typename precision<T>::type;
-  constexpr int R = FEW_TERMS_ROWS, N = 8;
+  constexpr int R = FEW_TERMS_ROWS; /* N: the contraction rounded up to 4 or 8, the width of the read of a row of A */
   const size_t t = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (t >= row_groups * packs_per_row) return;
   size_t group, col;
@@ -572,13 +572,18 @@ inline void few_terms(const T* a, const T* b, T* c, bool b_transposed, double al
   const size_t blocks = (row_groups * packs_per_row + 255) / 256;
   require(blocks < 0x7fffffffull, "inner_product: too many outputs for one grid");
   const dim3 grid((unsigned)blocks), block(256);
-#define MP_FEW_TERMS(BT_)                                                                                           \
+#define MP_FEW_TERMS(N_, BT_)                                                                                       \
   do {                                                                                                              \
-    if (beta != 0.0) few_terms_kernel<T, W, BT_, true><<<grid, block, 0, stream>>>(a, b, c, (P)alpha, (P)beta, m, (unsigned)n, k, packs_per_row, row_groups); \
-    else few_terms_kernel<T, W, BT_, false><<<grid, block, 0, stream>>>(a, b, c, (P)alpha, (P)beta, m, (unsigned)n, k, packs_per_row, row_groups);          \
+    if (beta != 0.0) few_terms_kernel<T, W, N_, BT_, true><<<grid, block, 0, stream>>>(a, b, c, (P)alpha, (P)beta, m, (unsigned)n, k, packs_per_row, row_groups); \
+    else few_terms_kernel<T, W, N_, BT_, false><<<grid, block, 0, stream>>>(a, b, c, (P)alpha, (P)beta, m, (unsigned)n, k, packs_per_row, row_groups);          \
   } while (0)
-  if (b_transposed) MP_FEW_TERMS(true);
-  else MP_FEW_TERMS(false);
+  if (n <= 4) {
+    if (b_transposed) MP_FEW_TERMS(4, true);
+    else MP_FEW_TERMS(4, false);
+  } else {
+    if (b_transposed) MP_FEW_TERMS(8, true);
+    else MP_FEW_TERMS(8, false);
+  }
 #undef MP_FEW_TERMS
   MP_CHECK_LAUNCH();
 }
