@@ -1,6 +1,6 @@
 /*
- * Exports of the kernel library that are not per-dtype launchers: workspace sizing and the
- * diagnostic row-regime override. Compiled once (no `Scalar` replication).
+ * Exports of the kernel library that are not per-dtype launchers: workspace sizing and (test
+ * build only) the row-regime and cluster-tuning overrides. Compiled once (no `Scalar` replication).
  */
 #include "row_reduce.h"
 #include "row_softmax.h"
@@ -61,6 +61,8 @@ extern "C" len_t mpReduceScratchBytes(len_t dtype, len_t m, len_t n) {
   }
 }
 
+#ifdef MP_DIAGNOSTICS
+// Test build only: neither function exists in the library as shipped.
 // Diagnostic: force the row regime of the softmax / RMSNorm launchers (0 auto; 1..5 = groups of
 // 64, 128, 256, 512, 1024 threads per row; 6 = streaming; 7 = shared rows (cluster path) of the
 // softmax launchers; 8, 9 = sub-wave groups of 16 and 32 lanes of the softmax kernels). A group that cannot hold a row falls through to the next wider one. Process-wide; meant for tests and tuning, not for concurrent use with launches.
@@ -79,3 +81,4 @@ extern "C" void mpSetClusterTuning(len_t packs_per_block, len_t spin_limit) {
   mp::cluster_tuning().packs_per_block = (int)packs_per_block;
   mp::cluster_tuning().spin_limit = (unsigned)spin_limit;
 }
+#endif

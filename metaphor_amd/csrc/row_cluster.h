@@ -27,6 +27,14 @@ template <class V> __device__ __forceinline__ void forget(V& v) {
   v = __builtin_bit_cast(V, w);
 }
 
+/* Whether two operands of `bytes` bytes each share any byte. A row shared by several workgroups
+ * may be read again by a workgroup that stopped waiting for its partners, after those have
+ * written their chunks: the output must not touch an input at all, not only not equal it. */
+inline bool ranges_overlap(const void* a, const void* b, size_t bytes) {
+  const uintptr_t pa = reinterpret_cast<uintptr_t>(a), pb = reinterpret_cast<uintptr_t>(b);
+  return pa < pb + bytes && pb < pa + bytes;
+}
+
 template <class P> struct slot_word { using type = unsigned; };
 template <> struct slot_word<double> { using type = unsigned long long; };
 
@@ -35,14 +43,33 @@ template <class Word> __global__ __launch_bounds__(256) void cluster_zero_slots(
   if (i < words) slots[i] = 0;
 }
 
-/* Diagnostic knobs of the cluster path (set through mpSetClusterTuning). */
+/* Chunk size and poll limit of the cluster path. Constants in the library as shipped; the test
+ * build (MP_DIAGNOSTICS) lets mpSetClusterTuning change them, to split short rows over several
+ * workgroups and to drive the path of a workgroup that stops waiting. */
 struct ClusterTuning {
   int packs_per_block = 0; /* 0: one pack per thread less than the register tile holds */
   unsigned spin_limit = 1u << 22;
 };
+#ifdef MP_DIAGNOSTICS
 inline ClusterTuning& cluster_tuning() {
   static ClusterTuning t;
   return t;
+}
+#else
+constexpr ClusterTuning cluster_tuning() { return ClusterTuning{}; }
+#endif
+
+/* Workgroups per row that a workspace must provide words for, given the number c the launcher
+ * would use now. As shipped that is c itself (nothing can change it between the size query and
+ * the launch). The test build sizes for the most workgroups any override can ask for, so a
+ * workspace sized under one regime or tuning is never too small for a launch under another. */
+inline size_t cluster_size_for_scratch(int c) {
+#ifdef MP_DIAGNOSTICS
+  (void)c;
+  return (size_t)CLUSTER_MAX;
+#else
+  return c > 1 ? (size_t)c : 0;
+#endif
 }
 
 /* Sums over the C workgroups that share a row. Every workgroup calls this with its NVAL partial

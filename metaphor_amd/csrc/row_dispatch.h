@@ -35,11 +35,19 @@ namespace mp {
 enum RowRegime { REGIME_AUTO = 0, REGIME_G64 = 1, REGIME_G128 = 2, REGIME_G256 = 3, REGIME_G512 = 4,
                  REGIME_G1024 = 5, REGIME_STREAM = 6, REGIME_CLUSTER = 7, REGIME_G16 = 8, REGIME_G32 = 9 };
 
-/* Diagnostic override set through mpSetRowRegime; AUTO in normal use. */
+/* The regime the launchers plan with. The library as shipped has no switch: this is the constant
+ * AUTO, the launchers hold no mutable state and the workspace sizes are functions of
+ * (dtype, m, n) alone. Only the test build (MP_DIAGNOSTICS, linked into a library of its own that
+ * the parity tests load to drive every regime) keeps a process-wide override behind
+ * mpSetRowRegime. */
+#ifdef MP_DIAGNOSTICS
 inline int& row_regime_override() {
   static int regime = REGIME_AUTO;
   return regime;
 }
+#else
+constexpr int row_regime_override() { return REGIME_AUTO; }
+#endif
 
 /* Largest NV a kernel may use, from the 32-bit registers it can spend on ONE row-shaped
  * register array (a 1024-thread workgroup leaves 128 registers per lane in total). */

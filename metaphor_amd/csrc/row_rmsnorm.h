@@ -302,8 +302,8 @@ template <class T> inline int rmsnorm_cluster_size(size_t packs) {
 
 template <class T> inline size_t rmsnorm_scratch_bytes(size_t m, size_t n) {
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  const int c = rmsnorm_cluster_size<T>((n + W - 1) / W);
-  return c > 1 ? m * (size_t)c * sizeof(typename precision<T>::type) : 0;
+  const size_t c = cluster_size_for_scratch(rmsnorm_cluster_size<T>((n + W - 1) / W));
+  return m * c * sizeof(typename precision<T>::type);
 }
 
 /* ------------------------------------------------------------------ resident reverse */
@@ -892,8 +892,8 @@ inline size_t rmsnorm_reverse_partial_rows(size_t m) {
 template <class T>
 inline size_t rmsnorm_reverse_scratch_bytes(size_t m, size_t n) {
   /* the partial rows of dg, then (shared rows only) two words per row and workgroup of the row */
-  const size_t c = (size_t)rmsnorm_rev_cluster_size<T>(n);
-  return (rmsnorm_reverse_partial_rows(m) * n + (c > 1 ? m * c * 2 : 0)) * sizeof(typename precision<T>::type);
+  const size_t c = cluster_size_for_scratch(rmsnorm_rev_cluster_size<T>(n));
+  return (rmsnorm_reverse_partial_rows(m) * n + m * c * 2) * sizeof(typename precision<T>::type);
 }
 
 template <class T>
@@ -919,7 +919,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   constexpr int MAXNV = max_nv_for<T>(32);
   if (!mismatch) {
     const int C = rmsnorm_cluster_size<T>((n + W - 1) / W);
-    const bool shareable = scratch != nullptr && static_cast<const void*>(x) != static_cast<const void*>(y);
+    const bool shareable = scratch != nullptr && !ranges_overlap(x, y, m * n * sizeof(T));
     if (C >= 1 && (C == 1 || shareable) && m * (size_t)C < 0x7fffffffull) {
       using Word = typename slot_word<P>::type;
       Word* slots = static_cast<Word*>(scratch);
@@ -991,8 +991,7 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
   constexpr int MAXNV = max_nv_for<T>(16);
   /* shared rows: dx distinct from x and dy (a workgroup that stops waiting re-reads the row), and
    * rows beyond the resident kernel unless the regime is forced */
-  const bool distinct = static_cast<const void*>(dx) != static_cast<const void*>(x) &&
-                        static_cast<const void*>(dx) != static_cast<const void*>(dy);
+  const bool distinct = !ranges_overlap(dx, x, m * n * sizeof(T)) && !ranges_overlap(dx, dy, m * n * sizeof(T));
   const int C = distinct ? rmsnorm_rev_cluster_size<T>(n) : 0;
   const bool force_shared = C >= 1 && row_regime_override() == REGIME_CLUSTER;
   const RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row(packs, MAXNV, 1, 8);

@@ -603,8 +603,8 @@ template <class T> inline int cluster_size(size_t packs) {
 template <class T> inline size_t softmax_scratch_bytes(size_t m, size_t n) {
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  const int c = cluster_size<T>((n + W - 1) / W);
-  return c > 1 ? m * (size_t)c * 2 * sizeof(P) : 0;
+  const size_t c = cluster_size_for_scratch(cluster_size<T>((n + W - 1) / W));
+  return m * c * 2 * sizeof(P);
 }
 
 /* ------------------------------------------------------------------ streaming reverse */
@@ -867,7 +867,7 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   const int C = cluster_size<T>(packs);
   /* in place, a workgroup that gives up waiting would re-read chunks its partners already
    * overwrote: shared rows need distinct buffers */
-  const bool shareable = scratch != nullptr && static_cast<const void*>(x) != static_cast<const void*>(y);
+  const bool shareable = scratch != nullptr && !ranges_overlap(x, y, m * n * sizeof(T));
   if (C >= 1 && (C == 1 || shareable) && m * (size_t)C < 0x7fffffffull) {
     using Word = typename slot_word<P>::type;
     Word* slots = static_cast<Word*>(scratch);
@@ -912,8 +912,8 @@ template <class T> inline int cluster_rev_size(size_t packs) {
 template <class T> inline size_t softmax_reverse_scratch_bytes(size_t m, size_t n) {
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  const int c = cluster_rev_size<T>((n + W - 1) / W);
-  return c > 1 ? m * (size_t)c * sizeof(P) : 0;
+  const size_t c = cluster_size_for_scratch(cluster_rev_size<T>((n + W - 1) / W));
+  return m * c * sizeof(P);
 }
 
 template <class T>
@@ -952,8 +952,7 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   }
   const size_t packs = (n + W - 1) / W;
   const int C = cluster_rev_size<T>(packs);
-  const bool distinct = static_cast<const void*>(dx) != static_cast<const void*>(y) &&
-                        static_cast<const void*>(dx) != static_cast<const void*>(dy);
+  const bool distinct = !ranges_overlap(dx, y, m * n * sizeof(T)) && !ranges_overlap(dx, dy, m * n * sizeof(T));
   if (C >= 1 && (C == 1 || (scratch != nullptr && distinct)) && m * (size_t)C < 0x7fffffffull) {
     using Word = typename slot_word<P>::type;
     Word* slots = static_cast<Word*>(scratch);

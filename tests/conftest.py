@@ -14,7 +14,8 @@ def pytest_configure(config):
 def pytest_sessionstart(session):
     """Tests load what is built; only when nothing is built (a fresh checkout) build it once."""
     from metaphor_amd import ffi, kernelgen
-    needed = ("libmp_kernels.so", "libdev_utils.so", "mp_kernels.a", "libmetaphor_host.so", "host_check")
+    needed = ("libmp_kernels.so", "libmp_kernels_diag.so", "libdev_utils.so", "mp_kernels.a",
+              "libmetaphor_host.so", "host_check")
     if not all(os.path.exists(os.path.join(ffi.LIB_DIR, n)) for n in needed):
         kernelgen.build(verbose=True)
 

@@ -34,6 +34,52 @@ def lib():
     return kernels, utils
 
 
+# ---------------------------------------------------------------- the test build of the row launchers
+#
+# The shipped library has no regime switch. lib/libmp_kernels_diag.so holds the softmax / RMSNorm
+# launchers and their workspace-size functions compiled with -DMP_DIAGNOSTICS, plus
+# mpSetRowRegime / mpSetClusterTuning. While an override is in force the wrappers below call into
+# that library; otherwise they call the shipped one.
+
+ROW_STEMS = ("softmax_ij_j", "softmax_ij_j_reverse", "rmsnorm_ij_j", "rmsnorm_ij_j_reverse")
+ROW_SIZE_FNS = ("mpSoftmaxScratchBytes", "mpSoftmaxReverseScratchBytes", "mpRmsnormScratchBytes",
+                "mpRmsnormReverseScratchBytes")
+_diag = {"lib": None, "regime": 0, "tuned": False}
+
+
+def diag_lib():
+    if _diag["lib"] is None:
+        import ctypes
+        import os
+        path = os.path.join(ffi.LIB_DIR, "libmp_kernels_diag.so")
+        if not os.path.exists(path):
+            raise ffi.BoundaryMissing(f"{path} is not built; run `python -m metaphor_amd.kernelgen`")
+        ffi.load()  # the shipped library first: the test build must not shadow it
+        d = ctypes.CDLL(path, mode=ctypes.RTLD_LOCAL)
+        wanted = {f"launch_{s}_{t}" for s in ROW_STEMS for t in ("r16", "r32", "r64")} | set(ROW_SIZE_FNS)
+        for ret, name, args in ffi.parse_declarations():
+            if name in wanted:
+                fn = getattr(d, name)
+                fn.argtypes = [ffi._CTYPE[t] for t, _ in args]
+                fn.restype = None if ret == "void" else ffi._CTYPE[ret]
+        d.mpSetRowRegime.argtypes = [ffi.len_t]
+        d.mpSetRowRegime.restype = None
+        d.mpSetClusterTuning.argtypes = [ffi.len_t, ffi.len_t]
+        d.mpSetClusterTuning.restype = None
+        _diag["lib"] = d
+    return _diag["lib"]
+
+
+def _override_active():
+    return _diag["regime"] != 0 or _diag["tuned"]
+
+
+def row_size(fn, dtype, m, n):
+    """Workspace bytes from the library that will run the launch."""
+    src = diag_lib() if _override_active() else lib()[0]
+    return int(getattr(src, fn)(KEY[dtype], m, n))
+
+
 def ctx():
     return ffi.StreamContext.from_handle(torch.cuda.current_stream().cuda_stream)
 
@@ -134,6 +180,10 @@ def rmsnorm_reverse_scales(x, g, dy, eps, dx_in=None, dg_in=None, alpha=0.0):
 # ---------------------------------------------------------------- launcher wrappers
 
 def _call(stem, dtype, *args):
+    if stem in ROW_STEMS and _override_active():
+        name = f"launch_{stem}_" + ("r16", "r32", "r64")[KEY[dtype]]
+        getattr(diag_lib(), name)(*args, ctx())
+        return
     kernels, _ = lib()
     ffi.invoke(getattr(kernels, stem), KEY[dtype], *args, ctx())
 
@@ -219,8 +269,7 @@ def reduce_ij_j_scratch(src, dst, alpha, m, n, scratch="auto"):
 
 
 def softmax_scratch(dtype, m, n):
-    kernels, _ = lib()
-    nbytes = int(kernels.mpSoftmaxScratchBytes(KEY[dtype], m, n))
+    nbytes = row_size("mpSoftmaxScratchBytes", dtype, m, n)
     return (Guarded((nbytes,), torch.uint8) if nbytes else None), nbytes
 
 
@@ -243,8 +292,7 @@ def softmax_reverse(y, dy, dx, alpha=0.0, scratch="auto"):
     m, n = y.shape
     guard = None
     if isinstance(scratch, str):
-        kernels, _ = lib()
-        nbytes = int(kernels.mpSoftmaxReverseScratchBytes(KEY[y.dtype], m, n))
+        nbytes = row_size("mpSoftmaxReverseScratchBytes", y.dtype, m, n)
         guard = Guarded((nbytes,), torch.uint8) if nbytes else None
         scratch = guard.t if guard is not None else None
     _call("softmax_ij_j_reverse", y.dtype, y.data_ptr(), dy.data_ptr(), dx.data_ptr(),
@@ -259,8 +307,7 @@ def rmsnorm(x, g, y, eps, scratch="auto"):
     m, n = x.shape
     guard = None
     if isinstance(scratch, str):
-        kernels, _ = lib()
-        nbytes = int(kernels.mpRmsnormScratchBytes(KEY[x.dtype], m, n))
+        nbytes = row_size("mpRmsnormScratchBytes", x.dtype, m, n)
         guard = Guarded((nbytes,), torch.uint8) if nbytes else None
         scratch = guard.t if guard is not None else None
     _call("rmsnorm_ij_j", x.dtype, x.data_ptr(), g.data_ptr(), y.data_ptr(),
@@ -271,8 +318,7 @@ def rmsnorm(x, g, y, eps, scratch="auto"):
 
 
 def rmsnorm_scratch(dtype, m, n):
-    kernels, _ = lib()
-    nbytes = int(kernels.mpRmsnormReverseScratchBytes(KEY[dtype], m, n))
+    nbytes = row_size("mpRmsnormReverseScratchBytes", dtype, m, n)
     return Guarded((max(nbytes, 1),), torch.uint8), nbytes
 
 
@@ -283,13 +329,15 @@ def rmsnorm_reverse(x, g, dy, dx, dg, scratch, eps, alpha=0.0):
 
 
 def set_regime(r):
-    kernels, _ = lib()
-    kernels.mpSetRowRegime(int(r))
+    """Force a row regime (0 = automatic) in the test build, which then serves the row launchers."""
+    diag_lib().mpSetRowRegime(int(r))
+    _diag["regime"] = int(r)
 
 
 def set_cluster_tuning(packs_per_block=0, spin_limit=1 << 22):
-    kernels, _ = lib()
-    kernels.mpSetClusterTuning(int(packs_per_block), int(spin_limit))
+    """Chunk size and poll limit of the shared-row kernels in the test build (defaults restore it)."""
+    diag_lib().mpSetClusterTuning(int(packs_per_block), int(spin_limit))
+    _diag["tuned"] = not (int(packs_per_block) == 0 and int(spin_limit) == 1 << 22)
 
 
 def permutate(src, dst, alpha=0.0):

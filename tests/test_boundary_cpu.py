@@ -40,6 +40,21 @@ def test_static_archive_holds_the_same_launchers():
         assert name in defined, name
 
 
+def test_shipped_libraries_export_no_process_wide_switches():
+    """Launchers must be re-entrant across streams: the regime and cluster-tuning overrides of the
+    parity tests live in a library of their own, not in the shipped ones."""
+    import subprocess
+    for name in ("libmp_kernels.so", "mp_kernels.a"):
+        flags = ["-D", "--defined-only"] if name.endswith(".so") else ["--defined-only"]
+        out = subprocess.run(["nm"] + flags + [os.path.join(ffi.LIB_DIR, name)],
+                             capture_output=True, text=True, check=True).stdout
+        assert "mpSetRowRegime" not in out and "mpSetClusterTuning" not in out, name
+        assert "row_regime_override" not in out and "cluster_tuning" not in out, name
+    diag = subprocess.run(["nm", "-D", "--defined-only", os.path.join(ffi.LIB_DIR, "libmp_kernels_diag.so")],
+                          capture_output=True, text=True, check=True).stdout
+    assert " T mpSetRowRegime" in diag and " T mpSetClusterTuning" in diag
+
+
 def test_dispatch_arrays_are_r16_r32_r64_in_scalar_tag_order():
     table = kernelgen.kernel_table()
     for stem, arr in table.items():
