@@ -57,7 +57,7 @@ def _open(name):
 _CTYPE = {
     "const void*": ctypes.c_void_p, "void*": ctypes.c_void_p, "void const*": ctypes.c_void_p,
     "double": ctypes.c_double, "len_t": len_t, "StreamContext": StreamContext,
-    "uint32_t": ctypes.c_uint32,
+    "uint32_t": ctypes.c_uint32, "int": ctypes.c_int,
 }
 _PROTO = re.compile(r"EXTERN_C\s+(\w[\w ]*?\*?)\s*(\w+)\s*\(([^)]*)\)\s*;")
 
