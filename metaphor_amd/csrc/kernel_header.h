@@ -365,6 +365,16 @@ __device__ __forceinline__ P group_allreduce(P v, P* slots, int lane_in_group) {
   }
 }
 
+/* A workgroup barrier that orders LDS traffic only. __syncthreads() also waits for every global
+ * load and store of the wave (s_waitcnt vmcnt(0)), which ends a prefetch at the first reduction
+ * that follows it; this one leaves global accesses in flight. For exchanges through LDS only:
+ * it publishes nothing that was written to global memory. */
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+/* Makes the compiler treat a register-held value as consumed and redefined here: everything that
+ * produces it (a load in flight) is waited for at this point and not later. */
+template <class V> __device__ __forceinline__ void settle(V& v) { asm volatile("" : "+v"(v)); }
+
 /* ---------------------------------------------------------------------------------------
  * row geometry: [head scalars][nvec aligned packs][tail scalars]
  * ------------------------------------------------------------------------------------- */

@@ -419,6 +419,154 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
   }
 }
 
+/* ------------------------------------------------------------------ resident reverse, rows in pairs */
+
+/* Two sums folded over a G-thread group (G > 64) behind the LDS-only barrier. */
+template <int G, class P>
+__device__ __forceinline__ void group_allreduce_sum2_lds(P& a, P& b, P* slots_a, P* slots_b, int lane) {
+  static_assert(G > WAVE, "groups of more than one wavefront");
+  a = wave_allreduce<AddOP>(a);
+  b = wave_allreduce<AddOP>(b);
+  if ((lane & (WAVE - 1)) == 0) {
+    slots_a[lane / WAVE] = a;
+    slots_b[lane / WAVE] = b;
+  }
+  lds_barrier();
+  constexpr int NW = G / WAVE;
+  a = fold_partials<AddOP, NW>(slots_a[lane & (NW - 1)]);
+  b = fold_partials<AddOP, NW>(slots_b[lane & (NW - 1)]);
+}
+
+/* The resident reverse for aligned rows of whole packs held by groups of 128 ... 1024 threads,
+ * with the loads of the next row in flight while the current one is reduced and written: two
+ * register sets (in the storage type) that take turns, loads without conditions (a row index
+ * beyond the last row reads the last row, a pack index beyond the row reads the row's first pack;
+ * both are dropped), and reductions behind a barrier that does not wait for global loads. One
+ * workgroup per CU then moves what two of the unpaired kernel move (r32 [8192, 4096]: 66.4 -> 63.9 us,
+ * against 63.1 for a plain two-reads-one-write pass over the same bytes), and leaves half as
+ * many partial rows. EXACT: every thread's NV packs lie inside the row (n == G * NV * W). */
+template <class T, int W, int G, int NV, bool BLEND, bool EXACT>
+__global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
+    const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
+    typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
+  using P = typename precision<T>::type;
+  using V = typename vec_of<T, W>::type;
+  static_assert(G > WAVE && G <= NORM_BLOCK, "groups of 128 ... 1024 threads");
+  constexpr int RPB = NORM_BLOCK / G;
+  __shared__ P slots[2][2][RPB][G / WAVE];
+  __shared__ P comb[RPB > 1 ? NORM_BLOCK * NV * W : 1];
+
+  const int sub = threadIdx.x / G, lane = threadIdx.x % G;
+  const int npk = (int)(n / W);
+  const size_t last = m - 1, stride = (size_t)gridDim.x * RPB;
+
+  P gv[NV][W], acc[NV][W];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
+#pragma unroll
+    for (int i = 0; i < W; ++i) acc[k][i] = gv[k][i] = (P)0;
+    if (p < npk) load_pack<T, W>(gain + (size_t)p * W, gv[k]);
+  }
+
+  auto fetch = [&](V (&xs)[NV], V (&ds)[NV], size_t base) {
+    size_t row = base + sub;
+    row = row < last ? row : last;
+    const T* xr = x + row * n;
+    const T* dr = dy + row * n;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      const size_t at = (size_t)(EXACT || p < npk ? p : 0) * W;
+      xs[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(xr + at));
+      ds[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(dr + at));
+    }
+  };
+  auto finish = [&](const V (&xs)[NV], const V (&ds)[NV], size_t base, P (*sl)[RPB][G / WAVE]) {
+    const size_t row = base + sub;
+    const bool live = row < m;
+    P xv[NV][W], dv[NV][W];
+    P ss = (P)0, c = (P)0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const bool inside = EXACT || k * G + lane < npk;
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        xv[k][i] = inside ? (P)xs[k][i] : (P)0;
+        dv[k][i] = inside ? (P)ds[k][i] : (P)0;
+        ss += xv[k][i] * xv[k][i];
+        c += dv[k][i] * gv[k][i] * xv[k][i];
+      }
+    }
+    group_allreduce_sum2_lds<G>(ss, c, sl[0][sub], sl[1][sub], lane);
+    const P r = rsqrt_of(ss / (P)n + eps);
+    const P cc = c / (P)n * r * r;
+    if (live) {
+      T* out_row = dx + row * n;
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        const int p = k * G + lane;
+        if (EXACT || p < npk) {
+          P out[W];
+#pragma unroll
+          for (int i = 0; i < W; ++i) {
+            out[i] = r * (dv[k][i] * gv[k][i] - xv[k][i] * cc);
+            acc[k][i] += dv[k][i] * xv[k][i] * r;
+          }
+          if constexpr (BLEND) {
+            P old[W];
+            load_pack<T, W>(out_row + (size_t)p * W, old);
+#pragma unroll
+            for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+          }
+          store_pack_nt<T, W>(out_row + (size_t)p * W, out);
+        }
+      }
+    }
+  };
+
+  V ax[NV], ad[NV], bx[NV], bd[NV];
+  size_t base = (size_t)blockIdx.x * RPB;
+  fetch(ax, ad, base);
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) settle(gv[k][i]); /* the gain is waited for here, not inside the loop */
+  for (; base < m; base += 2 * stride) {
+    fetch(bx, bd, base + stride);
+    __builtin_amdgcn_sched_barrier(0);
+    finish(ax, ad, base, slots[0]);
+    fetch(ax, ad, base + 2 * stride);
+    __builtin_amdgcn_sched_barrier(0);
+    finish(bx, bd, base + stride, slots[1]);
+  }
+
+  /* one partial row per workgroup */
+  P* mine = partials + (size_t)blockIdx.x * n;
+  if constexpr (RPB > 1) {
+    constexpr int ROW = G * NV * W;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int i = 0; i < W; ++i) comb[sub * ROW + (k * G + lane) * W + i] = acc[k][i];
+    __syncthreads();
+    for (size_t col = threadIdx.x; col < n; col += NORM_BLOCK) {
+      P t = (P)0;
+      for (int s = 0; s < RPB; ++s) t += comb[s * ROW + col];
+      mine[col] = t;
+    }
+  } else {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      if (EXACT || p < npk) {
+#pragma unroll
+        for (int i = 0; i < W; ++i) mine[(size_t)p * W + i] = acc[k][i];
+      }
+    }
+  }
+}
+
 /* ------------------------------------------------------------------ streaming reverse */
 
 /* Rows too long to keep x and dy in registers: they are read twice (the second read mostly from
@@ -708,45 +856,48 @@ template <class T> inline int rmsnorm_rev_cluster_size(size_t n) {
   return c >= 1 && c <= (size_t)CLUSTER_MAX ? (int)c : 0;
 }
 
-/* dg_j = sum over partial rows (fixed order, fp64) + alpha * dg_j. A workgroup owns
- * FINISH_LANES * CW columns; its FINISH_SLICES slices split the partial rows, and a thread keeps
- * up to eight CW-wide loads in flight (CW = 4 when the partial rows are 16-byte aligned). */
-constexpr int FINISH_LANES = 16, FINISH_SLICES = 64;
+/* dg_j = sum over partial rows (fixed order, fp64) + alpha * dg_j. A workgroup owns LANES * CW
+ * columns (CW = 4 and a whole 128-byte line when the partial rows are 16-byte aligned, else single
+ * columns); its FINISH_SLICES slices split the partial rows, and a thread keeps up to eight
+ * CW-wide loads in flight. With whole lines a workgroup is 512 threads and 4096 columns make 128
+ * workgroups (r32 [512, 4096] partial rows: 3.6 -> 2.9 us against 64 workgroups of 1024). */
+constexpr int FINISH_SLICES = 64;
+template <int CW> constexpr int finish_lanes() { return CW == 4 ? 8 : 16; }
 template <class T, int CW>
-__global__ __launch_bounds__(FINISH_LANES * FINISH_SLICES) void rmsnorm_dgain_finish(
+__global__ __launch_bounds__(finish_lanes<CW>() * FINISH_SLICES) void rmsnorm_dgain_finish(
     const typename precision<T>::type* partials, T* dg, double alpha, int rows, size_t n) {
   using P = typename precision<T>::type;
-  __shared__ double part[FINISH_SLICES][FINISH_LANES * CW + 1];
-  const int c = threadIdx.x % FINISH_LANES, slice = threadIdx.x / FINISH_LANES;
-  const size_t col = ((size_t)blockIdx.x * FINISH_LANES + c) * CW;
+  constexpr int LANES = finish_lanes<CW>();
+  __shared__ double part[FINISH_SLICES][LANES * CW + 1];
+  const int c = threadIdx.x % LANES, slice = threadIdx.x / LANES;
+  const size_t col = ((size_t)blockIdx.x * LANES + c) * CW;
   double s[CW];
 #pragma unroll
   for (int i = 0; i < CW; ++i) s[i] = 0.0;
   if (col < n) { /* n is a multiple of CW, so a thread's CW columns are all in range */
     int p = slice;
-    for (; p + 7 * FINISH_SLICES < rows; p += 8 * FINISH_SLICES) {
-      P v[8][CW];
+    auto take = [&]<int U>() {
+      P v[U][CW];
 #pragma unroll
-      for (int u = 0; u < 8; ++u) load_pack<P, CW>(partials + (size_t)(p + u * FINISH_SLICES) * n + col, v[u]);
+      for (int u = 0; u < U; ++u) load_pack<P, CW>(partials + (size_t)(p + u * FINISH_SLICES) * n + col, v[u]);
 #pragma unroll
-      for (int u = 0; u < 8; ++u)
+      for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int i = 0; i < CW; ++i) s[i] += (double)v[u][i];
-    }
-    for (; p < rows; p += FINISH_SLICES) {
-      P v[CW];
-      load_pack<P, CW>(partials + (size_t)p * n + col, v);
-#pragma unroll
-      for (int i = 0; i < CW; ++i) s[i] += (double)v[i];
-    }
+      p += U * FINISH_SLICES;
+    };
+    while (p + 7 * FINISH_SLICES < rows) take.template operator()<8>();
+    if (p + 3 * FINISH_SLICES < rows) take.template operator()<4>();
+    if (p + FINISH_SLICES < rows) take.template operator()<2>();
+    if (p < rows) take.template operator()<1>();
   }
 #pragma unroll
   for (int i = 0; i < CW; ++i) part[slice][c * CW + i] = s[i];
   __syncthreads();
-  /* the first FINISH_LANES * CW threads finish one column each */
+  /* the first LANES * CW threads finish one column each */
   const int mine = threadIdx.x;
-  const size_t out = (size_t)blockIdx.x * FINISH_LANES * CW + mine;
-  if (mine < FINISH_LANES * CW && out < n) {
+  const size_t out = (size_t)blockIdx.x * LANES * CW + mine;
+  if (mine < LANES * CW && out < n) {
     double t = 0.0;
 #pragma unroll 8
     for (int i = 0; i < FINISH_SLICES; ++i) t += part[i][mine];
@@ -762,13 +913,14 @@ inline void sum_partial_rows(const typename precision<T>::type* partials, T* dst
   using P = typename precision<T>::type;
   /* wide loads need 16-byte aligned partial rows: fp32 accumulators, n % 4 == 0, aligned scratch */
   const bool wide = sizeof(P) == 4 && (n % 4) == 0 && aligned16(partials);
-  const dim3 fblock(FINISH_LANES * FINISH_SLICES);
   if (wide) {
-    const unsigned fin = (unsigned)((n + FINISH_LANES * 4 - 1) / (FINISH_LANES * 4));
-    rmsnorm_dgain_finish<T, 4><<<dim3(fin), fblock, 0, stream>>>(partials, dst, alpha, (int)rows, n);
+    constexpr int COLS = finish_lanes<4>() * 4;
+    rmsnorm_dgain_finish<T, 4><<<dim3((unsigned)((n + COLS - 1) / COLS)), dim3(finish_lanes<4>() * FINISH_SLICES), 0, stream>>>(
+        partials, dst, alpha, (int)rows, n);
   } else {
-    const unsigned fin = (unsigned)((n + FINISH_LANES - 1) / FINISH_LANES);
-    rmsnorm_dgain_finish<T, 1><<<dim3(fin), fblock, 0, stream>>>(partials, dst, alpha, (int)rows, n);
+    constexpr int COLS = finish_lanes<1>();
+    rmsnorm_dgain_finish<T, 1><<<dim3((unsigned)((n + COLS - 1) / COLS)), dim3(finish_lanes<1>() * FINISH_SLICES), 0, stream>>>(
+        partials, dst, alpha, (int)rows, n);
   }
   MP_CHECK_LAUNCH();
 }
@@ -997,10 +1149,27 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
   const RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row(packs, MAXNV, 1, 8);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
-    rows = (unsigned)(need < max_rows ? need : max_rows);
-    const dim3 grid(rows), block(NORM_BLOCK);
-    if (blend) rmsnorm_rev_resident<T, W, G, NV, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, rows_share_lines<T>(n));
-    else rmsnorm_rev_resident<T, W, G, NV, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, rows_share_lines<T>(n));
+    /* two register sets of x and dy beside the gain and the dg sums: up to eight registers an array
+     * fit the 128 of a 1024-thread workgroup without spills */
+    constexpr bool pairs_fit = NV * W * (int)(sizeof(P) / 4) <= 8;
+    if constexpr (!LOOSE && G > WAVE && pairs_fit) {
+      /* aligned rows of whole packs in groups of more than a wavefront: rows in pairs, the next
+       * row's loads in flight behind the current row's reduction, one workgroup per CU */
+      const size_t one_per_cu = (size_t)compute_units();
+      rows = (unsigned)(need < one_per_cu ? need : one_per_cu);
+      const dim3 grid(rows), block(NORM_BLOCK);
+      const bool exact = n == (size_t)G * NV * W;
+      auto go = [&]<bool BLEND, bool EXACT>() {
+        rmsnorm_rev_paired<T, W, G, NV, BLEND, EXACT><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+      };
+      if (blend) { if (exact) go.template operator()<true, true>(); else go.template operator()<true, false>(); }
+      else { if (exact) go.template operator()<false, true>(); else go.template operator()<false, false>(); }
+    } else {
+      rows = (unsigned)(need < max_rows ? need : max_rows);
+      const dim3 grid(rows), block(NORM_BLOCK);
+      if (blend) rmsnorm_rev_resident<T, W, G, NV, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, rows_share_lines<T>(n));
+      else rmsnorm_rev_resident<T, W, G, NV, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, rows_share_lines<T>(n));
+    }
   });
   bool shared = false;
   if (!resident && C >= 1) {
