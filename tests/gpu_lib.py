@@ -12,12 +12,11 @@ KEY = {torch.float16: ffi.R16, torch.float32: ffi.R32, torch.float64: ffi.R64}
 NP_OF = {torch.float16: np.float16, torch.float32: np.float32, torch.float64: np.float64}
 
 # r32: 1e-5 relative (softmax outputs: 1e-6 absolute); r16: 2e-3 relative with a floor of one
-# r16 subnormal ulp; r64 is held to 1e-12 relative. "Relative" is against
+# r16 subnormal ulp, softmax outputs included; r64 is held to 1e-12 relative. "Relative" is against
 # max(|ref|, RMS of the reference row or tensor), which keeps cancellation-prone entries
 # (dx of softmax, dg of RMSNorm) meaningful.
 RTOL = {torch.float16: 2e-3, torch.float32: 1e-5, torch.float64: 1e-12}
 FLOOR = {torch.float16: 2.0 ** -24, torch.float32: 0.0, torch.float64: 0.0}
-SOFTMAX_ATOL = {torch.float16: 2e-3, torch.float32: 1e-6, torch.float64: 1e-13}
 
 GUARD = 64
 _SENTINEL = 12345.0
@@ -118,39 +117,68 @@ def host(t):
     return t.detach().cpu().numpy()
 
 
+def parity_stats(got, ref, dtype, rowwise=True, rtol=None, atol=None, scale=None):
+    """Numbers of one comparison, without judging it: the error of `got` against the fp64
+    reference and the bound  rtol * max(|ref|, RMS(ref row|tensor), scale) + floor  (or a plain
+    atol). Returns a dict: n, max_abs (largest |got - ref|), max_rel (largest error over
+    max(|ref|, RMS), the form the tolerance is stated in), worst (largest error over its bound:
+    below 1 means inside), violations, and where the worst entry is."""
+    g = got.detach().double().cpu().numpy()
+    ref = np.asarray(ref, dtype=np.float64)
+    assert g.shape == ref.shape, f"shape {g.shape} vs {ref.shape}"
+    if g.size == 0:
+        return {"n": 0, "max_abs": 0.0, "max_rel": 0.0, "worst": 0.0, "violations": 0, "at": None}
+    both_nan = np.isnan(g) & np.isnan(ref)
+    fin = np.where(np.isfinite(ref), ref, 0.0)
+    if rowwise and ref.ndim >= 2:
+        rms = np.sqrt((fin ** 2).mean(axis=-1, keepdims=True))
+    else:
+        rms = np.sqrt((fin ** 2).mean())
+    plain = np.maximum(np.abs(fin), rms)
+    if atol is not None:
+        bound = np.full_like(ref, atol)
+    else:
+        rtol = RTOL[dtype] if rtol is None else rtol
+        mag = plain if scale is None else np.maximum(plain, np.asarray(scale, dtype=np.float64))
+        bound = rtol * mag + FLOOR[dtype]
+    with np.errstate(invalid="ignore", divide="ignore"):
+        err = np.where(both_nan | ((g == ref) & ~np.isnan(ref)), 0.0, np.abs(g - ref))
+        bad = ~(err <= bound)
+        ratio = np.where(bad & ~np.isfinite(err), np.inf, err / np.maximum(bound, 1e-300))
+        rel = np.where(np.isfinite(err), err / np.maximum(plain, 1e-300), np.inf)
+    at = np.unravel_index(np.argmax(ratio), ref.shape)
+    finite_err = np.where(np.isfinite(err), err, 0.0)
+    return {"n": int(ref.size), "max_abs": float(finite_err.max()), "max_rel": float(np.where(plain > 0, rel, 0.0).max()),
+            "worst": float(ratio[at]), "violations": int(bad.sum()), "at": tuple(int(i) for i in at),
+            "got": float(g[at]), "ref": float(ref[at]), "err": float(err[at]), "bound": float(bound[at])}
+
+
+PARITY_LOG = []  # (what, stats) of every comparison of this process, in order
+
+
 def compare(got, ref, dtype, what, rowwise=True, rtol=None, atol=None, scale=None):
     """|got - ref| <= rtol * max(|ref|, RMS(ref row|tensor), scale) + floor (or a plain atol).
 
     `scale` is the magnitude of the terms an entry is the difference of (see
     softmax_reverse_scale / rmsnorm_reverse_scales): where two terms of size s cancel to a
-    result far below s, no fp32 kernel can be closer than a few ulp of s."""
-    g = got.detach().double().cpu().numpy()
-    ref = np.asarray(ref, dtype=np.float64)
-    assert g.shape == ref.shape, f"{what}: shape {g.shape} vs {ref.shape}"
-    if g.size == 0:
-        return
-    both_nan = np.isnan(g) & np.isnan(ref)
-    fin = np.where(np.isfinite(ref), ref, 0.0)
-    if atol is not None:
-        bound = np.full_like(ref, atol)
-    else:
-        rtol = RTOL[dtype] if rtol is None else rtol
-        if rowwise and ref.ndim >= 2:
-            rms = np.sqrt((fin ** 2).mean(axis=-1, keepdims=True))
-        else:
-            rms = np.sqrt((fin ** 2).mean())
-        mag = np.maximum(np.abs(fin), rms)
-        if scale is not None:
-            mag = np.maximum(mag, np.asarray(scale, dtype=np.float64))
-        bound = rtol * mag + FLOOR[dtype]
-    with np.errstate(invalid="ignore"):
-        err = np.abs(g - ref)
-    bad = ~(err <= bound) & ~both_nan
-    if bad.any():
-        idx = np.unravel_index(np.argmax(np.where(bad, err / np.maximum(bound, 1e-300), 0)), ref.shape)
+    result far below s, no fp32 kernel can be closer than a few ulp of s. Prints and returns
+    the numbers of the comparison (parity_stats); raises when an entry is outside its bound."""
+    st = parity_stats(got, ref, dtype, rowwise, rtol, atol, scale)
+    PARITY_LOG.append((what, st))
+    if st["n"]:
+        print(f"[parity] {what}: n={st['n']} max_abs={st['max_abs']:.3e} max_rel={st['max_rel']:.3e} "
+              f"worst err/bound={st['worst']:.3f} violations={st['violations']}", flush=True)
+    if st["violations"]:
         raise AssertionError(
-            f"{what}: {int(bad.sum())} of {ref.size} outside tolerance; worst at {idx}: "
-            f"got {g[idx]!r} ref {ref[idx]!r} err {err[idx]:.3e} bound {bound[idx]:.3e}")
+            f"{what}: {st['violations']} of {st['n']} outside tolerance; worst at {st['at']}: "
+            f"got {st['got']!r} ref {st['ref']!r} err {st['err']:.3e} bound {st['bound']:.3e}")
+    return st
+
+
+def softmax_tol(dtype):
+    """Keyword arguments of compare() for softmax outputs: r32 within 1e-6 absolute (r64 1e-13);
+    r16 like every other r16 result, 2e-3 * max(|ref|, RMS of the row) + one r16 subnormal ulp."""
+    return {} if dtype == torch.float16 else {"atol": 1e-6 if dtype == torch.float32 else 1e-13}
 
 
 def softmax_reverse_scale(y, dy, dx_in=None, alpha=0.0):

@@ -71,7 +71,7 @@ def test_gpu_launchers_reproduce_the_fixtures():
     xm = G.dev(g["smc_x"], f16)
     ym = G.Guarded(xm.t.shape, f16)
     G.softmax(xm.t, ym.t)
-    G.compare(ym.t, g["smc_y"], f16, "golden causal softmax r16", atol=G.SOFTMAX_ATOL[f16])
+    G.compare(ym.t, g["smc_y"], f16, "golden causal softmax r16", **G.softmax_tol(f16))
     assert bool((ym.t[torch.isinf(xm.t)] == 0).all())
 
     G.say("golden: rmsnorm")

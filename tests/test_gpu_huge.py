@@ -63,7 +63,7 @@ def test_softmax_beyond_32_bit_offsets():
     G.softmax(x, y)
     torch.cuda.synchronize()
     rows = _row_windows(m, n)
-    G.compare(y[rows], O.softmax_ij_j(G.host(x[rows])), F16, "softmax windows", atol=G.SOFTMAX_ATOL[F16])
+    G.compare(y[rows], O.softmax_ij_j(G.host(x[rows])), F16, "softmax windows", **G.softmax_tol(F16))
     sums = torch.zeros(m, device="cuda", dtype=torch.float32)
     step = 1 << 18
     for r in range(0, m, step):

@@ -369,7 +369,7 @@ def test_softmax_forward_all_regimes(dtype, regime):
             y = G.Guarded((m, n), dtype)
             G.softmax(x.t, y.t)
             ref = O.softmax_ij_j(G.host(x.t))
-            G.compare(y.t, ref, dtype, f"softmax ({m},{n}) regime {regime}", atol=G.SOFTMAX_ATOL[dtype])
+            G.compare(y.t, ref, dtype, f"softmax ({m},{n}) regime {regime}", **G.softmax_tol(dtype))
             if masked:
                 assert bool((y.t[torch.isinf(x.t)] == 0).all()), "-inf must map to exactly 0"
             x.check("softmax x")
@@ -388,14 +388,14 @@ def test_softmax_unaligned_bases_and_in_place(dtype, regime):
             y = G.Guarded((m, n), dtype, sy)
             G.softmax(x.t, y.t)
             ref = O.softmax_ij_j(G.host(x.t))
-            G.compare(y.t, ref, dtype, f"softmax unaligned ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
+            G.compare(y.t, ref, dtype, f"softmax unaligned ({m},{n})", **G.softmax_tol(dtype))
             x.check("x")
             y.check("y")
         x = G.dev(r.normal(0, 3, (m, n)), dtype)
         ref = O.softmax_ij_j(G.host(x.t))
         G.say(f"softmax in place dtype={dtype} shape=({m},{n})")
         G.softmax(x.t, x.t)
-        G.compare(x.t, ref, dtype, f"softmax in place ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
+        G.compare(x.t, ref, dtype, f"softmax in place ({m},{n})", **G.softmax_tol(dtype))
         x.check("in place")
 
 
@@ -421,7 +421,7 @@ def test_softmax_forward_cluster_path(dtype, packs, spin):
                 G.softmax(x.t, y.t)
                 ref = O.softmax_ij_j(G.host(x.t))
                 G.compare(y.t, ref, dtype, f"softmax cluster ({m},{n}) packs {packs} spin {spin}",
-                          atol=G.SOFTMAX_ATOL[dtype])
+                          **G.softmax_tol(dtype))
                 if masked:
                     assert bool((y.t[torch.isinf(x.t)] == 0).all())
                 x.check("x")
@@ -560,7 +560,7 @@ def test_softmax_short_rows_any_length_and_alignment(dtype):
             y = G.Guarded((m, n), dtype, shifts[1])
             G.softmax(x.t, y.t)
             xh = G.host(x.t)
-            G.compare(y.t, O.softmax_ij_j(xh), dtype, f"softmax short ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
+            G.compare(y.t, O.softmax_ij_j(xh), dtype, f"softmax short ({m},{n})", **G.softmax_tol(dtype))
             x.check("x")
             y.check("y")
             dy = G.dev(r.normal(0, 1, (m, n)), dtype, shifts[2])
@@ -574,7 +574,7 @@ def test_softmax_short_rows_any_length_and_alignment(dtype):
                           scale=G.softmax_reverse_scale(yh, dyh, before if alpha else None, alpha))
                 dx.check("dx")
             G.softmax(x.t, x.t)
-            G.compare(x.t, O.softmax_ij_j(xh), dtype, f"softmax short in place ({m},{n})", atol=G.SOFTMAX_ATOL[dtype])
+            G.compare(x.t, O.softmax_ij_j(xh), dtype, f"softmax short in place ({m},{n})", **G.softmax_tol(dtype))
             x.check("in place")
 
 
@@ -880,7 +880,7 @@ def test_special_values_follow_the_closed_forms(dtype, n):
     xh = G.host(xd.t)
     with np.errstate(all="ignore"):
         ref_p, ref_y = O.softmax_ij_j(xh), O.rmsnorm_ij_j(xh, G.host(g.t), eps)
-    G.compare(p.t, ref_p, dtype, "softmax with special values", atol=G.SOFTMAX_ATOL[dtype])
+    G.compare(p.t, ref_p, dtype, "softmax with special values", **G.softmax_tol(dtype))
     G.compare(y.t, ref_y, dtype, "rmsnorm with special values")
     got_p, got_y = G.host(p.t).astype(np.float64), G.host(y.t).astype(np.float64)
     assert np.array_equal(np.isnan(got_p), np.isnan(ref_p)), "softmax: NaN exactly where the closed form is NaN"

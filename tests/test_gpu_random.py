@@ -44,7 +44,7 @@ def test_random_cases_match_the_oracle(seed):
         if op == 0:
             y = G.Guarded((m, n), dt, sh[1])
             G.softmax(x.t, y.t)
-            G.compare(y.t, O.softmax_ij_j(G.host(x.t)), dt, name, atol=G.SOFTMAX_ATOL[dt])
+            G.compare(y.t, O.softmax_ij_j(G.host(x.t)), dt, name, **G.softmax_tol(dt))
             y.check(name)
         elif op == 1:
             y = G.Guarded((m, n), dt, sh[0])
@@ -105,7 +105,7 @@ def test_random_cases_match_the_oracle(seed):
             g = G.dev(r.normal(1, 0.02, n), dt, sh[1])
             if r.integers(0, 2):
                 G.softmax(x.t, x.t)
-                G.compare(x.t, O.softmax_ij_j(xh), dt, "softmax in place", atol=G.SOFTMAX_ATOL[dt])
+                G.compare(x.t, O.softmax_ij_j(xh), dt, "softmax in place", **G.softmax_tol(dt))
             else:
                 G.rmsnorm(x.t, g.t, x.t, 1e-6)
                 G.compare(x.t, O.rmsnorm_ij_j(xh, G.host(g.t), 1e-6), dt, "rmsnorm in place")

@@ -52,7 +52,7 @@ def test_two_streams_run_side_by_side():
     for k, j in enumerate(jobs):
         xh, gh, dyh = G.host(j["x"].t), G.host(j["g"].t), G.host(j["dy"].t)
         G.compare(j["y"].t, O.rmsnorm_ij_j(xh, gh, eps), F32, f"stream {k} rmsnorm")
-        G.compare(j["p"].t, O.softmax_ij_j(xh), F32, f"stream {k} softmax", atol=G.SOFTMAX_ATOL[F32])
+        G.compare(j["p"].t, O.softmax_ij_j(xh), F32, f"stream {k} softmax", **G.softmax_tol(F32))
         rdx, rdg = O.rmsnorm_ij_j_reverse(xh, gh, dyh, eps)
         sdx, sdg = G.rmsnorm_reverse_scales(xh, gh, dyh, eps)
         G.compare(j["dx"].t, rdx, F32, f"stream {k} rmsnorm reverse dx", scale=sdx)
