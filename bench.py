@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the row-reduction / elementwise hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--no-extra] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--no-extra] [--no-cpu] [--no-ceilings]
 
 A step is one pass of the hot path over one batch of the headline workload (cfg2: RMSNorm
 forward + reverse, r32, [8192, 4096]) with all inputs resident in HBM. Successive steps
@@ -9,7 +9,10 @@ rotate over several buffer sets, and the reverse of a step works on a different 
 forward, so the 256 MiB memory-side cache cannot serve repeats. One JSON line is printed:
 whole-step throughput (`value`, GB/s of algorithmic bytes), the roofline of the dominant
 launcher measured with events on the launch stream inside the timed region, the CPU oracle
-timed on the host cores, and (unless --no-extra) forward/reverse rates of the other workloads.
+timed on the host cores with the measured parity of the GPU results against it, and (unless
+--no-extra) forward/reverse rates and roofline objects of the other workloads. Every roofline
+object also carries the rate of a plain pass with the same reads, writes and footprint
+(`copy_ceiling`, from lib/libmp_probe.so), timed in the same run.
 """
 import argparse
 import json
@@ -31,15 +34,20 @@ PROFILE_OF = {"cfg1": "cfg1_softmax", "cfg2": "cfg2_rmsnorm", "cfg3": "cfg3_soft
               "permutate": "permutate_transpose", "gemm": "gemm_rocblas_r16"}
 
 
-def traffic_from_profile(name):
-    """HBM bytes per launch of the dominant launcher, as derived from the rocprofv3 FETCH_SIZE /
-    WRITE_SIZE runs summarised under profiles/ (None when no summary is committed)."""
+def traffic_from_profile(name, direction=None):
+    """HBM bytes per launch of a launcher, as derived from the rocprofv3 FETCH_SIZE / WRITE_SIZE
+    runs summarised under profiles/ (None when no summary is committed). The summaries hold
+    `roofline_traffic_bytes_per_launch = N` for the dominant launcher and, where both directions
+    were measured, `forward_traffic_bytes_per_launch = N` / `reverse_traffic_bytes_per_launch = N`."""
     import re
     path = os.path.join(ROOT, "profiles", f"{PROFILE_OF.get(name, name)}_hbm_traffic.md")
     if not os.path.exists(path):
         return None
     with open(path) as f:
-        m = re.search(r"roofline_traffic_bytes_per_launch\s*=\s*(\d+)", f.read())
+        text = f.read()
+    m = re.search(rf"{direction}_traffic_bytes_per_launch\s*=\s*(\d+)", text) if direction else None
+    if m is None and direction in (None, "reverse"):
+        m = re.search(r"roofline_traffic_bytes_per_launch\s*=\s*(\d+)", text)
     return int(m.group(1)) if m else None
 
 
@@ -165,6 +173,118 @@ def rates(w, fwd_ms, rev_ms):
     return out
 
 
+def roofline_of(name, direction, nbytes, launch_ms, ceiling=None):
+    """The roofline object of one launcher: algorithmic bytes over the average launch duration
+    (events on the launch stream), against the 8 TB/s peak; `traffic` from the committed
+    FETCH_SIZE / WRITE_SIZE summary (reverse launcher of workloads that have one, else forward);
+    `copy_ceiling` is a plain pass with the same reads, writes and footprint, timed the same way
+    in this run."""
+    avg_ms = sum(launch_ms) / len(launch_ms)
+    achieved = nbytes / (avg_ms * 1e-3) / 1e9
+    out = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+           "frac": round(achieved / HBM_PEAK_GBPS, 4),
+           "traffic": traffic_from_profile(name, direction),
+           "kernel": f"{name} {direction} launcher", "bytes_per_launch": nbytes,
+           "avg_launch_ms": round(avg_ms, 5), "launches_timed": len(launch_ms)}
+    if ceiling:
+        out["copy_ceiling"] = ceiling
+        out["frac_of_copy_ceiling"] = round(achieved / ceiling["GBps"], 4)
+    return out
+
+
+_probe = {}
+
+
+def probe_lib():
+    """lib/libmp_probe.so: plain passes with a workload's stream mix (measurement only)."""
+    if "lib" not in _probe:
+        import ctypes
+        from metaphor_amd import ffi
+        path = os.path.join(ffi.LIB_DIR, "libmp_probe.so")
+        if not os.path.exists(path):
+            raise ffi.BoundaryMissing(f"{path} is not built; run `python -m metaphor_amd.kernelgen`")
+        lib = ctypes.CDLL(path)
+        pp = ctypes.POINTER(ctypes.c_void_p)
+        lib.mpProbeStreams.argtypes = [pp, pp, ctypes.c_int, ctypes.c_int, ffi.len_t, ctypes.c_int, ffi.StreamContext]
+        lib.mpProbeStreams.restype = ctypes.c_int
+        lib.mpProbeRowPairs.argtypes = [pp, ctypes.c_void_p, ctypes.c_int, ffi.len_t, ffi.len_t, ffi.StreamContext]
+        lib.mpProbeRowPairs.restype = ctypes.c_int
+        _probe["lib"] = lib
+    return _probe["lib"]
+
+
+def copy_ceiling(mix, stream_bytes, iters=20, row_pairs=None):
+    """Rate of a plain pass that reads mix[0] streams and writes mix[1] streams of stream_bytes
+    each: one-shot workgroups of 64 and of 256 threads, a 16-byte pack per lane and stream, and
+    (row_pairs = (rows, workgroups), 16 KiB rows) the structure of the paired RMSNorm reverse
+    without its arithmetic. Buffer sets rotate so that the memory-side cache cannot serve a
+    repeat; timed like the launchers, one event pair per launch, median. Best shape is reported."""
+    import ctypes
+    import torch
+    from metaphor_amd import ffi
+    lib = probe_lib()
+    nr, nw = mix
+    per_set = (nr + nw) * stream_bytes
+    sets = max(2, min(4, int((1 << 30) // per_set) + 1))
+    bufs = [[torch.empty(stream_bytes, dtype=torch.uint8, device="cuda") for _ in range(nr + nw)] for _ in range(sets)]
+    for bs in bufs:
+        for b in bs[:nr]:
+            b.zero_()
+    arr = ctypes.c_void_p * 5
+    ctx = ffi.StreamContext.from_handle(torch.cuda.current_stream().cuda_stream)
+    shapes = {}
+
+    def run(tag, launch):
+        for i in range(3):
+            launch(bufs[i % sets])
+        pairs = []
+        for i in range(iters):
+            a, b = _events(2)
+            a.record()
+            launch(bufs[i % sets])
+            b.record()
+            pairs.append((a, b))
+        torch.cuda.synchronize()
+        ms = _median([a.elapsed_time(b) for a, b in pairs])
+        shapes[tag] = round((nr + nw) * stream_bytes / (ms * 1e-3) / 1e9, 1)
+
+    for block in (64, 256):
+        def launch(bs, block=block):
+            ins = arr(*[b.data_ptr() for b in bs[:nr]])
+            outs = arr(*[b.data_ptr() for b in bs[nr:]])
+            rc = lib.mpProbeStreams(ins, outs, nr, nw, stream_bytes, block, ctx)
+            assert rc == 0, "probe refused the stream mix"
+        run(f"one-shot {block} threads", launch)
+    if row_pairs and nw == 1 and nr <= 2:
+        rows, wgs = row_pairs
+
+        def launch(bs):
+            ins = arr(*[b.data_ptr() for b in bs[:nr]])
+            rc = lib.mpProbeRowPairs(ins, bs[nr].data_ptr(), nr, rows, wgs, ctx)
+            assert rc == 0
+        run(f"row pairs, {wgs} workgroups of 1024", launch)
+    best = max(shapes, key=shapes.get)
+    del bufs
+    torch.cuda.empty_cache()
+    return {"GBps": shapes[best], "shape": best, "mix": f"{nr}R+{nw}W", "stream_bytes": stream_bytes,
+            "buffer_sets": sets, "all_shapes_GBps": shapes}
+
+
+def ceilings_for(w):
+    """Copy ceilings of a workload's forward and reverse stream mixes (None for the matrix workloads)."""
+    if not hasattr(w, "fwd_mix") or hasattr(w, "fwd_flops"):
+        return None, None
+    fb = w.fwd_bytes // sum(w.fwd_mix)
+    if fb % 16:
+        return None, None
+    pairs = None
+    if w.name == "cfg2":
+        pairs = (w.shape[0], 256)
+    fwd = copy_ceiling(w.fwd_mix, fb, row_pairs=pairs)
+    rev = copy_ceiling(w.rev_mix, w.rev_bytes // sum(w.rev_mix), row_pairs=pairs) if w.has_reverse else None
+    return fwd, rev
+
+
 def cpu_baseline_cfg2(w, budget_s=12.0):
     """The fp64 oracle on the host cores over the same bytes: whole cfg2 passes (forward, then
     the row-parallel reverse) until about `budget_s` seconds are spent. Also returns the
@@ -193,11 +313,26 @@ def cpu_baseline_cfg2(w, budget_s=12.0):
     sdx, sdg = G.rmsnorm_reverse_scales(x, g, dy, w.eps)
     G.compare(w.y, y, torch.float32, "bench cfg2 y")
     G.compare(w.dx, dx, torch.float32, "bench cfg2 dx", scale=sdx)
-    G.compare(w.dgain, dg, torch.float32, "bench cfg2 dgain", rowwise=False, scale=sdg)
+    G.compare(w.dgain, dg, torch.float32, "bench cfg2 dgain", rowwise=False)
+
+    def numbers(got, ref, rowwise, scale=None):
+        st = G.parity_stats(got, ref, torch.float32, rowwise=rowwise, scale=scale)
+        return {"n": st["n"], "max_abs": float(f"{st['max_abs']:.3e}"), "max_rel": float(f"{st['max_rel']:.3e}"),
+                "violations": st["violations"]}
+
+    parity = {
+        "reference": "fp64 oracle (oracle/mp_oracle.c) on the same input bytes, whole [8192, 4096] problem",
+        "bound": "|got - ref| <= 1e-5 * max(|ref|, RMS(ref row)); dgain: RMS of the whole vector; "
+                 "max_rel is the largest |got - ref| / max(|ref|, RMS)",
+        "y": numbers(w.y, y, True),
+        "dx": numbers(w.dx, dx, True),
+        "dgain": numbers(w.dgain, dg, False),
+        "dx_with_cancellation_scale": numbers(w.dx, dx, True, sdx),
+    }
     return {"value": round(gbps, 3), "unit": "GB/s", "cores": cores, "kind": "port",
             "rows_per_s": round(passes * w.rows / spent, 1),
             "sample": f"{passes} full passes of cfg2 (forward + reverse, all {w.rows} rows), "
-                      f"{spent:.1f} s on {cores} OpenMP threads"}, "pass (r32 1e-5 relative)"
+                      f"{spent:.1f} s on {cores} OpenMP threads"}, parity
 
 
 def main():
@@ -208,6 +343,7 @@ def main():
     ap.add_argument("--workload", default="cfg2", choices=sorted(SETS))
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity check")
+    ap.add_argument("--no-ceilings", action="store_true", help="skip the plain-copy ceilings of each stream mix")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (rows shard without "
@@ -230,9 +366,15 @@ def main():
     fwd_ms, rev_ms = time_each(sets, max(20, min(args.steps, 100)))
 
     dom_bytes, dom_name = (w.rev_bytes, "reverse") if w.has_reverse else (w.fwd_bytes, "forward")
-    avg_ms = sum(dom_ms) / len(dom_ms)
-    achieved = dom_bytes / (avg_ms * 1e-3) / 1e9
-    traffic = traffic_from_profile(name)
+    cpu_line = parity = None
+    if not args.no_cpu and name == "cfg2":
+        import contextlib
+        with contextlib.redirect_stdout(sys.stderr):  # stdout carries the one JSON line only
+            cpu_line, parity = cpu_baseline_cfg2(w)
+    per_workload = rates(w, fwd_ms, rev_ms)
+    del sets
+    torch.cuda.empty_cache()
+    fwd_ceiling, rev_ceiling = (None, None) if args.no_ceilings else ceilings_for(w)
 
     line = {
         "metric": "achieved HBM GB/s (% of peak) + rows/s, softmax/RMSNorm/elementwise fwd+rev",
@@ -247,29 +389,32 @@ def main():
         "vs_baseline": None,
         "dtype": {"cfg3": "f16", "gemm": "f16"}.get(name, "f32"),
         "data": "synthetic",
-        "config": {"workload": f"{name}: {W.DESCRIPTION[name]}", "buffer_sets": len(sets),
+        "config": {"workload": f"{name}: {W.DESCRIPTION[name]}", "buffer_sets": SETS[name],
                    "bytes_per_step": step_bytes},
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "rows_per_s": round(args.steps * w.rows / dt, 1),
-        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(achieved / HBM_PEAK_GBPS, 4), "traffic": traffic,
-                     "kernel": f"{name} {dom_name} launcher", "bytes_per_launch": dom_bytes,
-                     "avg_launch_ms": round(avg_ms, 5), "launches_timed": len(dom_ms)},
-        name: rates(w, fwd_ms, rev_ms),
+        # the dominant launcher, from events sampled inside the timed region
+        "roofline": roofline_of(name, dom_name, dom_bytes, dom_ms, rev_ceiling if w.has_reverse else fwd_ceiling),
+        name: per_workload,
     }
+    if w.has_reverse:
+        line[name]["roofline_fwd"] = roofline_of(name, "forward", w.fwd_bytes, fwd_ms, fwd_ceiling)
+    avg_ms = line["roofline"]["avg_launch_ms"]
     if name == "cfg1":
-        g_ms, same = graph_forward_ms(sets)
+        g_sets = make_sets(name)
+        g_ms, same = graph_forward_ms(g_sets)
         line[name].update({"fwd_graph_ms": round(g_ms, 5), "fwd_graph_matches_eager": same,
                            "fwd_graph_GBps": round(w.fwd_bytes / (g_ms * 1e-3) / 1e9, 1)})
+        del g_sets
 
     if name in MFMA_PEAK_TFLOPS:  # the matrix product is priced in flops against the matrix cores
         tf = w.rev_flops / (avg_ms * 1e-3) / 1e12
         line["roofline"].update({"bound": "mfma", "achieved": round(tf, 1), "peak": MFMA_PEAK_TFLOPS[name],
                                  "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
                                  "flops_per_launch": w.rev_flops})
-    if not args.no_cpu and name == "cfg2":
-        line["cpu_baseline"], line["parity"] = cpu_baseline_cfg2(w)
-    del sets, w
+    if cpu_line is not None:
+        line["cpu_baseline"], line["parity"] = cpu_line, parity
+    del w
     torch.cuda.empty_cache()
 
     if not args.no_extra:
@@ -278,17 +423,27 @@ def main():
             if other == name:
                 continue
             osets = make_sets(other)
+            o = osets[0]
             k = max(10, min(args.steps, 40 if other in ("cfg3", "cfg4") else 100))
             time_steps(osets, 5, 2)
             f_ms, r_ms = time_each(osets, k)
-            extra[other] = rates(osets[0], f_ms, r_ms)
+            extra[other] = rates(o, f_ms, r_ms)
             extra[other]["workload"] = W.DESCRIPTION[other]
             if other == "cfg1":  # launch-bound: also the rate with the host out of the loop
                 g_ms, same = graph_forward_ms(osets)
                 extra[other]["fwd_graph_ms"] = round(g_ms, 5)
-                extra[other]["fwd_graph_GBps"] = round(osets[0].fwd_bytes / (g_ms * 1e-3) / 1e9, 1)
+                extra[other]["fwd_graph_GBps"] = round(o.fwd_bytes / (g_ms * 1e-3) / 1e9, 1)
                 extra[other]["fwd_graph_matches_eager"] = same
             del osets
+            torch.cuda.empty_cache()
+            if other.startswith("cfg"):  # the same roofline object as the headline workload carries
+                f_ceil, r_ceil = (None, None) if args.no_ceilings or other == "cfg1" else ceilings_for(o)
+                if o.has_reverse:
+                    extra[other]["roofline"] = roofline_of(other, "reverse", o.rev_bytes, r_ms, r_ceil)
+                    extra[other]["roofline_fwd"] = roofline_of(other, "forward", o.fwd_bytes, f_ms, f_ceil)
+                else:
+                    extra[other]["roofline"] = roofline_of(other, "forward", o.fwd_bytes, f_ms, f_ceil)
+            del o
             torch.cuda.empty_cache()
         line["other_workloads"] = extra
 

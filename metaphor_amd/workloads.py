@@ -150,6 +150,9 @@ class Workload:
     name = ""
     dtype = torch.float32
     has_reverse = True
+    # (streams read, streams written) by one forward / reverse call; every stream has
+    # fwd_bytes / (reads + writes) bytes. bench.py times a plain pass with the same mix beside it.
+    fwd_mix, rev_mix = (1, 1), (2, 1)
 
     def forward(self):
         raise NotImplementedError
@@ -240,6 +243,7 @@ class Cfg3(Workload):
 class Cfg4(Workload):
     name, dtype = "cfg4", torch.float32
     n = 1 << 28
+    fwd_mix, rev_mix = (4, 1), (5, 4)
 
     def __init__(self, seed=0, n=None):
         self.n = n or self.n

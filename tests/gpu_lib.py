@@ -166,8 +166,12 @@ def compare(got, ref, dtype, what, rowwise=True, rtol=None, atol=None, scale=Non
     st = parity_stats(got, ref, dtype, rowwise, rtol, atol, scale)
     PARITY_LOG.append((what, st))
     if st["n"]:
+        plain = ""
+        if scale is not None:  # how the same result stands against the bound without the scale term
+            p = parity_stats(got, ref, dtype, rowwise, rtol, atol, None)
+            plain = f" (without scale: worst {p['worst']:.3f}, violations {p['violations']})"
         print(f"[parity] {what}: n={st['n']} max_abs={st['max_abs']:.3e} max_rel={st['max_rel']:.3e} "
-              f"worst err/bound={st['worst']:.3f} violations={st['violations']}", flush=True)
+              f"worst err/bound={st['worst']:.3f} violations={st['violations']}{plain}", flush=True)
     if st["violations"]:
         raise AssertionError(
             f"{what}: {st['violations']} of {st['n']} outside tolerance; worst at {st['at']}: "
@@ -191,18 +195,19 @@ def softmax_reverse_scale(y, dy, dx_in=None, alpha=0.0):
 
 
 def rmsnorm_reverse_scales(x, g, dy, eps, dx_in=None, dg_in=None, alpha=0.0):
-    """dx = r*dy*g - r^3*x*c: size of its two terms; dg = sum_i dy*x*r: sum of |terms|."""
+    """dx = r*dy*g - r^3*x*c: the size of its two terms (they cancel completely for rows of one
+    element, and largely for rows of a few). The second value, for dg = sum_i dy*x*r, is None: the
+    gain gradient is held to the plain bound rtol * max(|ref|, RMS(ref)). Over the 2064 dg
+    comparisons of this suite its worst error is 0.24 of that bound (16-row fp32 partial sums and an
+    fp64 finish leave no visible cancellation error)."""
     x, g, dy = (np.asarray(a, np.float64) for a in (x, g, dy))
     n = x.shape[-1]
     r = 1.0 / np.sqrt((x * x).mean(axis=-1, keepdims=True) + eps)
     c_abs = np.abs(dy * g * x).sum(axis=-1, keepdims=True) / n
     sdx = r * (np.abs(dy * g) + np.abs(x) * r * r * c_abs)
-    sdg = np.abs(dy * x * r).sum(axis=0)
     if dx_in is not None:
         sdx = sdx + abs(alpha) * np.abs(np.asarray(dx_in, np.float64))
-    if dg_in is not None:
-        sdg = sdg + abs(alpha) * np.abs(np.asarray(dg_in, np.float64))
-    return sdx, sdg
+    return sdx, None
 
 
 # ---------------------------------------------------------------- launcher wrappers
