@@ -46,7 +46,8 @@ def traffic_from_profile(name, direction=None):
     with open(path) as f:
         text = f.read()
     m = re.search(rf"{direction}_traffic_bytes_per_launch\s*=\s*(\d+)", text) if direction else None
-    if m is None and direction in (None, "reverse"):
+    forward_is_dominant = "forward_traffic_bytes_per_launch" not in text  # a workload without a reverse
+    if m is None and (direction in (None, "reverse") or forward_is_dominant):
         m = re.search(r"roofline_traffic_bytes_per_launch\s*=\s*(\d+)", text)
     return int(m.group(1)) if m else None
 
@@ -154,6 +155,21 @@ def graph_forward_ms(sets, replays=50):
     torch.cuda.synchronize()
     same = all(torch.equal(s.y, e) for s, e in zip(sets, eager))
     return a.elapsed_time(b) / (replays * len(sets)), same
+
+
+def native_launch_cost(launches=4000):
+    """Cost of one cfg1-sized launch to a native caller: lib/host_check --launch-cost enqueues the
+    softmax launcher back to back from C++ (no interpreter, no ctypes) in a child process and
+    reports the host time per call and the time per launch until the stream drains."""
+    import subprocess
+    from metaphor_amd import ffi
+    exe = os.path.join(ffi.LIB_DIR, "host_check")
+    if not os.path.exists(exe):
+        return None
+    res = subprocess.run([exe, "--launch-cost", str(launches)], capture_output=True, text=True, timeout=120)
+    if res.returncode != 0:
+        return {"error": (res.stderr or res.stdout).strip()[-200:]}
+    return json.loads(res.stdout.strip().splitlines()[-1])
 
 
 def rates(w, fwd_ms, rev_ms):
@@ -404,7 +420,8 @@ def main():
         g_sets = make_sets(name)
         g_ms, same = graph_forward_ms(g_sets)
         line[name].update({"fwd_graph_ms": round(g_ms, 5), "fwd_graph_matches_eager": same,
-                           "fwd_graph_GBps": round(w.fwd_bytes / (g_ms * 1e-3) / 1e9, 1)})
+                           "fwd_graph_GBps": round(w.fwd_bytes / (g_ms * 1e-3) / 1e9, 1),
+                           "native_caller": native_launch_cost()})
         del g_sets
 
     if name in MFMA_PEAK_TFLOPS:  # the matrix product is priced in flops against the matrix cores
@@ -434,6 +451,7 @@ def main():
                 extra[other]["fwd_graph_ms"] = round(g_ms, 5)
                 extra[other]["fwd_graph_GBps"] = round(o.fwd_bytes / (g_ms * 1e-3) / 1e9, 1)
                 extra[other]["fwd_graph_matches_eager"] = same
+                extra[other]["native_caller"] = native_launch_cost()
             del osets
             torch.cuda.empty_cache()
             if other.startswith("cfg"):  # the same roofline object as the headline workload carries

@@ -12,6 +12,7 @@
  * Part 3 is the matrix side: the reference's src/examples/experimental.zig, every inner-product
  * expression, permutate, reduce / broadcast, and checkpoint files.
  */
+#include <chrono>
 #include <cmath>
 #include <cstdio>
 #include <cstdlib>
@@ -354,9 +355,39 @@ static int matrix_ops(mp::Stream stream) {
   return 0;
 }
 
+/* What one launch costs a native caller: `launches` calls of launch_softmax_ij_j_r32 on
+ * [256, 1024] (the smallest benchmark configuration, a 2.7 us kernel) enqueued back to back on
+ * one stream of this library, no interpreter in between. enqueue_us is the host time per call,
+ * back_to_back_us the time per launch until the stream has drained. */
+static int launch_cost(int launches) {
+  mp::device::init(0);
+  mp::Stream s = mp::stream::init();
+  const size_t m = 256, n = 1024, bytes = m * n * sizeof(float);
+  void* x = mpMemAlloc(bytes, s->context);
+  void* y = mpMemAlloc(bytes, s->context);
+  std::vector<float> h(m * n, 0.25f);
+  mpMemcpyHtoD(x, h.data(), bytes, s->context);
+  for (int i = 0; i < 200; ++i) launch_softmax_ij_j_r32(x, y, nullptr, m, n, s->context);
+  mpStreamSynchronize(s->context);
+  const auto t0 = std::chrono::steady_clock::now();
+  for (int i = 0; i < launches; ++i) launch_softmax_ij_j_r32(x, y, nullptr, m, n, s->context);
+  const auto t1 = std::chrono::steady_clock::now();
+  mpStreamSynchronize(s->context);
+  const auto t2 = std::chrono::steady_clock::now();
+  mpCheckLastError();
+  const double enq = std::chrono::duration<double, std::micro>(t1 - t0).count() / launches;
+  const double all = std::chrono::duration<double, std::micro>(t2 - t0).count() / launches;
+  printf("{\"launches\": %d, \"enqueue_us\": %.3f, \"back_to_back_us\": %.3f}\n", launches, enq, all);
+  mpMemFree(x, s->context);
+  mpMemFree(y, s->context);
+  mp::stream::deinit(s);
+  return 0;
+}
+
 int main(int argc, char** argv) {
+  if (argc == 3 && std::string(argv[1]) == "--launch-cost") return launch_cost(atoi(argv[2]) > 0 ? atoi(argv[2]) : 2000);
   if (argc != 2) {
-    fprintf(stderr, "usage: host_check <output directory>\n");
+    fprintf(stderr, "usage: host_check <output directory> | host_check --launch-cost <launches>\n");
     return 2;
   }
   out_dir = argv[1];
