@@ -7,8 +7,8 @@
  *   - r16/r32/r64 keep their storage size (tensor_types.h:20-33); on the C side
  *     r16 is an opaque 2-byte struct, on the device side it is _Float16;
  *   - StreamContext keeps its 16-byte, two-pointer, pass-by-value layout; slot 0 now
- *     carries a hipStream_t, slot 1 is reserved for a BLAS handle and is NULL in this
- *     library (no contraction is on this path).
+ *     carries a hipStream_t, slot 1 the BLAS state of the stream (see below), NULL for a
+ *     stream that has none.
  *   - WAVE_SIZE is 64 (the reference's WARP_SIZE = 32, tensor_types.h:6).
  */
 #ifndef MP_TENSOR_TYPES_H

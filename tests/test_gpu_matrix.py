@@ -398,3 +398,39 @@ def test_sums_and_products_of_tall_narrow_matrices(dtype):
                     y.check(op)
                 for gd in (x, si, sj, v, d, u, e):
                     gd.check("narrow")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_inner_product_on_both_sides_of_every_dispatch_threshold(dtype):
+    """The launcher picks between the library's GEMM and four kernels of its own by size thresholds
+    (rows from 1024, tensors from 2^21 elements, contractions from 8192, sides of at most 8, rows of
+    C of at most 128): the shape just below and just above each of them, for both transposes and a
+    blend, must give the same answer whichever kernel takes it."""
+    r = rng(53)
+    shapes = [
+        # tiny map: n, k <= 8 and m >= 1024
+        (1023, 8, 8), (1024, 8, 8), (1024, 9, 8), (1024, 8, 9),
+        # few terms: 2 <= n <= 8 < k <= 128 and m * k >= 2^21
+        (16384, 8, 127), (16384, 8, 128), (16384, 8, 129), (16383, 8, 128), (262144, 2, 8), (262144, 2, 9),
+        (262144, 1, 9), (233017, 8, 9), (233018, 9, 9),
+        # few dots: 2 <= k <= 8 < n, m >= 1024 and m * n >= 2^21
+        (1023, 2051, 8), (1024, 2048, 8), (1024, 2047, 8), (1024, 2048, 9), (2048, 1024, 2), (2048, 1023, 2),
+        # small product: m, k <= 8 and n >= 8192
+        (8, 8191, 8), (8, 8192, 8), (9, 8192, 8), (8, 8192, 9), (4, 8192, 4), (4, 8191, 4),
+    ]
+    with G.BlasStream() as bs:
+        for (m, n, k) in shapes:
+            for form, ta, tb in FORMS:
+                for (alpha, beta) in ((1.0, 0.0), (-0.5, 0.75)):
+                    G.say(f"threshold {form} dtype={dtype} m,n,k=({m},{n},{k}) alpha={alpha} beta={beta}")
+                    a = G.dev(r.normal(0, 1, (n, m) if ta else (m, n)), dtype)
+                    b = G.dev(r.normal(0, 1, (k, n) if tb else (n, k)), dtype)
+                    c = G.dev(r.normal(0, 1, (m, k)), dtype)
+                    before = G.host(c.t).copy()
+                    bs.inner_product(form, a.t, b.t, alpha, c.t, beta, m, n, k)
+                    ref, scale = O.inner_product(G.host(a.t), G.host(b.t), alpha, before if beta else None, beta,
+                                                 ta=ta, tb=tb, with_scale=True)
+                    G.compare(c.t, ref, dtype, f"threshold {form} ({m},{n},{k}) {alpha},{beta}", rowwise=False,
+                              scale=scale)
+                    for gd in (a, b, c):
+                        gd.check("threshold")
