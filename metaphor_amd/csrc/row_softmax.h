@@ -704,9 +704,11 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_rev_stream(
  * workgroup that stops waiting reads the whole row again for the dot product, which is why the
  * shared path is not taken when dx overwrites y or dy. */
 /* packs of y and of dy per thread: kept in their storage type (four registers a pack whatever T
- * is) and widened where they are used, so a workgroup holds the same 48 KiB of each for r16, r32
- * and r64 within 64 registers a thread */
-constexpr int CLUSTER_REV_NV = 3;
+ * is) and widened where they are used, so a workgroup holds the same 64 KiB of each for r16, r32
+ * and r64 within 64 registers a thread (62-64 used, no spills), which keeps two workgroups a CU.
+ * Measured on r32, 2 / 3 / 4 / 5 / 6 / 8 packs (5 and more: one workgroup a CU):
+ * [512, 151936] 190 / 171 / 163 / 188 / 190 / 179 us, [2048, 50257] 244 / 217 / 211 / 238 / 243 / 225 us. */
+constexpr int CLUSTER_REV_NV = 4;
 
 template <class T, int W, bool BLEND>
 __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_rev_cluster(
