@@ -195,13 +195,18 @@ def roofline_of(name, direction, nbytes, launch_ms, ceiling=None):
     FETCH_SIZE / WRITE_SIZE summary (reverse launcher of workloads that have one, else forward);
     `copy_ceiling` is a plain pass with the same reads, writes and footprint, timed the same way
     in this run."""
-    avg_ms = sum(launch_ms) / len(launch_ms)
+    # an event pair also spans whatever the host does between recording the first event and
+    # enqueueing the launch; a sample several times the median is such a host stall, not a launch
+    med = _median(launch_ms)
+    kept = [t for t in launch_ms if t <= 3.0 * med]
+    avg_ms = sum(kept) / len(kept)
     achieved = nbytes / (avg_ms * 1e-3) / 1e9
     out = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
            "frac": round(achieved / HBM_PEAK_GBPS, 4),
            "traffic": traffic_from_profile(name, direction),
            "kernel": f"{name} {direction} launcher", "bytes_per_launch": nbytes,
-           "avg_launch_ms": round(avg_ms, 5), "launches_timed": len(launch_ms)}
+           "avg_launch_ms": round(avg_ms, 5), "launches_timed": len(kept),
+           "host_stalls_dropped": len(launch_ms) - len(kept)}
     if ceiling:
         out["copy_ceiling"] = ceiling
         out["frac_of_copy_ceiling"] = round(achieved / ceiling["GBps"], 4)
