@@ -72,6 +72,35 @@ inline size_t cluster_size_for_scratch(int c) {
 #endif
 }
 
+/* A row whose first pack is not at the start of a 128-byte line moves every chunk boundary back
+ * by the packs it is past one (at most 7), so that each wavefront's kilobyte covers eight whole
+ * lines rather than parts of nine: the first workgroup's chunk is that much shorter and its first
+ * lanes idle. Only when the C chunks still reach the end of the row; launchers size the chunks
+ * for CLUSTER_SKEW_MAX packs more than the row has, so that they do unless the tile is full. */
+constexpr int CLUSTER_SKEW_MAX = 7;
+template <class T>
+__device__ __forceinline__ int cluster_skew(const T* body, int C, int packs_per_block, int nvec) {
+  const int skew = (int)((reinterpret_cast<uintptr_t>(body) >> 4) & 7u);
+  return C * packs_per_block - nvec >= CLUSTER_SKEW_MAX ? skew : 0;
+}
+
+/* Packs of a row that each of its C workgroups takes: an even share, rounded up to whole
+ * kilobytes (64 packs, what a wavefront reads at once) so that a chunk does not start in the
+ * middle of a wavefront's access. Measured on the softmax forward: [512, 151936] r32 104.0 ->
+ * 102.1 us, [2048, 50257] and [1000, 100000] equal within their scatter, never slower. Shares
+ * below a pack a thread (only the test build's small chunks) stay as they are, so that those
+ * tests still spread a short row over many workgroups. The last workgroups get what is left.
+ * `spare` packs are added to the row before it is shared out when the register tile allows it. */
+inline int cluster_chunk_packs(size_t packs, int C, size_t tile, size_t spare = 0) {
+  if ((packs + spare + (size_t)C - 1) / (size_t)C <= tile) packs += spare;
+  size_t share = (packs + (size_t)C - 1) / (size_t)C;
+  if (share >= (size_t)CLUSTER_THREADS) {
+    const size_t whole = (share + WAVE - 1) / WAVE * WAVE;
+    if (whole <= tile && whole * (size_t)(C - 1) < packs) share = whole; /* no workgroup left empty */
+  }
+  return (int)share;
+}
+
 /* Sums over the C workgroups that share a row. Every workgroup calls this with its NVAL partial
  * sums; all threads return with the row totals in vals, and the result says whether every
  * partner was heard from. `mine` points at this row's C * NVAL scratch words, zero before the

@@ -211,14 +211,14 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void rmsnorm_fwd_cluster(
   T* yr = y + row * n;
   const RowGeom<T, W> g(xr, n, true);
   const T* body = xr + g.head;
-  const int lo = rank * packs_per_block;
+  const int lo = rank * packs_per_block - cluster_skew(body, C, packs_per_block, g.nvec);
   const int hi = lo + packs_per_block < g.nvec ? lo + packs_per_block : g.nvec;
 
   V v[NV];
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int p = lo + k * G + lane;
-    if (p < hi) {
+    if (p >= 0 && p < hi) {
       v[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(body + (size_t)p * W));
     } else {
 #pragma unroll
@@ -271,7 +271,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void rmsnorm_fwd_cluster(
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int p = lo + k * G + lane;
-    if (p < hi) {
+    if (p >= 0 && p < hi) {
       P gv[W], out[W];
       if (gain_packed) {
         load_pack<T, W>(gbody + (size_t)p * W, gv);
@@ -1075,7 +1075,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
     if (C >= 1 && (C == 1 || shareable) && m * (size_t)C < 0x7fffffffull) {
       using Word = typename slot_word<P>::type;
       Word* slots = static_cast<Word*>(scratch);
-      const int ppb = (int)(((n + W - 1) / W + C - 1) / C);
+      const int ppb = cluster_chunk_packs((n + W - 1) / W, C, (size_t)CLUSTER_THREADS * NORM_CLUSTER_NV, CLUSTER_SKEW_MAX);
       require(ppb <= CLUSTER_THREADS * NORM_CLUSTER_NV, "rmsnorm: cluster chunk exceeds the register tile");
       if (C > 1) {
         const size_t words = m * (size_t)C;
@@ -1178,7 +1178,7 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
     if (S > m) S = m;
     if (S == 0) S = 1;
     rows = (unsigned)S;
-    const int ppb = (int)((packs + C - 1) / C);
+    const int ppb = cluster_chunk_packs(packs, C, (size_t)CLUSTER_THREADS * norm_rev_cluster_nv<T>());
     require(ppb <= CLUSTER_THREADS * norm_rev_cluster_nv<T>(), "rmsnorm reverse: cluster chunk exceeds the register tile");
     Word* slots = reinterpret_cast<Word*>(partials + rmsnorm_reverse_partial_rows(m) * n);
     if (C > 1) {

@@ -439,7 +439,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
   T* yr = y + row * n;
   const RowGeom<T, W> g(xr, n, true);
   const T* body = xr + g.head;
-  const int lo = rank * packs_per_block;
+  const int lo = rank * packs_per_block - cluster_skew(body, C, packs_per_block, g.nvec);
   const int hi = lo + packs_per_block < g.nvec ? lo + packs_per_block : g.nvec;
 
   /* this workgroup's chunk; rank 0 also holds the row's head / tail scalars */
@@ -450,7 +450,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int p = lo + k * G + lane;
-    if (p < hi) {
+    if (p >= 0 && p < hi) {
       if constexpr (RAW) v[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(body + (size_t)p * W));
       else load_pack_nt<T, W>(body + (size_t)p * W, v[k]);
     } else {
@@ -558,7 +558,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = lo + k * G + lane;
-      if (p < hi) {
+      if (p >= 0 && p < hi) {
         P out[W];
 #pragma unroll
         for (int i = 0; i < W; ++i) out[i] = exp_shifted((P)v[k][i], shM) * inv;
@@ -570,7 +570,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = lo + k * G + lane;
-      if (p < hi) {
+      if (p >= 0 && p < hi) {
 #pragma unroll
         for (int i = 0; i < W; ++i) v[k][i] *= scale;
         store_pack_nt<T, W>(ybody + (size_t)p * W, v[k]);
@@ -731,14 +731,14 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_rev_cluster(
   const T* ybody = yr + g.head;
   const T* gbody = gr + g.head;
   T* dbody = dr + g.head;
-  const int lo = rank * packs_per_block;
+  const int lo = rank * packs_per_block - cluster_skew(ybody, C, packs_per_block, g.nvec);
   const int hi = lo + packs_per_block < g.nvec ? lo + packs_per_block : g.nvec;
 
   V a[NV], b[NV];
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int p = lo + k * G + lane;
-    if (p < hi) {
+    if (p >= 0 && p < hi) {
       a[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(ybody + (size_t)p * W));
       b[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(gbody + (size_t)p * W));
     } else {
@@ -800,7 +800,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_rev_cluster(
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int p = lo + k * G + lane;
-    if (p < hi) {
+    if (p >= 0 && p < hi) {
       P out[W];
 #pragma unroll
       for (int i = 0; i < W; ++i) out[i] = (P)a[k][i] * ((P)b[k][i] - dot);
@@ -873,7 +873,7 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   if (C >= 1 && (C == 1 || shareable) && m * (size_t)C < 0x7fffffffull) {
     using Word = typename slot_word<P>::type;
     Word* slots = static_cast<Word*>(scratch);
-    const int ppb = (int)((packs + C - 1) / C);
+    const int ppb = cluster_chunk_packs(packs, C, (size_t)CLUSTER_THREADS * cluster_nv<T>(), CLUSTER_SKEW_MAX);
     require(ppb <= CLUSTER_THREADS * cluster_nv<T>(), "softmax: cluster chunk exceeds the register tile");
     if (C > 1) {
       const size_t words = m * (size_t)C * 2;
@@ -958,7 +958,7 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   if (C >= 1 && (C == 1 || (scratch != nullptr && distinct)) && m * (size_t)C < 0x7fffffffull) {
     using Word = typename slot_word<P>::type;
     Word* slots = static_cast<Word*>(scratch);
-    const int ppb = (int)((packs + C - 1) / C);
+    const int ppb = cluster_chunk_packs(packs, C, (size_t)CLUSTER_THREADS * CLUSTER_REV_NV, CLUSTER_SKEW_MAX);
     require(ppb <= CLUSTER_THREADS * CLUSTER_REV_NV, "softmax reverse: cluster chunk exceeds the register tile");
     if (C > 1) {
       const size_t words = m * (size_t)C;

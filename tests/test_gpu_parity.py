@@ -428,6 +428,36 @@ def test_softmax_forward_cluster_path(dtype, packs, spin):
                 y.check("y")
 
 
+@pytest.mark.parametrize("dtype", [torch.float16, torch.float32], ids=["r16", "r32"])
+def test_shared_rows_starting_at_every_offset_from_a_128_byte_line(dtype):
+    """Rows of 16 bytes more than a multiple of 128: nine consecutive rows start at each of the
+    eight pack offsets from a line, and the chunks of a shared row move back by that offset (the
+    first workgroup's first lanes idle, the last chunk ends at the row's end). Forward, reverse
+    and RMSNorm forward of the library as shipped, whole outputs against the oracle."""
+    r = rng(35)
+    per_pack = 16 // torch.empty((), dtype=dtype).element_size()
+    n = 10001 * per_pack
+    m = 9
+    for shift in (0, 1):
+        G.say(f"line offsets dtype={dtype} ({m},{n}) shift={shift}")
+        x = G.dev(r.normal(0, 2, (m, n)), dtype, shift)
+        y = G.Guarded((m, n), dtype, shift)
+        G.softmax(x.t, y.t)
+        G.compare(y.t, O.softmax_ij_j(G.host(x.t)), dtype, f"softmax line offsets shift {shift}", **G.softmax_tol(dtype))
+        dy = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+        dx = G.Guarded((m, n), dtype, shift)
+        G.softmax_reverse(y.t, dy.t, dx.t, 0.0)
+        yh, dyh = G.host(y.t), G.host(dy.t)
+        G.compare(dx.t, O.softmax_ij_j_reverse(yh, dyh), dtype, f"softmax rev line offsets shift {shift}",
+                  scale=G.softmax_reverse_scale(yh, dyh))
+        g = G.dev(r.normal(1, 0.02, n), dtype, shift)
+        z = G.Guarded((m, n), dtype, shift)
+        G.rmsnorm(x.t, g.t, z.t, 1e-6)
+        G.compare(z.t, O.rmsnorm_ij_j(G.host(x.t), G.host(g.t), 1e-6), dtype, f"rmsnorm line offsets shift {shift}")
+        for b in (x, y, dy, dx, g, z):
+            b.check("line offsets")
+
+
 def test_softmax_long_rows_without_scratch_take_the_two_pass_kernel():
     r = rng(33)
     for (m, n) in [(3, 151936), (4, 50257)]:
