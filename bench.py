@@ -25,7 +25,8 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0
-SETS = {"cfg1": 16, "cfg2": 4, "cfg3": 2, "cfg4": 2, "cfg5a": 3, "cfg5b": 3, "copy": 2, "permutate": 2, "gemm": 2}
+SETS = {"cfg1": 16, "cfg2": 4, "cfg3": 2, "cfg4": 2, "cfg5a": 3, "cfg5b": 3, "copy": 2, "permutate": 2, "gemm": 2,
+        "chain": 2}
 MFMA_PEAK_TFLOPS = {"gemm": 2500.0}  # dense fp16 matrix rate of the MI355X
 
 
@@ -446,7 +447,7 @@ def main():
                 continue
             osets = make_sets(other)
             o = osets[0]
-            k = max(10, min(args.steps, 40 if other in ("cfg3", "cfg4") else 100))
+            k = max(10, min(args.steps, 40 if other in ("cfg3", "cfg4", "chain") else 100))
             time_steps(osets, 5, 2)
             f_ms, r_ms = time_each(osets, k)
             extra[other] = rates(o, f_ms, r_ms)
@@ -459,7 +460,7 @@ def main():
                 extra[other]["native_caller"] = native_launch_cost()
             del osets
             torch.cuda.empty_cache()
-            if other.startswith("cfg"):  # the same roofline object as the headline workload carries
+            if other.startswith("cfg") or other == "chain":  # the same roofline object as the headline workload carries
                 f_ceil, r_ceil = (None, None) if args.no_ceilings or other == "cfg1" else ceilings_for(o)
                 if o.has_reverse:
                     extra[other]["roofline"] = roofline_of(other, "reverse", o.rev_bytes, r_ms, r_ceil)

@@ -1,0 +1,494 @@
+/*
+ * Elementwise expressions fused at run time: mpChainForward / mpChainReverse take an expression
+ * over add, sub, mul, neg, relu, selu as text, and run it as ONE kernel of the flat elementwise
+ * engine (elementwise.h) and its reverse as ONE kernel that writes every leaf gradient. The first
+ * call for an (expression, dtype) writes the three functors (forward, reverse that overwrites,
+ * reverse that blends), compiles them with hiprtc against the very headers this library is built
+ * from (their text is embedded at build time) and keeps the code object for the life of the
+ * process; each device loads it once. Later calls are a map lookup and a launch.
+ *
+ * The reference has no counterpart: its generator replicates fixed kernel sources at build time
+ * (file_gen.zig:200-328) and each op launches its own kernel through its own temporary
+ * (src/ops/addition.zig:37-47, src/ops/hadamard.zig:35-45). The expressions listed in
+ * chains.json take the same route at build time (chaingen.py); this file is the same generator,
+ * line for line, for expressions nobody listed. tests/test_chain_fusion.py holds the two to the
+ * same text.
+ *
+ * Errors: unlike the launchers (print and exit, src/cuda/kernel_header.h:64-98) these entry points
+ * return non-zero and enqueue nothing, because the caller has a fallback (one launch per op);
+ * mpChainError() gives the reason.
+ */
+#include "elementwise.h"
+
+#include <hip/hiprtc.h>
+
+#include <map>
+#include <memory>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "chain_fusion.h"
+#include "chain_headers.inc" /* CHAIN_HEADER_NAMES, CHAIN_HEADER_TEXT, CHAIN_HEADER_COUNT: written by the build */
+
+#ifndef MP_GPU_ARCH
+#define MP_GPU_ARCH "gfx950"
+#endif
+
+namespace {
+
+constexpr int MAX_LEAVES = 8, MAX_NODES = 64, MAX_DEVICES = 64;
+
+enum Op { LEAF, ADD, SUB, MUL, NEG, RELU, SELU };
+
+struct Node {
+  Op op;
+  int leaf;    /* LEAF: its number */
+  int arg[2];  /* indices into Expr::nodes */
+  std::string name; /* the forward value's spelling in the generated code */
+};
+
+struct Expr {
+  std::vector<Node> nodes;
+  int root = -1;
+  int leaves = 0;
+};
+
+thread_local std::string last_error;
+
+int fail(const std::string& what) {
+  last_error = what;
+  return 1;
+}
+
+/* ---------------------------------------------------------------- text -> tree */
+
+struct Parser {
+  const char* p;
+  Expr& e;
+  std::string err;
+  int next_leaf = 0; /* leaves must appear as 0, 1, 2, ... in order of first appearance */
+
+  void skip() {
+    while (*p == ' ' || *p == '\t') ++p;
+  }
+  bool take(char c) {
+    skip();
+    if (*p != c) {
+      err = std::string("expected '") + c + "' at \"" + p + "\"";
+      return false;
+    }
+    ++p;
+    return true;
+  }
+  int node() {
+    skip();
+    if ((int)e.nodes.size() >= MAX_NODES) {
+      err = "more than 64 nodes";
+      return -1;
+    }
+    const char* q = p;
+    if (*q == 'x') ++q;
+    if (*q >= '0' && *q <= '9') { /* a leaf: 3 or x3 */
+      int v = 0;
+      while (*q >= '0' && *q <= '9' && v < 1000) v = v * 10 + (*q++ - '0');
+      p = q;
+      if (v > next_leaf) {
+        err = "number the leaves in order of first appearance";
+        return -1;
+      }
+      if (v == next_leaf) ++next_leaf;
+      if (next_leaf > MAX_LEAVES) {
+        err = "more than 8 leaves";
+        return -1;
+      }
+      e.nodes.push_back(Node{LEAF, v, {-1, -1}, "in[" + std::to_string(v) + "]"});
+      return (int)e.nodes.size() - 1;
+    }
+    std::string word;
+    while ((*p >= 'a' && *p <= 'z') || *p == '_') word += *p++;
+    Op op;
+    if (word == "add") op = ADD;
+    else if (word == "sub") op = SUB;
+    else if (word == "mul") op = MUL;
+    else if (word == "neg") op = NEG;
+    else if (word == "relu") op = RELU;
+    else if (word == "selu") op = SELU;
+    else {
+      err = "unknown op \"" + word + "\"";
+      return -1;
+    }
+    if (!take('(')) return -1;
+    int a = node(), b = -1;
+    if (a < 0) return -1;
+    if (op == ADD || op == SUB || op == MUL) {
+      if (!take(',')) return -1;
+      b = node();
+      if (b < 0) return -1;
+    }
+    if (!take(')')) return -1;
+    e.nodes.push_back(Node{op, -1, {a, b}, ""});
+    return (int)e.nodes.size() - 1;
+  }
+};
+
+bool parse(const char* text, Expr& e, std::string& err) {
+  if (text == nullptr) {
+    err = "no expression";
+    return false;
+  }
+  Parser ps{text, e, "", 0};
+  e.root = ps.node();
+  if (e.root < 0) {
+    err = ps.err;
+    return false;
+  }
+  ps.skip();
+  if (*ps.p != '\0') {
+    err = std::string("trailing text \"") + ps.p + "\"";
+    return false;
+  }
+  if (e.nodes[e.root].op == LEAF) {
+    err = "a bare leaf is not a chain";
+    return false;
+  }
+  e.leaves = ps.next_leaf;
+  return true;
+}
+
+/* The expression as the cache spells it: bare leaf numbers, no blanks ("add(x0, x1)" -> "add(0,1)"). */
+void spell(const Expr& e, int n, std::string& out) {
+  static const char* const names[] = {"", "add", "sub", "mul", "neg", "relu", "selu"};
+  const Node& node = e.nodes[n];
+  if (node.op == LEAF) {
+    out += std::to_string(node.leaf);
+    return;
+  }
+  out += names[node.op];
+  out += '(';
+  spell(e, node.arg[0], out);
+  if (node.arg[1] >= 0) {
+    out += ',';
+    spell(e, node.arg[1], out);
+  }
+  out += ')';
+}
+
+/* ---------------------------------------------------------------- tree -> functor bodies
+ * The same lines, names and order as chaingen.py writes (_forward_lines, _reverse_lines). */
+
+void forward_lines(Expr& e, int n, int& counter, std::vector<std::string>& lines) {
+  Node& node = e.nodes[n];
+  if (node.op == LEAF) return;
+  forward_lines(e, node.arg[0], counter, lines);
+  if (node.arg[1] >= 0) forward_lines(e, node.arg[1], counter, lines);
+  const std::string& a = e.nodes[node.arg[0]].name;
+  const std::string b = node.arg[1] >= 0 ? e.nodes[node.arg[1]].name : "";
+  std::string rhs;
+  switch (node.op) {
+    case ADD: rhs = a + " + " + b; break;
+    case SUB: rhs = a + " - " + b; break;
+    case MUL: rhs = a + " * " + b; break;
+    case NEG: rhs = "-" + a; break;
+    case RELU: rhs = "mp::relu_value(" + a + ")"; break;
+    case SELU: rhs = "mp::selu_value(" + a + ")"; break;
+    default: break;
+  }
+  node.name = "t" + std::to_string(counter++);
+  lines.push_back("    const P " + node.name + " = " + rhs + ";");
+}
+
+void sweep(const Expr& e, int n, const std::string& adjoint, int& counter, std::vector<std::string>& lines,
+           std::vector<std::vector<std::string>>& leaf_terms) {
+  const Node& node = e.nodes[n];
+  if (node.op == LEAF) {
+    leaf_terms[node.leaf].push_back(adjoint);
+    return;
+  }
+  auto fresh = [&](const std::string& expr) {
+    const std::string name = "a" + std::to_string(counter++);
+    lines.push_back("    const P " + name + " = " + expr + ";");
+    return name;
+  };
+  const std::string& v0 = e.nodes[node.arg[0]].name;
+  switch (node.op) {
+    case ADD:
+      sweep(e, node.arg[0], adjoint, counter, lines, leaf_terms);
+      sweep(e, node.arg[1], adjoint, counter, lines, leaf_terms);
+      break;
+    case SUB:
+      sweep(e, node.arg[0], adjoint, counter, lines, leaf_terms);
+      sweep(e, node.arg[1], fresh("-" + adjoint), counter, lines, leaf_terms);
+      break;
+    case MUL: {
+      const std::string& v1 = e.nodes[node.arg[1]].name;
+      sweep(e, node.arg[0], fresh(adjoint + " * " + v1), counter, lines, leaf_terms);
+      sweep(e, node.arg[1], fresh(adjoint + " * " + v0), counter, lines, leaf_terms);
+      break;
+    }
+    case NEG: sweep(e, node.arg[0], fresh("-" + adjoint), counter, lines, leaf_terms); break;
+    case RELU: sweep(e, node.arg[0], fresh(adjoint + " * mp::relu_slope(" + v0 + ")"), counter, lines, leaf_terms); break;
+    case SELU: sweep(e, node.arg[0], fresh(adjoint + " * mp::selu_slope(" + v0 + ")"), counter, lines, leaf_terms); break;
+    default: break;
+  }
+}
+
+std::string join(const std::vector<std::string>& v, const char* sep) {
+  std::string out;
+  for (size_t i = 0; i < v.size(); ++i) out += (i ? sep : "") + v[i];
+  return out;
+}
+
+const char* storage_type(int dtype) { return dtype == MP_R16 ? "_Float16" : dtype == MP_R32 ? "float" : "double"; }
+
+std::string functor(const char* name, int nin, int nout, const std::string& body) {
+  return std::string("struct ") + name + " {\n  double alpha;\n  template <class P> __device__ __forceinline__ void apply(const P (&in)[" +
+         std::to_string(nin) + "], P (&out)[" + std::to_string(nout) + "]) const {\n" + body + "  }\n};\n\n";
+}
+
+/* The whole source of one (expression, dtype): three functors, nine kernels (each functor in the
+ * three operand layouts of the engine). */
+std::string chain_source(Expr& e, int dtype) {
+  const int k = e.leaves;
+  int counter = 0;
+  std::vector<std::string> fwd;
+  forward_lines(e, e.root, counter, fwd);
+  const std::string value = e.nodes[e.root].name;
+
+  std::vector<std::string> rev(fwd.begin(), fwd.end() - 1); /* no adjoint rule needs the root's own value */
+  std::vector<std::vector<std::string>> leaf_terms(k);
+  counter = 0;
+  sweep(e, e.root, "in[" + std::to_string(k) + "]", counter, rev, leaf_terms);
+
+  std::string fwd_body = join(fwd, "\n") + "\n    out[0] = " + value + ";\n";
+  std::string rev_body = rev.empty() ? "" : join(rev, "\n") + "\n";
+  std::string over = rev_body, blend = "    const P al = (P)alpha;\n" + rev_body;
+  for (int i = 0; i < k; ++i) {
+    const std::string g = join(leaf_terms[i], " + ");
+    over += "    out[" + std::to_string(i) + "] = " + g + ";\n";
+    blend += "    out[" + std::to_string(i) + "] = " + g + " + al * in[" + std::to_string(k + 1 + i) + "];\n";
+  }
+
+  std::string s = "#include \"elementwise.h\"\n\nnamespace {\n\n";
+  s += functor("ChainForward", k, 1, fwd_body);
+  s += functor("ChainReverseOverwrite", k + 1, k, over);
+  s += functor("ChainReverseBlend", 2 * k + 1, k, blend);
+  s += "}  // namespace\n\n";
+  s += std::string("typedef ") + storage_type(dtype) + " ChainT;\n";
+  s += "#define MP_CHAIN_KERNEL(NAME, LAYOUT, NIN, NOUT, F) \\\n"
+       "  extern \"C\" __global__ __launch_bounds__(mp::EW_BLOCK) void NAME(mp::EwPtrs<NIN, NOUT> ptrs, size_t n, unsigned head, F f) { \\\n"
+       "    mp::ew_body<ChainT, mp::PACK_BYTES / (int)sizeof(ChainT), LAYOUT, NIN, NOUT, 1, F>(ptrs, n, head, f); \\\n"
+       "  }\n";
+  const char* layouts[3] = {"mp::EW_ALIGNED", "mp::EW_PEELED", "mp::EW_LOOSE"};
+  const struct { const char* stem; const char* fn; int nin, nout; } kinds[3] = {
+      {"chain_forward", "ChainForward", k, 1},
+      {"chain_reverse_overwrite", "ChainReverseOverwrite", k + 1, k},
+      {"chain_reverse_blend", "ChainReverseBlend", 2 * k + 1, k}};
+  for (const auto& kind : kinds)
+    for (int l = 0; l < 3; ++l)
+      s += std::string("MP_CHAIN_KERNEL(") + kind.stem + "_" + std::to_string(l) + ", " + layouts[l] + ", " +
+           std::to_string(kind.nin) + ", " + std::to_string(kind.nout) + ", " + kind.fn + ")\n";
+  return s;
+}
+
+/* ---------------------------------------------------------------- source -> code object */
+
+bool compile(const std::string& source, std::vector<char>& code, std::string& err) {
+  hiprtcProgram prog;
+  hiprtcResult r = hiprtcCreateProgram(&prog, source.c_str(), "chain.hip", CHAIN_HEADER_COUNT, CHAIN_HEADER_TEXT, CHAIN_HEADER_NAMES);
+  if (r != HIPRTC_SUCCESS) {
+    err = std::string("hiprtcCreateProgram: ") + hiprtcGetErrorString(r);
+    return false;
+  }
+  /* the flags the library's own device objects are built with; packed fp32 arithmetic stays off */
+  const char* options[] = {"--offload-arch=" MP_GPU_ARCH, "-O3", "-std=c++20", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"};
+  r = hiprtcCompileProgram(prog, (int)(sizeof(options) / sizeof(options[0])), options);
+  if (r != HIPRTC_SUCCESS) {
+    size_t n = 0;
+    hiprtcGetProgramLogSize(prog, &n);
+    std::string log(n, '\0');
+    if (n) hiprtcGetProgramLog(prog, log.data());
+    err = std::string("hiprtcCompileProgram: ") + hiprtcGetErrorString(r) + "\n" + log;
+    hiprtcDestroyProgram(&prog);
+    return false;
+  }
+  size_t n = 0;
+  r = hiprtcGetCodeSize(prog, &n);
+  if (r == HIPRTC_SUCCESS) {
+    code.resize(n);
+    r = hiprtcGetCode(prog, code.data());
+  }
+  hiprtcDestroyProgram(&prog);
+  if (r != HIPRTC_SUCCESS) {
+    err = std::string("hiprtcGetCode: ") + hiprtcGetErrorString(r);
+    return false;
+  }
+  return true;
+}
+
+/* ---------------------------------------------------------------- the process-wide cache */
+
+struct Loaded {
+  hipModule_t module = nullptr;
+  hipFunction_t fn[9] = {};
+};
+
+struct Chain {
+  int leaves = 0;
+  std::string source;
+  std::vector<char> code;
+  Loaded on_device[MAX_DEVICES];
+};
+
+std::mutex cache_lock;
+std::map<std::pair<std::string, int>, std::unique_ptr<Chain>> cache; /* entries are never removed */
+
+/* The chain of (signature, dtype): its source on first sight, its code object when `compiled` is
+ * asked for. NULL with last_error set when it cannot be had. A failure is not cached: it is as
+ * cheap to find again as to look up. */
+Chain* chain_for(const char* signature, int dtype, bool compiled) {
+  if (dtype != MP_R16 && dtype != MP_R32 && dtype != MP_R64) {
+    fail("dtype must be 0 (r16), 1 (r32) or 2 (r64)");
+    return nullptr;
+  }
+  /* parsing costs a microsecond; it also gives the text the cache is keyed by */
+  Expr e;
+  std::string err;
+  if (!parse(signature, e, err)) {
+    fail(std::string("chain \"") + (signature ? signature : "") + "\": " + err);
+    return nullptr;
+  }
+  std::string canonical;
+  spell(e, e.root, canonical);
+  std::lock_guard<std::mutex> hold(cache_lock);
+  auto key = std::make_pair(canonical, dtype);
+  auto it = cache.find(key);
+  if (it == cache.end()) {
+    auto c = std::make_unique<Chain>();
+    c->leaves = e.leaves;
+    c->source = chain_source(e, dtype);
+    it = cache.emplace(std::move(key), std::move(c)).first;
+  }
+  Chain* c = it->second.get();
+  if (compiled && c->code.empty()) {
+    std::vector<char> code;
+    if (!compile(c->source, code, err)) {
+      fail(std::string("chain \"") + signature + "\": " + err);
+      return nullptr;
+    }
+    c->code = std::move(code);
+  }
+  return c;
+}
+
+/* The nine kernels of a chain on the current device, loading the code object there on first use. */
+const Loaded* loaded_here(Chain* c) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= MAX_DEVICES) {
+    fail("no current device");
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> hold(cache_lock);
+  Loaded& l = c->on_device[dev];
+  if (l.module != nullptr) return &l;
+  hipModule_t module = nullptr;
+  hipError_t r = hipModuleLoadData(&module, c->code.data());
+  if (r != hipSuccess) {
+    fail(std::string("hipModuleLoadData: ") + hipGetErrorString(r));
+    return nullptr;
+  }
+  const char* stems[3] = {"chain_forward_", "chain_reverse_overwrite_", "chain_reverse_blend_"};
+  for (int k = 0; k < 3; ++k)
+    for (int layout = 0; layout < 3; ++layout) {
+      const std::string name = stems[k] + std::to_string(layout);
+      r = hipModuleGetFunction(&l.fn[k * 3 + layout], module, name.c_str());
+      if (r != hipSuccess) {
+        fail("hipModuleGetFunction(" + name + "): " + hipGetErrorString(r));
+        (void)hipModuleUnload(module);
+        return nullptr;
+      }
+    }
+  l.module = module;
+  return &l;
+}
+
+int layout_index(int layout) { return layout == mp::EW_ALIGNED ? 0 : layout == mp::EW_PEELED ? 1 : 2; }
+
+/* One launch: kind 0 forward, 1 reverse that overwrites, 2 reverse that blends. */
+int enqueue(Chain* c, int kind, int dtype, const void* const* in, int nin, void* const* out, int nout, double alpha,
+            size_t n, hipStream_t stream) {
+  if (n == 0) return 0;
+  for (int s = 0; s < nin; ++s)
+    if (in[s] == nullptr) return fail("a NULL operand");
+  for (int s = 0; s < nout; ++s)
+    if (out[s] == nullptr) return fail("a NULL output");
+  if (n / mp::EW_BLOCK >= 0x7fffffffull) return fail("too many elements for one grid");
+  const Loaded* l = loaded_here(c);
+  if (l == nullptr) return 1;
+  const size_t elem = dtype == MP_R16 ? 2 : dtype == MP_R32 ? 4 : 8;
+  const mp::EwPlan plan = mp::ew_plan(in, nin, out, nout, n, elem, mp::EW_BLOCK, 1);
+  /* the kernel's first parameter is EwPtrs<nin, nout> by value: the inputs, then the outputs */
+  const void* ptrs[2 * MAX_LEAVES + 1 + MAX_LEAVES];
+  for (int s = 0; s < nin; ++s) ptrs[s] = in[s];
+  for (int s = 0; s < nout; ++s) ptrs[nin + s] = out[s];
+  unsigned head = plan.head;
+  void* params[4] = {ptrs, &n, &head, &alpha};
+  const hipError_t r = hipModuleLaunchKernel(l->fn[kind * 3 + layout_index(plan.layout)], plan.blocks, 1, 1, mp::EW_BLOCK, 1, 1,
+                                             0, stream, params, nullptr);
+  if (r != hipSuccess) return fail(std::string("hipModuleLaunchKernel: ") + hipGetErrorString(r));
+  return 0;
+}
+
+}  // namespace
+
+extern "C" int mpChainCompile(const char* signature, int dtype) { return chain_for(signature, dtype, true) ? 0 : 1; }
+
+extern "C" int mpChainLeaves(const char* signature) {
+  Expr e;
+  std::string err;
+  if (!parse(signature, e, err)) {
+    fail(std::string("chain \"") + (signature ? signature : "") + "\": " + err);
+    return -1;
+  }
+  return e.leaves;
+}
+
+extern "C" const char* mpChainSource(const char* signature, int dtype) {
+  Chain* c = chain_for(signature, dtype, false);
+  return c ? c->source.c_str() : nullptr;
+}
+
+extern "C" const void* mpChainCodeObject(const char* signature, int dtype, len_t* bytes) {
+  Chain* c = chain_for(signature, dtype, true);
+  if (bytes) *bytes = c ? (len_t)c->code.size() : 0;
+  return c ? c->code.data() : nullptr;
+}
+
+extern "C" int mpChainForward(const char* signature, int dtype, const void* const* x, void* out, len_t n, StreamContext stream) {
+  Chain* c = chain_for(signature, dtype, true);
+  if (c == nullptr) return 1;
+  void* outs[1] = {out};
+  return enqueue(c, 0, dtype, x, c->leaves, outs, 1, 0.0, (size_t)n, get_stream(stream));
+}
+
+extern "C" int mpChainReverse(const char* signature, int dtype, const void* const* x, const void* out_grads, void* const* g,
+                              double alpha, len_t n, StreamContext stream) {
+  Chain* c = chain_for(signature, dtype, true);
+  if (c == nullptr) return 1;
+  const int k = c->leaves;
+  const void* in[2 * MAX_LEAVES + 1];
+  for (int i = 0; i < k; ++i) in[i] = x[i];
+  in[k] = out_grads;
+  if (alpha == 0.0) return enqueue(c, 1, dtype, in, k + 1, g, k, 0.0, (size_t)n, get_stream(stream));
+  for (int i = 0; i < k; ++i) in[k + 1 + i] = g[i];
+  return enqueue(c, 2, dtype, in, 2 * k + 1, g, k, alpha, (size_t)n, get_stream(stream));
+}
+
+extern "C" len_t mpChainCacheSize(void) {
+  std::lock_guard<std::mutex> hold(cache_lock);
+  len_t n = 0;
+  for (const auto& kv : cache) n += kv.second->code.empty() ? 0 : 1;
+  return n;
+}
+
+extern "C" const char* mpChainError(void) { return last_error.c_str(); }

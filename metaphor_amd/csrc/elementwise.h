@@ -52,7 +52,7 @@ enum EwLayout { EW_ALIGNED, EW_PEELED, EW_LOOSE };
 /* F::apply(const P (&in)[NIN], P (&out)[NOUT]) computes one element. head: the elements before the
  * first pack (EW_PEELED only, less than a cache line of them). */
 template <class T, int W, int LAYOUT, int NIN, int NOUT, int UNROLL, class F>
-__global__ __launch_bounds__(ew_block<NIN>()) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, size_t n, unsigned head_arg, F f) {
+__device__ __forceinline__ void ew_body(const EwPtrs<NIN, NOUT>& ptrs, size_t n, unsigned head_arg, const F& f) {
   using P = typename precision<T>::type;
   constexpr int NA = NIN > 0 ? NIN : 1, EW_BLOCK = ew_block<NIN>();
   constexpr bool LOOSE = LAYOUT == EW_LOOSE;
@@ -111,6 +111,44 @@ __global__ __launch_bounds__(ew_block<NIN>()) void ew_kernel(EwPtrs<NIN, NOUT> p
   }
 }
 
+template <class T, int W, int LAYOUT, int NIN, int NOUT, int UNROLL, class F>
+__global__ __launch_bounds__(ew_block<NIN>()) void ew_kernel(EwPtrs<NIN, NOUT> ptrs, size_t n, unsigned head_arg, F f) {
+  ew_body<T, W, LAYOUT, NIN, NOUT, UNROLL, F>(ptrs, n, head_arg, f);
+}
+
+/* How a launch over n elements is laid out: which kernel variant, how many elements come before
+ * the first pack, how many workgroups. The one place that decides it, for the launchers compiled
+ * into the library and for chains compiled at run time alike. */
+struct EwPlan {
+  int layout;
+  unsigned head;
+  unsigned blocks;
+};
+#ifdef MP_HOST_SIDE
+inline EwPlan ew_plan(const void* const* in, int nin, void* const* out, int nout, size_t n, size_t elem_bytes,
+                      int block_threads, int unroll) {
+  const int W = PACK_BYTES / (int)elem_bytes;
+  /* the place in a cache line that the operands share, or ~0u when they differ */
+  auto in_line = [](const void* p) { return (unsigned)(reinterpret_cast<uintptr_t>(p) & 127u); };
+  unsigned mis = nin > 0 ? in_line(in[0]) : in_line(out[0]);
+  bool packed = true;
+  for (int s = 0; s < nin; ++s) {
+    mis = in_line(in[s]) == mis ? mis : ~0u;
+    packed = packed && aligned16(in[s]);
+  }
+  for (int s = 0; s < nout; ++s) {
+    mis = in_line(out[s]) == mis ? mis : ~0u;
+    packed = packed && aligned16(out[s]);
+  }
+  const bool peel = mis != 0 && mis != ~0u && mis % elem_bytes == 0 && n >= (size_t)(128 / elem_bytes) + W;
+  const unsigned head = peel ? (unsigned)((128 - mis) / elem_bytes) : 0;
+  const size_t npacks = (n - head) / W;
+  const size_t per_block = (size_t)block_threads * unroll;
+  size_t blocks = (npacks + per_block - 1) / per_block;
+  if (blocks == 0) blocks = 1; /* only single elements */
+  return EwPlan{peel ? EW_PEELED : packed ? EW_ALIGNED : EW_LOOSE, head, (unsigned)blocks};
+}
+
 /* Enqueue f over n elements: one pack per stream per lane, laid out as EwLayout says.
  * n == 0 enqueues nothing. */
 template <class T, int NIN, int NOUT, int UNROLL, class F>
@@ -119,31 +157,16 @@ inline void ew_launch(const EwPtrs<NIN, NOUT>& ptrs, size_t n, F f, hipStream_t 
   constexpr int EW_BLOCK = ew_block<NIN>();
   require(n / EW_BLOCK < 0x7fffffffull, "elementwise launch: too many elements for one grid");
   constexpr int W = PACK_BYTES / (int)sizeof(T);
-  /* the place in a cache line that the operands share, or ~0u when they differ */
-  auto in_line = [](const void* p) { return (unsigned)(reinterpret_cast<uintptr_t>(p) & 127u); };
-  unsigned mis = NIN > 0 ? in_line(ptrs.in[0]) : in_line(ptrs.out[0]);
-  bool packed = true;
-  for (int s = 0; s < NIN; ++s) {
-    mis = in_line(ptrs.in[s]) == mis ? mis : ~0u;
-    packed = packed && aligned16(ptrs.in[s]);
-  }
-  for (int s = 0; s < NOUT; ++s) {
-    mis = in_line(ptrs.out[s]) == mis ? mis : ~0u;
-    packed = packed && aligned16(ptrs.out[s]);
-  }
   static_assert(128 / sizeof(T) <= 64, "the first workgroup's threads cover the head");
-  const bool peel = mis != 0 && mis != ~0u && mis % sizeof(T) == 0 && n >= (size_t)(128 / sizeof(T)) + W;
-  const unsigned head = peel ? (unsigned)((128 - mis) / sizeof(T)) : 0;
-  const size_t npacks = (n - head) / W;
-  const size_t per_block = (size_t)EW_BLOCK * UNROLL;
-  size_t blocks = (npacks + per_block - 1) / per_block;
-  if (blocks == 0) blocks = 1; /* only single elements */
-  const dim3 grid((unsigned)blocks), block(EW_BLOCK);
-  if (peel) ew_kernel<T, W, EW_PEELED, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, head, f);
-  else if (packed) ew_kernel<T, W, EW_ALIGNED, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
+  const EwPlan plan = ew_plan(ptrs.in, NIN, ptrs.out, NOUT, n, sizeof(T), EW_BLOCK, UNROLL);
+  const unsigned head = plan.head;
+  const dim3 grid(plan.blocks), block(EW_BLOCK);
+  if (plan.layout == EW_PEELED) ew_kernel<T, W, EW_PEELED, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, head, f);
+  else if (plan.layout == EW_ALIGNED) ew_kernel<T, W, EW_ALIGNED, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
   else ew_kernel<T, W, EW_LOOSE, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
   MP_CHECK_LAUNCH();
 }
+#endif /* MP_HOST_SIDE */
 
 }  // namespace mp
 

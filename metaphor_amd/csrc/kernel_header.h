@@ -26,12 +26,19 @@
 
 #if defined(__cplusplus) && defined(__HIPCC__)
 
+/* A source compiled at run time (hiprtc defines __HIPCC_RTC__ and brings the device runtime with
+ * it) sees the device side of this header only: no library headers exist there, and nothing of
+ * the host side is needed. */
+#ifndef __HIPCC_RTC__
+#define MP_HOST_SIDE 1
 #include <hip/hip_runtime.h>
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
 #include <cstdlib>
+#endif
 
+#ifdef MP_HOST_SIDE
 inline hipStream_t get_stream(StreamContext context) {
   return static_cast<hipStream_t>(context.hip_stream.ptr);
 }
@@ -46,9 +53,11 @@ inline void mpHandleHipError(hipError_t err, const char* file, int line) {
 
 /* a launch that the runtime rejects (bad grid, missing code object) must not pass silently */
 #define MP_CHECK_LAUNCH() HIP_ASSERT(hipGetLastError())
+#endif /* MP_HOST_SIDE */
 
 namespace mp {
 
+#ifdef MP_HOST_SIDE
 /* argument checks of the launchers: same print-and-exit convention as a HIP error */
 inline void require(bool ok, const char* what) {
   if (!ok) {
@@ -56,6 +65,7 @@ inline void require(bool ok, const char* what) {
     exit(EXIT_FAILURE);
   }
 }
+#endif
 
 constexpr int WAVE = MP_WAVE_SIZE;
 constexpr int PACK_BYTES = 16;
@@ -260,8 +270,10 @@ __device__ __forceinline__ void store_cut_pack(T* p, const P (&in)[W], unsigned 
   store_cut_pack_from<T, W, 0, W / 2>(p, in, c);
 }
 
+#ifdef MP_HOST_SIDE
 inline bool aligned16(const void* p) { return (reinterpret_cast<uintptr_t>(p) & 15u) == 0; }
 inline unsigned misalign16(const void* p) { return (unsigned)(reinterpret_cast<uintptr_t>(p) & 15u); }
+#endif
 
 /* ---------------------------------------------------------------------------------------
  * cross-lane reductions (all 64 lanes must be active)
@@ -453,6 +465,7 @@ template <class T, int W, int G, int NV, bool RAGGED> struct RowTile {
  * row-regime selection shared by the softmax and RMSNorm launchers
  * ------------------------------------------------------------------------------------- */
 
+#ifdef MP_HOST_SIDE
 /* Packs a thread must hold so that a G-thread group covers `packs` packs; 0 = too long. */
 inline int packs_per_thread(size_t packs, int G, int max_nv) {
   for (int nv = 1; nv <= max_nv; nv *= 2)
@@ -470,6 +483,7 @@ inline int compute_units() {
   }();
   return cus;
 }
+#endif /* MP_HOST_SIDE */
 
 }  // namespace mp
 

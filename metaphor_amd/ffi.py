@@ -57,7 +57,9 @@ def _open(name):
 _CTYPE = {
     "const void*": ctypes.c_void_p, "void*": ctypes.c_void_p, "void const*": ctypes.c_void_p,
     "double": ctypes.c_double, "len_t": len_t, "StreamContext": StreamContext,
-    "uint32_t": ctypes.c_uint32, "int": ctypes.c_int,
+    "uint32_t": ctypes.c_uint32, "int": ctypes.c_int, "const char*": ctypes.c_char_p,
+    "const void* const*": ctypes.POINTER(ctypes.c_void_p), "void* const*": ctypes.POINTER(ctypes.c_void_p),
+    "len_t*": ctypes.POINTER(len_t),
 }
 _PROTO = re.compile(r"EXTERN_C\s+(\w[\w ]*?\*?)\s*(\w+)\s*\(([^)]*)\)\s*;")
 
@@ -70,6 +72,8 @@ def parse_declarations(path=DECLS):
     for ret, name, params in _PROTO.findall(text):
         args = []
         for p in filter(None, (q.strip() for q in params.split(","))):
+            if p == "void":
+                continue
             m = re.match(r"(.*?)(\w+)?$", p)
             typ = m.group(1).strip() or m.group(2)
             arg = m.group(2) if m.group(1).strip() else ""
@@ -115,6 +119,18 @@ def load():
         _state["device_utils"] = utils
         _state["kernels"] = _DispatchArrays(_open("libmp_kernels.so"))
     return _state["kernels"], _state["device_utils"]
+
+
+def load_fusion():
+    """lib/libmp_fusion.so with the prototypes of include/chain_fusion.h (expressions fused at run time)."""
+    if "fusion" not in _state:
+        lib = _open("libmp_fusion.so")
+        for ret, name, args in parse_declarations(os.path.join(ROOT, "include", "chain_fusion.h")):
+            fn = getattr(lib, name)
+            fn.argtypes = [_CTYPE[t] for t, _ in args]
+            fn.restype = None if ret == "void" else _CTYPE[ret]
+        _state["fusion"] = lib
+    return _state["fusion"]
 
 
 def invoke(kernel_array, key, *args):

@@ -210,6 +210,35 @@ static int fused_chain(mp::Stream stream) {
     dump("plain_sub_da", a.native_grad<float>()); dump("plain_sub_db", b.native_grad<float>());
   }
 
+  /* a graph that fuses whatever it meets: the repeated-input expression above, which no table
+   * lists, is compiled at run time into one kernel per direction; a is ONE leaf whose two
+   * contributions the reverse kernel adds */
+  {
+    mp::Graph* R = mp::Graph::init({stream, mp::Mode::train, mp::Fusion::any});
+    mp::Tensor ra = leaf(R, mp::TensorClass::wgt, {n}, ha), rc = leaf(R, mp::TensorClass::wgt, {n}, hc);
+    mp::Tensor rd = leaf(R, mp::TensorClass::wgt, {n}, hd);
+    size_t l = R->launches;
+    mp::Tensor f2 = mp::ops::selu(mp::ops::hadamard(mp::ops::add(ra, ra), mp::ops::sub(rc, rd)));
+    dump("any_f", f2.native<float>());
+    CHECK(R->launches == l + 1);
+    l = R->launches;
+    f2.reverse(mp::ReverseCleanup::keep);
+    CHECK(R->launches == l + 2); /* the seed fill and one reverse kernel */
+    dump("any_da", ra.native_grad<float>()); dump("any_dc", rc.native_grad<float>()); dump("any_dd", rd.native_grad<float>());
+    /* a second pass accumulates into the existing gradients (alpha = 1) */
+    mp::Tensor f3 = mp::ops::selu(mp::ops::hadamard(mp::ops::add(ra, ra), mp::ops::sub(rc, rd)));
+    f3.reverse(mp::ReverseCleanup::free);
+    dump("any_da2", ra.native_grad<float>());
+    CHECK(R->runtime_chains_.size() == 1);
+    /* a single op stays the op's own kernel and keeps its own reverse */
+    l = R->launches;
+    mp::Tensor s3 = mp::ops::sub(rc, rd);
+    dump("any_sub", s3.native<float>());
+    CHECK(R->launches == l + 1);
+    CHECK(R->runtime_chains_.size() == 1);
+    R->deinit();
+  }
+
   /* eval mode attaches nothing and reverse is refused by construction: only forward here */
   mp::Graph* E = mp::Graph::init({stream, mp::Mode::eval});
   mp::Tensor ea = leaf(E, mp::TensorClass::inp, {n}, ha), eb = leaf(E, mp::TensorClass::inp, {n}, hb);

@@ -108,6 +108,7 @@ Graph* Graph::init(GraphConfig config) {
   Graph* g = new Graph();
   g->stream = config.stream;
   g->mode = config.mode;
+  g->fusion = config.fusion;
   return g;
 }
 
@@ -299,6 +300,7 @@ static void hadamard_reverse(const std::vector<OpDatum>& a);
 static void selu_reverse(const std::vector<OpDatum>& a);
 static void relu_reverse(const std::vector<OpDatum>& a);
 static void chain_reverse(const std::vector<OpDatum>& a);
+static void runtime_chain_reverse(const std::vector<OpDatum>& a);
 
 static const char* pending_name(Pending op) {
   switch (op) {
@@ -367,7 +369,8 @@ void materialise(Tensor t) {
     std::string signature;
     std::vector<Tensor> leaves;
     int budget = 64;
-    const FusedChain* chain = spell(g, t, signature, leaves, budget) ? find_chain(signature) : nullptr;
+    const bool spelled = spell(g, t, signature, leaves, budget);
+    const FusedChain* chain = spelled ? find_chain(signature) : nullptr;
     if (chain) {
       void* x[8];
       for (size_t i = 0; i < leaves.size(); ++i) {
@@ -382,6 +385,31 @@ void materialise(Tensor t) {
         args.push_back(OpDatum((double)(chain - fused_chains)));
         args.push_back(t);
         attach_op(t, chain_reverse, std::move(args));
+      }
+      return;
+    }
+    /* not listed: compiled now if the graph asks for that and the expression has more than one op
+     * (a single op is already one kernel). A refusal (too many leaves, a compile failure) falls
+     * through to one launch per op. */
+    const bool several = signature.find('(') != signature.rfind('(');
+    if (g->fusion == Fusion::any && spelled && several &&
+        mpChainCompile(signature.c_str(), (int)key) == 0) {
+      void* x[8];
+      for (size_t i = 0; i < leaves.size(); ++i) {
+        if (leaves[i].len() == 0) panic("materialise: an input of a pending node was freed");
+        x[i] = leaves[i].data_ptr();
+      }
+      void* out = take_buffer();
+      if (mpChainForward(signature.c_str(), (int)key, x, out, (len_t)n, ctx) != 0) panic(mpChainError());
+      g->launches++;
+      if (g->mode == Mode::train) {
+        size_t idx = 0;
+        while (idx < g->runtime_chains_.size() && g->runtime_chains_[idx] != signature) ++idx;
+        if (idx == g->runtime_chains_.size()) g->runtime_chains_.push_back(signature);
+        std::vector<OpDatum> args(leaves.begin(), leaves.end());
+        args.push_back(OpDatum((double)idx));
+        args.push_back(t);
+        attach_op(t, runtime_chain_reverse, std::move(args));
       }
       return;
     }
@@ -494,6 +522,30 @@ static void chain_reverse(const std::vector<OpDatum>& a) {
     grads[i] = t.grad_ptr();
   }
   chain.reverse(dkey(out), x, out.grad_ptr(), grads, any ? 1.0 : 0.0, (len_t)out.len(), out.context());
+  g->launches++;
+}
+
+/* The same for an expression compiled at run time: args = leaves..., index into the graph's
+ * runtime_chains_, output. */
+static void runtime_chain_reverse(const std::vector<OpDatum>& a) {
+  const size_t k = a.size() - 2;
+  const Tensor out = a[k + 1].t;
+  Graph* g = out.ptr;
+  const std::string& signature = g->runtime_chains_[(size_t)a[k].s];
+  bool any = false;
+  for (size_t i = 0; i < k; ++i) any = any || a[i].t.has_grad();
+  void* x[8];
+  void* grads[8];
+  for (size_t i = 0; i < k; ++i) {
+    const Tensor t = a[i].t;
+    if (any) enable_gradient(t);
+    else t.ptr->grad_of(t) = t.ptr->allocator_.alloc(t.dtype(), t.len(), t.ptr->stream);
+    x[i] = t.data_ptr();
+    grads[i] = t.grad_ptr();
+  }
+  if (mpChainReverse(signature.c_str(), (int)dkey(out), x, out.grad_ptr(), grads, any ? 1.0 : 0.0, (len_t)out.len(),
+                     out.context()) != 0)
+    panic(mpChainError());
   g->launches++;
 }
 

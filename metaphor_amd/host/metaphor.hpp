@@ -23,7 +23,8 @@
  * becomes ONE launch of launch_fused_selu_hadamard_add_add and, in reverse, one launch of its
  * _reverse twin. An expression that is not in the table runs one launch per op exactly as the
  * reference does (src/ops/addition.zig:27-58, src/ops/hadamard.zig:25-56), each of its operands
- * getting the same chance first.
+ * getting the same chance first -- unless the graph was made with Fusion::any, which has such an
+ * expression compiled at run time (mpChainForward / mpChainReverse) and runs it as one kernel too.
  */
 #ifndef MP_HOST_METAPHOR_HPP
 #define MP_HOST_METAPHOR_HPP
@@ -34,6 +35,7 @@
 #include <unordered_map>
 #include <vector>
 
+#include "chain_fusion.h"
 #include "device_utils.h"
 #include "kernel_decls.h"
 
@@ -152,9 +154,17 @@ struct OpInterface {
   bool live = false;
 };
 
+/* Which pending elementwise expressions become one kernel per direction: the ones the build
+ * listed (the generated table of chains.hpp), or any expression, compiled when it is first met
+ * (chain_fusion.h). With `any` the tensors inside an expression never exist, so they have neither
+ * values nor gradients of their own unless somebody asks for their bytes; `listed` keeps every
+ * expression outside the table exactly as the reference runs it, one launch and one tensor per op. */
+enum class Fusion { listed, any };
+
 struct GraphConfig {
   Stream stream = nullptr;
   Mode mode = Mode::train;
+  Fusion fusion = Fusion::listed;
 };
 
 /* Exact-byte-size free-list cache over the stream-ordered allocator
@@ -190,6 +200,9 @@ class Graph {
 
   Mode mode = Mode::train;
   Stream stream = nullptr;
+  Fusion fusion = Fusion::listed;
+  /* expressions this graph had compiled at run time; a reverse entry refers to them by index */
+  std::vector<std::string> runtime_chains_;
 
   /* kernels enqueued through this graph so far (fusion is observable through it) */
   size_t launches = 0;

@@ -267,6 +267,30 @@ class Cfg4(Workload):
         fused_reverse(self.a, self.b, self.c, self.d, self.de, self.da, self.db, self.dc, self.dd, 0.0)
 
 
+class RuntimeChain(Cfg4):
+    """cfg4's size and stream mix (4 reads + 1 write forward, 5 + 4 reverse) for an expression no
+    build listed: relu((a - b) * (c + d)) is compiled by the fusion library on first use."""
+    name = "chain"
+    expr = b"relu(mul(sub(0,1),add(2,3)))"
+
+    def __init__(self, seed=0, n=None):
+        import ctypes
+        super().__init__(seed, n)
+        self._fusion = ffi.load_fusion()
+        self._x = (ctypes.c_void_p * 4)(*[t.data_ptr() for t in (self.a, self.b, self.c, self.d)])
+        self._g = (ctypes.c_void_p * 4)(*[t.data_ptr() for t in (self.da, self.db, self.dc, self.dd)])
+
+    def _check(self, status):
+        if status != 0:
+            raise RuntimeError(self._fusion.mpChainError().decode())
+
+    def forward(self):
+        self._check(self._fusion.mpChainForward(self.expr, ffi.R32, self._x, self.e.data_ptr(), self.n, _ctx()))
+
+    def reverse(self):
+        self._check(self._fusion.mpChainReverse(self.expr, ffi.R32, self._x, self.de.data_ptr(), self._g, 0.0, self.n, _ctx()))
+
+
 class _Vocab(Workload):
     dtype, has_reverse = torch.float32, True  # the configs name the forward; the reverse is measured beside it
 
@@ -374,7 +398,7 @@ class Gemm(Workload):
         inner_product("ji_jk_ik", self.a, self.gc, 1.0, self.gb, 1.0, n, m, k)
 
 
-WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b, Copy, Permutate, Gemm)}
+WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b, Copy, Permutate, Gemm, RuntimeChain)}
 
 DESCRIPTION = {
     "cfg1": "softmax fwd r32 [256,1024]",
@@ -383,6 +407,7 @@ DESCRIPTION = {
     "cfg4": "fused selu((a+b)*(c+d)) fwd+rev r32 flat 2^28",
     "cfg5a": "vocabulary softmax fwd (+rev) r32 [512,151936]",
     "cfg5b": "vocabulary softmax fwd (+rev) r32 [2048,50257]",
+    "chain": "relu((a-b)*(c+d)) fwd+rev r32 flat 2^28, an expression no build listed, compiled at run time",
     "copy": "plain copy r32 flat 2^28 (calibration)",
     "permutate": "transpose r32 [16384,16384], reverse = accumulating transpose",
     "gemm": "matrix product r16 (fp32 accumulate) 8192^3 on rocBLAS, reverse = its two gradient products",

@@ -280,6 +280,27 @@ def fused_reverse(a, b, c, d, de, da, db, dc, dd, alpha=0.0):
           float(alpha), a.numel())
 
 
+def _pointer_array(tensors):
+    import ctypes
+    return (ctypes.c_void_p * len(tensors))(*[t.data_ptr() for t in tensors])
+
+
+def chain_forward(expr, xs, out):
+    """An expression fused at run time: returns the entry point's status (0 = enqueued)."""
+    f = ffi.load_fusion()
+    return f.mpChainForward(expr.encode(), KEY[out.dtype], _pointer_array(xs), out.data_ptr(), out.numel(), ctx())
+
+
+def chain_reverse(expr, xs, out_grads, grads, alpha=0.0):
+    f = ffi.load_fusion()
+    return f.mpChainReverse(expr.encode(), KEY[out_grads.dtype], _pointer_array(xs), out_grads.data_ptr(),
+                            _pointer_array(grads), float(alpha), out_grads.numel(), ctx())
+
+
+def chain_error():
+    return ffi.load_fusion().mpChainError().decode()
+
+
 def matrix_op(stem, src, dst, alpha, m, n):
     """reduce_ij_i, reduce_ij_j, broadcast_i_ij, broadcast_j_ij: (src, dst, alpha, m, n)."""
     _call(stem, src.dtype, src.data_ptr(), dst.data_ptr(), float(alpha), m, n)

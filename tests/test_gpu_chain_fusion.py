@@ -1,0 +1,174 @@
+"""Expressions fused at run time, on the GPU, through the C-ABI of lib/libmp_fusion.so.
+
+Two kinds of evidence. The expressions of chains.json exist twice, compiled into the library at
+build time and compiled by hiprtc at run time from the same functor text and the same engine:
+their results must agree to the rounding of the storage type, at every operand layout, dtype and
+blend (not bit for bit: the two compilations pick fused or separate conversions to r16 differently,
+which moves a result at a rounding tie by one unit in the last place). Expressions nobody listed
+are checked against torch autograd in fp64 on the same (storage-rounded) inputs. Both bounds scale
+with the magnitudes an entry is combined from."""
+import numpy as np
+import pytest
+import torch
+
+import gpu_lib as G
+from metaphor_amd import chaingen
+from test_chain_fusion import random_expression
+from test_chaingen import _torch_eval
+
+pytestmark = pytest.mark.gpu
+
+DTYPES = [torch.float16, torch.float32, torch.float64]
+IDS = ["r16", "r32", "r64"]
+SIZES = [1, 7, 1000, 4099, (1 << 20) + 5]
+LAM, ALP = 1.0507010, 1.6732632
+
+
+def _static(name, dtype, *args):
+    G._call(name, dtype, *args)
+
+
+ULP = {torch.float16: 2.0 ** -10, torch.float32: 2.0 ** -23, torch.float64: 2.0 ** -52}
+
+
+def _same_to_rounding(a, b, scale, dtype, what):
+    """|a - b| <= 2 units in the last place of the terms the entry is combined from."""
+    err = (a.double() - b.double()).abs().cpu().numpy()
+    bound = 2.0 * ULP[dtype] * np.maximum(scale, np.abs(b.double().cpu().numpy()))
+    bad = err > bound
+    exact = float((err == 0).mean()) if err.size else 1.0
+    assert not bad.any(), f"{what}: {int(bad.sum())} entries apart by more than rounding (largest {err.max():.3e})"
+    return exact
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+@pytest.mark.parametrize("chain", chaingen.load_chains(), ids=lambda c: c["name"])
+def test_listed_chains_agree_with_their_build_time_kernels(chain, dtype):
+    expr, name = chain["expr"], chain["name"]
+    root, k = chaingen.parse(expr)
+    r = np.random.default_rng(3)
+    fewest = 1.0
+    for n in SIZES:
+        for shifts in ([0] * (2 * k + 2), [1] * (2 * k + 2), [int(v) for v in r.integers(0, 3, 2 * k + 2)]):
+            for alpha in (0.0, -0.5):
+                G.say(f"chain {name} dtype={dtype} n={n} shifts={shifts} alpha={alpha}")
+                xs = [G.dev(r.uniform(-2, 2, n), dtype, shifts[i]) for i in range(k)]
+                out_a, out_b = G.Guarded((n,), dtype, shifts[k]), G.Guarded((n,), dtype, shifts[k])
+                assert G.chain_forward(expr, [x.t for x in xs], out_a.t) == 0, G.chain_error()
+                _static(name, dtype, *[x.t.data_ptr() for x in xs], out_b.t.data_ptr(), n)
+                up = G.dev(r.normal(0, 1, n), dtype, shifts[k + 1])
+                old = [r.normal(0, 1, n) for _ in range(k)]
+                ga = [G.dev(old[i], dtype, shifts[k + 2 + i]) for i in range(k)]
+                gb = [G.dev(old[i], dtype, shifts[k + 2 + i]) for i in range(k)]
+                hold = [G.host(g.t).astype(np.float64) for g in ga]
+                assert G.chain_reverse(expr, [x.t for x in xs], up.t, [g.t for g in ga], alpha) == 0, G.chain_error()
+                _static(name + "_reverse", dtype, *[x.t.data_ptr() for x in xs], up.t.data_ptr(),
+                        *[g.t.data_ptr() for g in gb], float(alpha), n)
+                vmag, gmag = _magnitudes(root, [G.host(x.t) for x in xs], G.host(up.t))
+                fewest = min(fewest, _same_to_rounding(out_a.t, out_b.t, vmag, dtype, f"{name} value"))
+                for i in range(k):
+                    fewest = min(fewest, _same_to_rounding(ga[i].t, gb[i].t, gmag[i] + abs(alpha) * np.abs(hold[i]), dtype,
+                                                           f"{name} gradient of leaf {i}"))
+                for b in xs + [out_a, out_b, up] + ga + gb:
+                    b.check(name)
+    print(f"[chain-agreement] {name} {dtype}: at least {fewest:.5f} of the entries of every result are bit-identical")
+
+
+def _magnitudes(root, leaves, up):
+    """Upper bounds, entry by entry, of the terms the value and each leaf gradient are combined
+    from: the expression on |leaves| with every op replaced by a bound of its magnitude and slope."""
+    bound_op = {"add": torch.add, "sub": torch.add, "mul": torch.mul, "neg": lambda a: a, "relu": lambda a: a,
+                "selu": lambda a: LAM * ALP * a}
+
+    def ev(n):
+        if n.op == "leaf":
+            return ts[n.leaf]
+        return bound_op[n.op](*[ev(a) for a in n.args])
+
+    ts = [torch.from_numpy(np.abs(x)).double().requires_grad_(True) for x in leaves]
+    v = ev(root)
+    v.backward(torch.from_numpy(np.abs(up)).double())
+    return v.detach().numpy(), [t.grad.numpy() if t.grad is not None else np.zeros_like(up) for t in ts]
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_unlisted_expressions_match_autograd(dtype):
+    r = np.random.default_rng(17)
+    for case in range(12):
+        expr = random_expression(r, int(r.integers(1, 9)), int(r.integers(2, 5)))
+        root, k = chaingen.parse(expr)
+        n = int(r.choice([5, 777, 70001]))
+        shift = int(r.integers(0, 2))
+        alpha = float(r.choice([0.0, 1.0, -0.5]))
+        G.say(f"unlisted chain {expr} dtype={dtype} n={n} shift={shift} alpha={alpha}")
+        xs = [G.dev(r.uniform(-1.5, 1.5, n), dtype, shift) for _ in range(k)]
+        up = G.dev(r.normal(0, 1, n), dtype, shift)
+        old = [G.dev(r.normal(0, 1, n), dtype, shift) for _ in range(k)]
+        hx, hup, hold = [G.host(x.t) for x in xs], G.host(up.t), [G.host(o.t).copy() for o in old]
+        out = G.Guarded((n,), dtype, shift)
+        assert G.chain_forward(expr, [x.t for x in xs], out.t) == 0, G.chain_error()
+        assert G.chain_reverse(expr, [x.t for x in xs], up.t, [o.t for o in old], alpha) == 0, G.chain_error()
+
+        ts = [torch.from_numpy(x.astype(np.float64)).requires_grad_(True) for x in hx]
+        ref = _torch_eval(root, ts)
+        ref.backward(torch.from_numpy(hup.astype(np.float64)))
+        vmag, gmag = _magnitudes(root, hx, hup)
+        G.compare(out.t, ref.detach().numpy(), dtype, f"{expr} value", rowwise=False, scale=vmag)
+        for i in range(k):
+            g = ts[i].grad.numpy() if ts[i].grad is not None else np.zeros(n)
+            want = g + alpha * hold[i].astype(np.float64)
+            G.compare(old[i].t, want, dtype, f"{expr} gradient of leaf {i}", rowwise=False,
+                      scale=gmag[i] + abs(alpha) * np.abs(hold[i].astype(np.float64)))
+        for b in xs + [up, out] + old:
+            b.check(expr)
+
+
+def test_output_may_alias_a_leaf_and_empty_and_null_calls_enqueue_nothing():
+    r = np.random.default_rng(5)
+    f32 = torch.float32
+    expr = "sub(mul(0,1),relu(0))"
+    a, b = G.dev(r.uniform(-2, 2, 5000), f32), G.dev(r.uniform(-2, 2, 5000), f32)
+    ha, hb = G.host(a.t).astype(np.float64), G.host(b.t).astype(np.float64)
+    G.say("chain in place")
+    assert G.chain_forward(expr, [a.t, b.t], a.t) == 0, G.chain_error()
+    G.compare(a.t, ha * hb - np.where(ha >= 0, ha, 0.0), f32, "in place", rowwise=False, scale=np.abs(ha * hb) + np.abs(ha))
+    a.check("in place")
+    before = a.t.clone()
+    empty = a.t[:0]
+    assert G.chain_forward(expr, [empty, empty], empty) == 0
+    f = G.ffi.load_fusion()
+    import ctypes
+    ptrs = (ctypes.c_void_p * 2)(a.t.data_ptr(), None)
+    assert f.mpChainForward(expr.encode(), 1, ptrs, a.t.data_ptr(), 10, G.ctx()) != 0
+    assert "NULL" in G.chain_error()
+    assert G.chain_forward("add(0,frob(1))", [a.t, b.t], a.t) != 0
+    assert "unknown op" in G.chain_error()
+    torch.cuda.synchronize()
+    assert torch.equal(a.t, before)
+
+
+def test_fusion_at_full_rate_of_the_build_time_chain():
+    """2^26 r32 elements: the run-time kernel of the benchmark chain takes the time of the build-time
+    one (same engine, same functor), measured with events around 10 launches each."""
+    n = 1 << 26
+    xs = [torch.empty(n, device="cuda").uniform_(-2, 2) for _ in range(4)]
+    out = torch.empty(n, device="cuda")
+    expr = "selu(mul(add(0,1),add(2,3)))"
+
+    def timed(fn):
+        for _ in range(3):
+            fn()
+        a, b = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        a.record()
+        for _ in range(10):
+            fn()
+        b.record()
+        torch.cuda.synchronize()
+        return a.elapsed_time(b) / 10
+
+    G.say("chain rate")
+    t_run = timed(lambda: G.chain_forward(expr, xs, out))
+    t_build = timed(lambda: G.fused(*xs, out))
+    print(f"[chain-rate] run-time {t_run * 1e3:.1f} us, build-time {t_build * 1e3:.1f} us, "
+          f"{20 * n / t_run / 1e6:.0f} GB/s")
+    assert t_run < 1.1 * t_build + 0.02

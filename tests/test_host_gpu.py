@@ -52,6 +52,18 @@ def test_host_library_end_to_end(tmp_path):
     _cmp(_load(d, "rep_da"), 2.0 * g * v, "host repeated-input da", rowwise=False, rtol=2e-5)
     _cmp(_load(d, "rep_dc"), g * u, "host repeated-input dc", rowwise=False, rtol=2e-5)
 
+    # the same repeated-input shape on a graph that fuses at run time: f = selu((a+a)*(c-d)), one kernel
+    # per direction (host_check asserts the launch counts); da = 2*g*v, dc = g*u, dd = -g*u
+    ua, va = 2.0 * a.astype(np.float64), c.astype(np.float64) - dd.astype(np.float64)
+    wa = ua * va
+    ga_ = O.selu_reverse(wa, np.ones_like(wa))
+    _cmp(_load(d, "any_f"), O.selu(wa), "run-time chain f", rowwise=False, scale=np.abs(wa))
+    _cmp(_load(d, "any_da"), 2.0 * ga_ * va, "run-time chain da", rowwise=False)
+    _cmp(_load(d, "any_dc"), ga_ * ua, "run-time chain dc", rowwise=False)
+    _cmp(_load(d, "any_dd"), -ga_ * ua, "run-time chain dd", rowwise=False)
+    _cmp(_load(d, "any_da2"), 4.0 * ga_ * va, "run-time chain da accumulated twice", rowwise=False)
+    _cmp(_load(d, "any_sub"), va, "single op on a fusing graph", rowwise=False)
+
     # other generated chains (fp64 compositions of the pinned oracle pieces; upstream gradient = 1)
     a64, b64, c64, d64 = (z.astype(np.float64) for z in (a, b, c, dd))
     u, v = a64 + b64, c64 + d64
