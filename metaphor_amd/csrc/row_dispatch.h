@@ -96,14 +96,45 @@ inline RowPlan plan_row(size_t packs, int max_nv, int nv_target, int min_group =
   return RowPlan{0, 0};
 }
 
+/* plan_row, reconsidered for rows that leave more than an eighth of the planned group idle (a row
+ * of 1280 packs on 1024 threads x 2 packs uses five lanes in eight): the group and the packs a
+ * thread, now any number up to max_nv, that waste the fewest lanes; among equals the count
+ * closest to nv_target, then the narrower group. Rows of a power of two of packs keep their plan. */
+inline RowPlan plan_row_fit(size_t packs, int max_nv, int nv_target, int min_group = WAVE) {
+  const RowPlan base = plan_row(packs, max_nv, nv_target, min_group);
+  if (row_regime_override() != REGIME_AUTO || base.G < WAVE || packs == 0) return base;
+  const size_t base_slots = (size_t)base.G * base.NV;
+  if (packs * 8 >= base_slots * 7) return base;
+  static const int ladder[] = {64, 128, 256, 512, 1024};
+  RowPlan best = base;
+  size_t best_slots = base_slots;
+  auto off_target = [&](int nv) { return nv > nv_target ? nv - nv_target : nv_target - nv; };
+  for (int g : ladder)
+    for (int nv = 1; nv <= (max_nv < 8 ? max_nv : 8); ++nv) {
+      const size_t slots = (size_t)g * nv;
+      if (slots < packs) continue;
+      const bool better = slots < best_slots ||
+                          (slots == best_slots && (off_target(nv) < off_target(best.NV) ||
+                                                   (off_target(nv) == off_target(best.NV) && g < best.G)));
+      if (better) {
+        best = RowPlan{g, nv};
+        best_slots = slots;
+      }
+    }
+  return best;
+}
+
 /* Calls f.template operator()<G, NV>() for the plan; returns false for the streaming plan. */
-template <int MAXNV, bool SUBWAVE = false, class F> inline bool for_row_plan(const RowPlan& plan, F&& f) {
+/* ODD: the plan may hold 3, 5, 6 or 7 packs a thread (plan_row_fit); only callers that ask for such plans
+ * pay for the extra kernels. */
+template <int MAXNV, bool SUBWAVE = false, bool ODD = false, class F> inline bool for_row_plan(const RowPlan& plan, F&& f) {
 #define MP_PLAN_CASE(G_, NV_) \
   if constexpr (NV_ <= MAXNV) { \
     if (plan.G == G_ && plan.NV == NV_) { f.template operator()<G_, NV_>(); return true; } \
   }
 #define MP_PLAN_GROUP(G_) \
-  MP_PLAN_CASE(G_, 1) MP_PLAN_CASE(G_, 2) MP_PLAN_CASE(G_, 4) MP_PLAN_CASE(G_, 8) MP_PLAN_CASE(G_, 16)
+  MP_PLAN_CASE(G_, 1) MP_PLAN_CASE(G_, 2) MP_PLAN_CASE(G_, 4) MP_PLAN_CASE(G_, 8) MP_PLAN_CASE(G_, 16) \
+  if constexpr (ODD) { MP_PLAN_CASE(G_, 3) MP_PLAN_CASE(G_, 5) MP_PLAN_CASE(G_, 6) MP_PLAN_CASE(G_, 7) }
   if constexpr (SUBWAVE) {
     MP_PLAN_CASE(8, 1)
     MP_PLAN_GROUP(16)

@@ -1146,8 +1146,13 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
   const bool distinct = !ranges_overlap(dx, x, m * n * sizeof(T)) && !ranges_overlap(dx, dy, m * n * sizeof(T));
   const int C = distinct ? rmsnorm_rev_cluster_size<T>(n) : 0;
   const bool force_shared = C >= 1 && row_regime_override() == REGIME_CLUSTER;
-  const RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row(packs, MAXNV, 1, 8);
-  const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
+  RowPlan plan = force_shared ? RowPlan{0, 0} : plan_row(packs, MAXNV, 1, 8);
+  /* a plan of several packs a thread that idles more than an eighth of its lanes gives way to the
+   * tightest fit (r32 n = 5120: 1024 x 2 -> 512 x 3, 5.46 -> 5.98 TB/s; n = 6144: 5.63 -> 5.98); at
+   * one pack a thread the wide group stays (n = 3072: 1024 x 1 6.00 against 256 x 3 5.85), and the
+   * forward loses by the same change at every length tried (n = 5120: 5.68 -> 5.49) */
+  if (plan.NV >= 2) plan = plan_row_fit(packs, MAXNV, 1, 8);
+  const bool resident = for_row_plan<MAXNV, true, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     /* two register sets of x and dy beside the gain and the dg sums: up to eight registers an array
      * fit the 128 of a 1024-thread workgroup without spills */

@@ -754,6 +754,35 @@ def test_rmsnorm_reverse_cluster_path(dtype, packs, spin):
                 gd.check("rmsnorm rev cluster")
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["r32", "r64"])
+def test_rmsnorm_reverse_rows_held_at_three_packs_a_thread(dtype):
+    """Hidden sizes that are not a power of two: the reverse of the library as shipped holds such a
+    row at three packs a thread in a narrower group instead of idling lanes of a wider one (r32
+    n = 5120, 6144, 10240, 12288; r64 at half those). Whole problem against the oracle, both blends,
+    more rows than one workgroup's share so that the pairing of rows wraps."""
+    r = rng(66)
+    per_pack = 16 // torch.empty((), dtype=dtype).element_size()
+    for packs in (1280, 1536, 2560, 3072):
+        n, m = packs * per_pack, 37
+        for alpha in (0.0, -0.5):
+            G.say(f"rmsnorm rev odd plan dtype={dtype} ({m},{n}) alpha={alpha}")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype)
+            g = G.dev(r.normal(1, 0.02, n), dtype)
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dx = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dg = G.dev(r.normal(0, 1, n), dtype)
+            hdx, hdg = G.host(dx.t).copy(), G.host(dg.t).copy()
+            scratch, _ = G.rmsnorm_scratch(dtype, m, n)
+            G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, 1e-6, alpha)
+            xh, gh, dyh = G.host(x.t), G.host(g.t), G.host(dy.t)
+            rdx, rdg = O.rmsnorm_ij_j_reverse(xh, gh, dyh, 1e-6, hdx if alpha else None, hdg if alpha else None, alpha)
+            sdx, sdg = G.rmsnorm_reverse_scales(xh, gh, dyh, 1e-6, hdx if alpha else None, hdg if alpha else None, alpha)
+            G.compare(dx.t, rdx, dtype, f"rmsnorm rev odd plan dx ({m},{n}) alpha {alpha}", scale=sdx)
+            G.compare(dg.t, rdg, dtype, f"rmsnorm rev odd plan dg ({m},{n}) alpha {alpha}", rowwise=False, scale=sdg)
+            for b in (x, g, dy, dx, dg, scratch):
+                b.check("rmsnorm rev odd plan")
+
+
 def test_rmsnorm_reverse_long_rows_in_place():
     # dx written over dy: the shared-row path must not be taken
     r = rng(63)
