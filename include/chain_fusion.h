@@ -14,7 +14,9 @@
  *
  * The first use of an (expression, dtype) in a process compiles it (about half a second, with
  * hiprtc, no compiler driver needed on the machine); the result is kept until the process ends.
- * Every function is safe to call from several threads.
+ * Every function is safe to call from several threads. Under HIP graph capture a call is one
+ * kernel node, provided the (expression, dtype) has been used on that device before the capture
+ * began: compiling and loading cannot be captured.
  *
  * Errors: these functions return 0 on success and non-zero when nothing was enqueued (text that
  * does not parse, too many leaves, a compile or launch failure); mpChainError() then describes

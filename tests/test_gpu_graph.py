@@ -1,6 +1,6 @@
 """The launchers under HIP graph capture: they enqueue kernels only (no allocation, no memset
 nodes: the shared-row softmax clears its slots with a fill kernel), so a captured sequence can be
-replayed. Every replay is checked against the eager result, with eager work and synchronisation
+replayed; so can an expression fused at run time once its first call has compiled it. Every replay is checked against the eager result, with eager work and synchronisation
 between replays."""
 import numpy as np
 import pytest
@@ -33,7 +33,12 @@ def test_replays_of_a_captured_forward_and_reverse_sequence_match_eager():
     assert fs is not None and rs is not None
     a, b, c, d = (torch.rand(10007, generator=gen, device="cuda", dtype=f32) * 4 - 2 for _ in range(4))
     e = torch.empty_like(a)
-    for t in (x, gain, dy, y, dx, dg, logits, p, dp, dl, a, b, c, d, e):
+    # an expression compiled at run time: its first (eager) call compiles and loads it, which a
+    # capture could not do; after that a call is one kernel launch like any other
+    chain = "relu(mul(sub(0,1),add(2,3)))"
+    e2, up = torch.empty_like(a), rnd(10007)
+    grads = [torch.empty_like(a) for _ in range(4)]
+    for t in (x, gain, dy, y, dx, dg, logits, p, dp, dl, a, b, c, d, e, e2, up, *grads):
         assert t.dtype == f32
 
     def sequence():
@@ -42,8 +47,10 @@ def test_replays_of_a_captured_forward_and_reverse_sequence_match_eager():
         W.softmax_forward(logits, p, fs)
         W.softmax_reverse(p, dp, dl, 0.0, rs)
         W.fused_forward(a, b, c, d, e)
+        assert G.chain_forward(chain, [a, b, c, d], e2) == 0, G.chain_error()
+        assert G.chain_reverse(chain, [a, b, c, d], up, grads, 0.0) == 0, G.chain_error()
 
-    outputs = (y, dx, dg, p, dl, e)
+    outputs = (y, dx, dg, p, dl, e, e2, *grads)
     G.say("eager sequence")
     sequence()
     torch.cuda.synchronize()
