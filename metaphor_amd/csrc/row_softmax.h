@@ -589,9 +589,11 @@ template <class T> inline int cluster_size(size_t packs) {
    * register tile (n = 49152: 5.4 -> 5.7 TB/s) where r32 is better one pack per thread below it */
   const size_t resident = (size_t)CLUSTER_THREADS * 2 - (sizeof(T) >= 4 ? 1 : 0);
   if (regime == REGIME_AUTO && packs <= resident) return 0;
-  /* r32 rows of 32 ... 128 KiB: sixteen packs per thread in a group of 256 or 512 threads beat
-   * the shared row in the forward direction (n = 16384: 5.3 -> 5.7 TB/s, n = 32768: 5.5 -> 5.7) */
-  if (regime == REGIME_AUTO && sizeof(T) == 4 && packs > resident + 1 && packs <= 512 * 16) return 0;
+  /* r32 rows of 32 ... 64 KiB stay with one workgroup of 1024 threads at four packs a thread
+   * (interleaved repeats, 2^28 elements: n = 12288 6.12 TB/s against 5.94 shared, 16384 equal; above,
+   * two workgroups a row win or tie: n = 24576 6.10 against 5.76, 32768 equal; sixteen packs a thread
+   * in 256 or 512 threads, an earlier choice, 5.78 / 5.37 / 5.58 / 5.70) */
+  if (regime == REGIME_AUTO && sizeof(T) == 4 && packs > resident + 1 && packs <= 4096) return 0;
   constexpr size_t tile = (size_t)CLUSTER_THREADS * cluster_nv<T>();
   size_t ppb = (size_t)cluster_tuning().packs_per_block;
   if (ppb == 0) ppb = sizeof(T) == 2 ? tile : tile - CLUSTER_THREADS;
@@ -886,9 +888,7 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   }
   const bool ragged = !(aligned16(x) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(64);
-  RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, 16);
-  if (row_regime_override() == REGIME_AUTO && sizeof(T) == 4 && packs > 2048 && packs <= 512 * 16)
-    plan = RowPlan{packs <= 256 * 16 ? 256 : 512, 16}; /* see cluster_size */
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, 16);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
@@ -972,7 +972,9 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   }
   const bool ragged = !(aligned16(y) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(32);
-  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, 16);
+  /* two packs a thread up to 256 packs a row, one from 512 on (interleaved repeats: r32 n = 2048
+   * 512 x 1 6.25 TB/s against 256 x 2 5.95, r16 n = 4096 6.37 against 6.15, n = 8192 6.40 against 6.27) */
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, packs >= 512 ? 1 : 2, 16);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) {
