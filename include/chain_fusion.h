@@ -7,9 +7,12 @@
  * points are for a host side that defers elementwise ops and wants whatever expression it ends
  * up with as one kernel per direction, also when nobody listed that expression at build time.
  *
- * An expression is text over the ops add, sub, mul (hadamard), neg, relu, selu with its leaves
- * written as 0, 1, ... (or x0, x1, ...) and numbered in order of first appearance; a leaf may
- * appear more than once. Example: "selu(mul(add(0,1),add(2,3)))". At most 8 leaves, 64 nodes.
+ * An expression is text over the ops add, sub, mul (hadamard), neg, relu, selu and, with a literal
+ * constant as second argument, scale (the reference's dilate: x * c) and shift (its translate:
+ * x + c), with its leaves written as 0, 1, ... (or x0, x1, ...) and numbered in order of first
+ * appearance; a leaf may appear more than once. Examples: "selu(mul(add(0,1),add(2,3)))",
+ * "relu(scale(mul(0,1),0.125))". At most 8 leaves, 64 nodes. A constant is part of the expression:
+ * another value is another expression, compiled separately.
  * dtype is MP_R16, MP_R32 or MP_R64 (tensor_types.h).
  *
  * The first use of an (expression, dtype) in a process compiles it (about half a second, with

@@ -1,7 +1,8 @@
 """Fused elementwise chains: from an expression to HIP kernel sources.
 
 ``chains.json`` lists elementwise expressions over leaves ``x0, x1, ...`` built from
-``add, sub, mul, neg, relu, selu``. For every entry this module writes two kernel sources into
+``add, sub, mul, neg, relu, selu`` and, with a literal constant as second argument, ``scale`` (the
+reference's dilate, x * c) and ``shift`` (its translate, x + c). For every entry this module writes two kernel sources into
 ``csrc/hipcc_src`` — ``<name>.hip`` (forward, one pass) and ``<name>_reverse.hip`` (all leaf
 gradients in one pass, obtained by reverse-mode differentiation of the expression tree) — in the
 form the rest of the generator expects: written against ``Scalar``, one launcher per file.
@@ -25,21 +26,31 @@ SRC_DIR = os.path.join(PKG, "csrc", "hipcc_src")
 HOST_DIR = os.path.join(PKG, "host")
 CHAINS = os.path.join(PKG, "chains.json")
 
-ARITY = {"add": 2, "sub": 2, "mul": 2, "neg": 1, "relu": 1, "selu": 1}
+ARITY = {"add": 2, "sub": 2, "mul": 2, "neg": 1, "relu": 1, "selu": 1, "scale": 1, "shift": 1}
+WITH_CONSTANT = ("scale", "shift")  # one tensor argument and one literal: scale(x0,0.5)
 MAX_LEAVES = 8
 
-_TOKEN = re.compile(r"\s*([A-Za-z_]\w*|\(|\)|,)")
+_NUMBER = r"[-+]?(?:\d+\.?\d*|\.\d+)(?:[eE][-+]?\d+)?"
+_TOKEN = re.compile(r"\s*([A-Za-z_]\w*|\(|\)|,|" + _NUMBER + ")")
+
+
+def constant_text(value):
+    """How a constant is spelled in signatures and in generated code: the same in every generator."""
+    return "%.17g" % float(value)
 
 
 class Node:
-    def __init__(self, op, args=(), leaf=None):
-        self.op, self.args, self.leaf = op, list(args), leaf
+    def __init__(self, op, args=(), leaf=None, constant=None):
+        self.op, self.args, self.leaf, self.constant = op, list(args), leaf, constant
 
     def signature(self):
         """Canonical text the host side builds from a pending tree: leaves are bare indices."""
         if self.op == "leaf":
             return str(self.leaf)
-        return f"{self.op}({','.join(a.signature() for a in self.args)})"
+        inner = ",".join(a.signature() for a in self.args)
+        if self.op in WITH_CONSTANT:
+            inner += "," + constant_text(self.constant)
+        return f"{self.op}({inner})"
 
 
 def parse(expr):
@@ -70,8 +81,15 @@ def parse(expr):
         while len(args) < ARITY[tok]:
             take(",")
             args.append(node())
+        constant = None
+        if tok in WITH_CONSTANT:
+            take(",")
+            literal = take()
+            if not re.fullmatch(_NUMBER, literal):
+                raise ValueError(f"{tok} wants a number as second argument, found {literal!r} in {expr!r}")
+            constant = float(literal)
         take(")")
-        return Node(tok, args)
+        return Node(tok, args, constant=constant)
 
     root = node()
     if pos != len(tokens):
@@ -117,6 +135,8 @@ def _forward_lines(root):
             "neg": lambda: f"-{a[0]}",
             "relu": lambda: f"mp::relu_value({a[0]})",
             "selu": lambda: f"mp::selu_value({a[0]})",
+            "scale": lambda: f"{a[0]} * (P)({constant_text(n.constant)})",
+            "shift": lambda: f"{a[0]} + (P)({constant_text(n.constant)})",
         }[n.op]()
         lines.append(f"    const P {name} = {rhs};")
         names[id(n)] = name
@@ -159,6 +179,10 @@ def _reverse_lines(root, k):
             sweep(n.args[0], fresh(f"{a} * mp::relu_slope({v[0]})"))
         elif n.op == "selu":
             sweep(n.args[0], fresh(f"{a} * mp::selu_slope({v[0]})"))
+        elif n.op == "scale":
+            sweep(n.args[0], fresh(f"{a} * (P)({constant_text(n.constant)})"))
+        elif n.op == "shift":
+            sweep(n.args[0], a)
 
     sweep(root, f"in[{k}]")
     grads = [" + ".join(leaf_terms[i]) for i in range(k)]

@@ -1,6 +1,6 @@
 /*
  * Elementwise expressions fused at run time: mpChainForward / mpChainReverse take an expression
- * over add, sub, mul, neg, relu, selu as text, and run it as ONE kernel of the flat elementwise
+ * over add, sub, mul, neg, relu, selu, scale(x, c) and shift(x, c) as text, and run it as ONE kernel of the flat elementwise
  * engine (elementwise.h) and its reverse as ONE kernel that writes every leaf gradient. The first
  * call for an (expression, dtype) writes the three functors (forward, reverse that overwrites,
  * reverse that blends), compiles them with hiprtc against the very headers this library is built
@@ -39,13 +39,14 @@ namespace {
 
 constexpr int MAX_LEAVES = 8, MAX_NODES = 64, MAX_DEVICES = 64;
 
-enum Op { LEAF, ADD, SUB, MUL, NEG, RELU, SELU };
+enum Op { LEAF, ADD, SUB, MUL, NEG, RELU, SELU, SCALE, SHIFT };
 
 struct Node {
   Op op;
   int leaf;    /* LEAF: its number */
   int arg[2];  /* indices into Expr::nodes */
   std::string name; /* the forward value's spelling in the generated code */
+  std::string constant; /* SCALE, SHIFT: the literal, as printf("%.17g") spells it */
 };
 
 struct Expr {
@@ -102,7 +103,7 @@ struct Parser {
         err = "more than 8 leaves";
         return -1;
       }
-      e.nodes.push_back(Node{LEAF, v, {-1, -1}, "in[" + std::to_string(v) + "]"});
+      e.nodes.push_back(Node{LEAF, v, {-1, -1}, "in[" + std::to_string(v) + "]", ""});
       return (int)e.nodes.size() - 1;
     }
     std::string word;
@@ -114,6 +115,8 @@ struct Parser {
     else if (word == "neg") op = NEG;
     else if (word == "relu") op = RELU;
     else if (word == "selu") op = SELU;
+    else if (word == "scale") op = SCALE;
+    else if (word == "shift") op = SHIFT;
     else {
       err = "unknown op \"" + word + "\"";
       return -1;
@@ -126,8 +129,23 @@ struct Parser {
       b = node();
       if (b < 0) return -1;
     }
+    std::string constant;
+    if (op == SCALE || op == SHIFT) { /* a literal second argument: scale(0,0.5) */
+      if (!take(',')) return -1;
+      skip();
+      char* end = nullptr;
+      const double value = strtod(p, &end);
+      if (end == p || !(value == value) || value - value != 0.0) {
+        err = std::string("expected a finite number at \"") + p + "\"";
+        return -1;
+      }
+      p = end;
+      char text[40];
+      snprintf(text, sizeof text, "%.17g", value);
+      constant = text;
+    }
     if (!take(')')) return -1;
-    e.nodes.push_back(Node{op, -1, {a, b}, ""});
+    e.nodes.push_back(Node{op, -1, {a, b}, "", constant});
     return (int)e.nodes.size() - 1;
   }
 };
@@ -158,7 +176,7 @@ bool parse(const char* text, Expr& e, std::string& err) {
 
 /* The expression as the cache spells it: bare leaf numbers, no blanks ("add(x0, x1)" -> "add(0,1)"). */
 void spell(const Expr& e, int n, std::string& out) {
-  static const char* const names[] = {"", "add", "sub", "mul", "neg", "relu", "selu"};
+  static const char* const names[] = {"", "add", "sub", "mul", "neg", "relu", "selu", "scale", "shift"};
   const Node& node = e.nodes[n];
   if (node.op == LEAF) {
     out += std::to_string(node.leaf);
@@ -171,6 +189,7 @@ void spell(const Expr& e, int n, std::string& out) {
     out += ',';
     spell(e, node.arg[1], out);
   }
+  if (!node.constant.empty()) out += "," + node.constant;
   out += ')';
 }
 
@@ -192,6 +211,8 @@ void forward_lines(Expr& e, int n, int& counter, std::vector<std::string>& lines
     case NEG: rhs = "-" + a; break;
     case RELU: rhs = "mp::relu_value(" + a + ")"; break;
     case SELU: rhs = "mp::selu_value(" + a + ")"; break;
+    case SCALE: rhs = a + " * (P)(" + node.constant + ")"; break;
+    case SHIFT: rhs = a + " + (P)(" + node.constant + ")"; break;
     default: break;
   }
   node.name = "t" + std::to_string(counter++);
@@ -229,6 +250,8 @@ void sweep(const Expr& e, int n, const std::string& adjoint, int& counter, std::
     case NEG: sweep(e, node.arg[0], fresh("-" + adjoint), counter, lines, leaf_terms); break;
     case RELU: sweep(e, node.arg[0], fresh(adjoint + " * mp::relu_slope(" + v0 + ")"), counter, lines, leaf_terms); break;
     case SELU: sweep(e, node.arg[0], fresh(adjoint + " * mp::selu_slope(" + v0 + ")"), counter, lines, leaf_terms); break;
+    case SCALE: sweep(e, node.arg[0], fresh(adjoint + " * (P)(" + node.constant + ")"), counter, lines, leaf_terms); break;
+    case SHIFT: sweep(e, node.arg[0], adjoint, counter, lines, leaf_terms); break;
     default: break;
   }
 }

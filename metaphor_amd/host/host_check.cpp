@@ -230,12 +230,24 @@ static int fused_chain(mp::Stream stream) {
     f3.reverse(mp::ReverseCleanup::free);
     dump("any_da2", ra.native_grad<float>());
     CHECK(R->runtime_chains_.size() == 1);
+    /* dilate and translate defer like the other elementwise ops and carry their constants into the
+     * expression: relu(0.125 * (a * c) + 0.5) is one kernel each way */
+    R->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+    l = R->launches;
+    mp::Tensor f4 = mp::ops::relu(mp::ops::translate(mp::ops::dilate(mp::ops::hadamard(ra, rc), 0.125), 0.5));
+    dump("any_affine", f4.native<float>());
+    CHECK(R->launches == l + 1);
+    l = R->launches;
+    f4.reverse(mp::ReverseCleanup::free);
+    CHECK(R->launches == l + 2);
+    dump("any_affine_da", ra.native_grad<float>()); dump("any_affine_dc", rc.native_grad<float>());
+    CHECK(R->runtime_chains_.size() == 2);
     /* a single op stays the op's own kernel and keeps its own reverse */
     l = R->launches;
     mp::Tensor s3 = mp::ops::sub(rc, rd);
     dump("any_sub", s3.native<float>());
     CHECK(R->launches == l + 1);
-    CHECK(R->runtime_chains_.size() == 1);
+    CHECK(R->runtime_chains_.size() == 2);
     R->deinit();
   }
 

@@ -283,8 +283,9 @@ bool is_pending(Tensor t) {
 }
 
 /* A pending node owns no bytes yet: its buffer is taken from the allocator when it is computed. */
-Tensor defer(Graph* g, Pending op, Tensor x, Tensor y) {
+Tensor defer(Graph* g, Pending op, Tensor x, Tensor y, double value) {
   Graph::Node node;
+  node.value = value;
   node.data = TensorData{nullptr, x.len(), x.dtype()};
   node.sizes = x.sizes();
   node.pending = op;
@@ -299,6 +300,8 @@ static void subtraction_reverse(const std::vector<OpDatum>& a);
 static void hadamard_reverse(const std::vector<OpDatum>& a);
 static void selu_reverse(const std::vector<OpDatum>& a);
 static void relu_reverse(const std::vector<OpDatum>& a);
+static void translate_reverse(const std::vector<OpDatum>& a);
+static void dilate_reverse(const std::vector<OpDatum>& a);
 static void chain_reverse(const std::vector<OpDatum>& a);
 static void runtime_chain_reverse(const std::vector<OpDatum>& a);
 
@@ -309,6 +312,8 @@ static const char* pending_name(Pending op) {
     case Pending::hadamard: return "mul";
     case Pending::selu: return "selu";
     case Pending::relu: return "relu";
+    case Pending::dilate: return "scale";
+    case Pending::translate: return "shift";
     default: return "?";
   }
 }
@@ -323,7 +328,11 @@ static bool spell(Graph* g, Tensor t, std::string& out, std::vector<Tensor>& lea
     out += pending_name(node.pending);
     out += '(';
     if (!spell(g, node.in0, out, leaves, budget)) return false;
-    if (node.pending != Pending::selu && node.pending != Pending::relu) {
+    if (node.pending == Pending::dilate || node.pending == Pending::translate) {
+      char text[40]; /* the constant as every generator of chains spells it */
+      snprintf(text, sizeof text, ",%.17g", node.value);
+      out += text;
+    } else if (node.pending != Pending::selu && node.pending != Pending::relu) {
       out += ',';
       if (!spell(g, node.in1, out, leaves, budget)) return false;
     }
@@ -351,6 +360,7 @@ void materialise(Tensor t) {
   Graph* g = t.ptr;
   const Pending op = g->nodes_[t.idx].pending;
   const Tensor in0 = g->nodes_[t.idx].in0, in1 = g->nodes_[t.idx].in1;
+  const double value = g->nodes_[t.idx].value;
   const size_t n = g->nodes_[t.idx].data.len;
   const Tag dt = g->nodes_[t.idx].data.dtype;
   const size_t key = (size_t)dt;
@@ -416,8 +426,17 @@ void materialise(Tensor t) {
   }
 
   /* anything else: one launch per op, as the reference's forward_impl does */
-  if (in0.len() == 0 || in1.len() == 0) panic("materialise: an input of a pending node was freed");
+  const bool with_constant = op == Pending::dilate || op == Pending::translate;
+  if (in0.len() == 0 || (!with_constant && in1.len() == 0)) panic("materialise: an input of a pending node was freed");
   void* p0 = in0.data_ptr();
+  if (with_constant) { /* src/ops/dilate.zig, src/ops/translate.zig */
+    void* pz = take_buffer();
+    if (op == Pending::dilate) kernels::dilate(key, p0, value, pz, (len_t)n, ctx);
+    else kernels::translate(key, p0, value, pz, (len_t)n, ctx);
+    g->launches++;
+    if (g->mode == Mode::train) attach_op(t, op == Pending::dilate ? dilate_reverse : translate_reverse, {in0, value, t});
+    return;
+  }
   if (op == Pending::selu || op == Pending::relu) {
     void* pz = take_buffer();
     if (op == Pending::selu) kernels::selu(key, p0, pz, (len_t)n, ctx);
@@ -757,25 +776,9 @@ Tensor rmsnorm(Tensor x, Tensor gain, double eps) {
   return z;
 }
 
-Tensor translate(Tensor x, double value) {
-  Graph* g = x.ptr;
-  void* px = x.data_ptr();
-  Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
-  kernels::translate(dkey(z), px, value, z.data_ptr(), (len_t)z.len(), z.context());
-  g->launches++;
-  if (g->mode == Mode::train) attach_op(z, translate_reverse, {x, value, z});
-  return z;
-}
+Tensor translate(Tensor x, double value) { return defer(x.ptr, Pending::translate, x, x, value); }
 
-Tensor dilate(Tensor x, double value) {
-  Graph* g = x.ptr;
-  void* px = x.data_ptr();
-  Tensor z = g->tensor(TensorClass::hid, x.dtype(), x.sizes());
-  kernels::dilate(dkey(z), px, value, z.data_ptr(), (len_t)z.len(), z.context());
-  g->launches++;
-  if (g->mode == Mode::train) attach_op(z, dilate_reverse, {x, value, z});
-  return z;
-}
+Tensor dilate(Tensor x, double value) { return defer(x.ptr, Pending::dilate, x, x, value); }
 
 Tensor reduce(Tensor x, const char* expr) {
   const std::string e = expr;

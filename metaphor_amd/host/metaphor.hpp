@@ -15,7 +15,8 @@
  * Errors follow the reference: an impossible request panics (prints and aborts), nothing returns
  * a status.
  *
- * What is new here is where the kernels come from. add / sub / hadamard / selu / relu do not launch:
+ * What is new here is where the kernels come from. add / sub / hadamard / selu / relu / dilate /
+ * translate do not launch:
  * they record a pending node. A pending node is materialised when something needs its bytes (a
  * non-elementwise op, data_ptr(), native(), reverse()). At that point the recorded expression is
  * written out with its leaves numbered in order of first appearance and looked up in the table
@@ -179,10 +180,10 @@ class TensorAllocator {
   std::unordered_map<size_t, std::vector<void*>> cache_;
 };
 
-enum class Pending : int { none = 0, add, sub, hadamard, selu, relu };
+enum class Pending : int { none = 0, add, sub, hadamard, selu, relu, dilate, translate };
 
-/* deferred elementwise nodes: record, query, compute */
-Tensor defer(Graph* g, Pending op, Tensor x, Tensor y);
+/* deferred elementwise nodes: record, query, compute; value is the constant of dilate / translate */
+Tensor defer(Graph* g, Pending op, Tensor x, Tensor y, double value = 0.0);
 bool is_pending(Tensor t);
 void materialise(Tensor t);
 
@@ -230,6 +231,7 @@ class Graph {
     bool attached = true;
     Pending pending = Pending::none; /* recorded, not yet computed */
     Tensor in0{}, in1{};
+    double value = 0.0; /* dilate, translate: the constant */
   };
   std::vector<Leaf> leaves_;
   std::vector<Node> nodes_;

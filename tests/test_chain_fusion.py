@@ -14,6 +14,7 @@ from test_chaingen import _run_lines, _torch_eval
 torch.set_default_dtype(torch.float64)
 
 EXTRA = ["mul(add(x0,x0),x1)", "relu(sub(mul(x0,x1),neg(x0)))", "selu(selu(add(x0,x1)))", "neg(x0)",
+         "selu(scale(mul(shift(x0,-1.5),x1),0.1))", "shift(scale(x0,3),2.5e-1)",
          "sub(mul(x0,x1),mul(x2,add(x3,add(x4,add(x5,add(x6,x7))))))"]
 
 
@@ -38,9 +39,11 @@ def random_expression(r, leaves, depth):
     def node(d):
         if d == 0 or (d < depth and r.random() < 0.25):
             return leaf()
-        op = str(r.choice(["add", "sub", "mul", "neg", "relu", "selu"]))
+        op = str(r.choice(["add", "sub", "mul", "neg", "relu", "selu", "scale", "shift"]))
         if op in ("neg", "relu", "selu"):
             return f"{op}({node(d - 1)})"
+        if op in ("scale", "shift"):
+            return f"{op}({node(d - 1)},{float(r.choice([0.5, -1.25, 3.0, 0.1, 1e-3])):.17g})"
         return f"{op}({node(d - 1)},{node(d - 1)})"
 
     text = node(depth)
@@ -112,7 +115,8 @@ def test_every_dtype_compiles_and_is_cached_once(dtype):
     ("0", "bare leaf"), ("add(0)", "expected ','"), ("add(0,1,2)", "expected ')'"), ("foo(0)", "unknown op"),
     ("add(1,0)", "order of first appearance"), ("add(0,2)", "order of first appearance"),
     ("add(0,1))", "trailing text"), ("add(0 1)", "expected ','"), ("", "unknown op"),
-    ("add(add(add(add(0,1),add(2,3)),add(add(4,5),add(6,7))),8)", "more than 8 leaves")])
+    ("add(add(add(add(0,1),add(2,3)),add(add(4,5),add(6,7))),8)", "more than 8 leaves"),
+    ("scale(0)", "expected ','"), ("scale(0,x1)", "finite number"), ("shift(0,abc)", "finite number"), ("scale(0,inf)", "finite number")])
 def test_bad_expressions_are_refused_with_a_reason(bad, why):
     lib = ffi.load_fusion()
     n = lib.mpChainCacheSize()

@@ -31,7 +31,12 @@ TORCH_OP = {"add": torch.add, "sub": torch.sub, "mul": torch.mul, "neg": torch.n
 def _torch_eval(node, leaves):
     if node.op == "leaf":
         return leaves[node.leaf]
-    return TORCH_OP[node.op](*[_torch_eval(a, leaves) for a in node.args])
+    args = [_torch_eval(a, leaves) for a in node.args]
+    if node.op == "scale":
+        return args[0] * node.constant
+    if node.op == "shift":
+        return args[0] + node.constant
+    return TORCH_OP[node.op](*args)
 
 
 class _MP:
@@ -45,14 +50,15 @@ class _MP:
 def _run_lines(lines, inputs):
     env = {"inp": inputs, "mp": _MP}
     for line in lines:
-        stmt = line.strip().rstrip(";").replace("const P ", "").replace("mp::", "mp.")
+        stmt = line.strip().rstrip(";").replace("const P ", "").replace("mp::", "mp.").replace("(P)(", "(")
         stmt = re.sub(r"\bin\[", "inp[", stmt)
         exec(stmt, {}, env)
     return env
 
 
 @pytest.mark.parametrize("expr", [c["expr"] for c in chaingen.load_chains()] + [
-    "mul(add(x0,x0),x1)", "relu(sub(mul(x0,x1),neg(x0)))", "selu(selu(add(x0,x1)))"])
+    "mul(add(x0,x0),x1)", "relu(sub(mul(x0,x1),neg(x0)))", "selu(selu(add(x0,x1)))",
+    "selu(scale(mul(shift(x0,-1.5),x1),0.1))", "shift(scale(x0,3),2.5e-1)"])
 def test_generated_arithmetic_matches_autograd(expr):
     root, k = chaingen.parse(expr)
     rng = np.random.default_rng(5)
@@ -81,10 +87,12 @@ def test_signatures_number_leaves_in_order_of_first_appearance():
     assert (root.signature(), k) == ("selu(mul(add(0,1),add(2,3)))", 4)
     root, k = chaingen.parse("mul(add(x0,x0),x1)")
     assert (root.signature(), k) == ("mul(add(0,0),1)", 2)
+    root, k = chaingen.parse("selu(scale(mul(shift(x0, -1.5), x1), 0.1))")
+    assert (root.signature(), k) == ("selu(scale(mul(shift(0,-1.5),1),0.10000000000000001))", 2)
 
 
 @pytest.mark.parametrize("bad", ["x0", "add(x0)", "add(x0,x1,x2)", "foo(x0)", "add(x1,x0)", "add(x0,x2)",
-                                 "add(x0,x1))", "add(x0 x1)"])
+                                 "add(x0,x1))", "add(x0 x1)", "scale(x0)", "scale(x0,x1)", "shift(x0,1,2)", "add(x0,0.5)"])
 def test_bad_expressions_are_rejected(bad):
     with pytest.raises(ValueError):
         chaingen.parse(bad)

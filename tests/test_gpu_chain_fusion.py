@@ -83,6 +83,10 @@ def _magnitudes(root, leaves, up):
     def ev(n):
         if n.op == "leaf":
             return ts[n.leaf]
+        if n.op == "scale":
+            return ev(n.args[0]) * abs(n.constant)
+        if n.op == "shift":
+            return ev(n.args[0]) + abs(n.constant)
         return bound_op[n.op](*[ev(a) for a in n.args])
 
     ts = [torch.from_numpy(np.abs(x)).double().requires_grad_(True) for x in leaves]

@@ -63,6 +63,13 @@ def test_host_library_end_to_end(tmp_path):
     _cmp(_load(d, "any_dd"), -ga_ * ua, "run-time chain dd", rowwise=False)
     _cmp(_load(d, "any_da2"), 4.0 * ga_ * va, "run-time chain da accumulated twice", rowwise=False)
     _cmp(_load(d, "any_sub"), va, "single op on a fusing graph", rowwise=False)
+    # relu(0.125 * (a * c) + 0.5) with its constants inside the kernel; upstream gradient = 1
+    a64_, c64_ = a.astype(np.float64), c.astype(np.float64)
+    pre = 0.125 * (a64_ * c64_) + 0.5
+    on = (pre >= 0).astype(np.float64)
+    _cmp(_load(d, "any_affine"), np.where(pre >= 0, pre, 0.0), "run-time chain with constants", rowwise=False)
+    _cmp(_load(d, "any_affine_da"), on * 0.125 * c64_, "run-time chain with constants da", rowwise=False)
+    _cmp(_load(d, "any_affine_dc"), on * 0.125 * a64_, "run-time chain with constants dc", rowwise=False)
 
     # other generated chains (fp64 compositions of the pinned oracle pieces; upstream gradient = 1)
     a64, b64, c64, d64 = (z.astype(np.float64) for z in (a, b, c, dd))
