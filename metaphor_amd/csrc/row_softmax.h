@@ -479,13 +479,17 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
 #pragma unroll
       for (int i = 0; i < W; ++i) mx = (P)v[k][i] > mx ? (P)v[k][i] : mx;
   }
-  mx = group_allreduce<MaxOP, G>(mx, red[0], lane);
+  /* one exchange inside the workgroup for both reductions: every wavefront shifts by its own
+   * maximum, and the (max, sum) pairs of the sixteen wavefronts meet behind one barrier (against a
+   * barrier for the maximum and one for the sum: [512, 151936] 111.1 -> 109.7 us, [2048, 50257]
+   * 146.9 -> 144.4, launcher times of interleaved repeats) */
+  const P base_mx = wave_allreduce<MaxOP>(mx);
   if constexpr (RAW) {
 #pragma unroll
     for (int k = 0; k < NV; ++k) forget(v[k]);
   }
   /* a chunk without a finite entry (fully masked) contributes exact zeros, not exp(-inf + inf) */
-  const P sh = shift_of(mx > neg_inf<P>() ? mx : (P)0);
+  const P sh = shift_of(base_mx > neg_inf<P>() ? base_mx : (P)0);
   P s = (P)0;
 #pragma unroll
   for (int k = 0; k < NV; ++k)
@@ -502,8 +506,18 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
   const P edge_x = edge;
   edge = exp_shifted(edge, sh);
   s += edge;
-  s = group_allreduce<AddOP, G>(s, red[1], lane);
-
+  s = wave_allreduce<AddOP>(s);
+  if ((lane & (WAVE - 1)) == 0) {
+    red[0][lane / WAVE] = base_mx;
+    red[1][lane / WAVE] = s;
+  }
+  __syncthreads();
+  {
+    constexpr int NW = G / WAVE;
+    const P wm = red[0][lane & (NW - 1)], ws = red[1][lane & (NW - 1)];
+    mx = fold_partials<MaxOP, NW>(wm); /* the chunk's maximum and, relative to it, its sum */
+    s = fold_partials<AddOP, NW>(wm > neg_inf<P>() ? ws * exp_shifted(wm, shift_of(mx)) : (P)0);
+  }
   P M = mx, S = s;
   if (C > 1) {
     Word* mine = slots + ((size_t)row * C + rank) * 2;
@@ -551,7 +565,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
     }
   }
 
-  const P scale = exp_shifted(mx, shift_of(M)) / S;
+  const P scale = exp_shifted(base_mx, shift_of(M)) / S;
   T* ybody = yr + g.head;
   if constexpr (RAW) {
     const P shM = shift_of(M), inv = (P)1 / S;
