@@ -24,13 +24,24 @@ KEY = {torch.float16: ffi.R16, torch.float32: ffi.R32, torch.float64: ffi.R64}
 DTYPE_NAME = {torch.float16: "r16", torch.float32: "r32", torch.float64: "r64"}
 
 
+_contexts = {}   # stream handle -> StreamContext (a launch-bound workload pays for every object it makes)
+_launchers = {}  # (stem, dtype) -> the C function
+
+
 def _ctx():
-    return ffi.StreamContext.from_handle(torch.cuda.current_stream().cuda_stream)
+    handle = torch.cuda.current_stream().cuda_stream
+    ctx = _contexts.get(handle)
+    if ctx is None:
+        ctx = _contexts[handle] = ffi.StreamContext.from_handle(handle)
+    return ctx
 
 
 def _launch(stem, dtype, *args):
-    kernels, _ = ffi.load()
-    ffi.invoke(getattr(kernels, stem), KEY[dtype], *args, _ctx())
+    fn = _launchers.get((stem, dtype))
+    if fn is None:
+        kernels, _ = ffi.load()
+        fn = _launchers[(stem, dtype)] = getattr(kernels, stem)[KEY[dtype]]
+    fn(*args, _ctx())
 
 
 _blas_contexts = {}
