@@ -902,8 +902,15 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   }
   const bool ragged = !(aligned16(x) && (n % W) == 0);
   constexpr int MAXNV = max_nv_for<T>(64);
-  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, 16);
-  const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
+  RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, 2, 16);
+  /* r16 rows that leave a 1024-thread group at two packs a thread more than an eighth idle take
+   * the tightest fit instead (n = 10240: 1024 x 2 -> 256 x 5, 5.44 -> 5.88 TB/s; n = 12288: 512 x 3,
+   * 5.68 -> 6.13; interleaved repeats). Everywhere else the wide group with idle lanes is the
+   * faster one: the same change loses 1-6 % on r32 rows, on r16 rows planned at other shapes and in
+   * the reverse. */
+  constexpr bool FIT = sizeof(T) == 2;
+  if (FIT && plan.G == 1024 && plan.NV == 2) plan = plan_row_fit(packs, MAXNV < 8 ? MAXNV : 8, 2, 16);
+  const bool resident = for_row_plan<MAXNV, true, FIT>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
     else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));

@@ -458,6 +458,25 @@ def test_shared_rows_starting_at_every_offset_from_a_128_byte_line(dtype):
             b.check("line offsets")
 
 
+def test_softmax_forward_r16_rows_held_at_three_or_five_packs_a_thread():
+    """r16 rows of 1152 ... 1792 packs leave a 1024-thread group at two packs a thread partly idle and
+    are held at 3, 5 or 7 packs a thread in a narrower group instead (n = 10240, 12288, 9232 with a
+    ragged end, and one element off alignment); masked and plain rows against the oracle."""
+    r = rng(36)
+    dtype = torch.float16
+    for (m, n, shift) in [(9, 10240, 0), (9, 12288, 0), (5, 9232, 0), (5, 12290, 1), (3, 14000, 0)]:
+        for masked in (False, True):
+            G.say(f"softmax r16 odd plan ({m},{n}) shift={shift} masked={masked}")
+            x = G.dev(_softmax_inputs(r, m, n, dtype, masked), dtype, shift)
+            y = G.Guarded((m, n), dtype, shift)
+            G.softmax(x.t, y.t)
+            G.compare(y.t, O.softmax_ij_j(G.host(x.t)), dtype, f"softmax r16 odd plan ({m},{n})", **G.softmax_tol(dtype))
+            if masked:
+                assert bool((y.t[torch.isinf(x.t)] == 0).all())
+            x.check("x")
+            y.check("y")
+
+
 def test_softmax_long_rows_without_scratch_take_the_two_pass_kernel():
     r = rng(33)
     for (m, n) in [(3, 151936), (4, 50257)]:
