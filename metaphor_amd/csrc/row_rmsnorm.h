@@ -570,6 +570,135 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
   }
 }
 
+/* The paired reverse for rows that a power of two of wavefronts would leave partly idle: a row is
+ * held by `gw` wavefronts (any number from 1 to 16, chosen by the launcher as the fewest that cover
+ * the row at NV packs a thread) and a workgroup is as many such groups as fit 1024 threads, so
+ * every lane but the last wavefront's tail holds data (n = 5120 r16: 640 packs on ten wavefronts,
+ * not on sixteen). The group's width is a kernel argument, not a template parameter: one kernel
+ * per (type, packs a thread, blend) serves every width. Sums of a group fold over sixteen slots of
+ * which the ones past gw read as zero. */
+constexpr int ANY_MAX_ROWS = 4; /* groups per workgroup the LDS below is sized for: widths from 4 wavefronts */
+
+template <class T, int W, int NV, bool BLEND>
+__global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
+    const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
+    typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n, int gw) {
+  using P = typename precision<T>::type;
+  using V = typename vec_of<T, W>::type;
+  constexpr int NW = NORM_BLOCK / WAVE;
+  __shared__ P slots[2][2][ANY_MAX_ROWS][NW];
+  __shared__ P comb[NORM_BLOCK * NV * W];
+
+  const int G = gw * WAVE, RPB = (int)blockDim.x / G;
+  const int sub = threadIdx.x / G, lane = threadIdx.x % G;
+  const int npk = (int)(n / W);
+  const size_t last = m - 1, stride = (size_t)gridDim.x * RPB;
+
+  P gv[NV][W], acc[NV][W];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
+#pragma unroll
+    for (int i = 0; i < W; ++i) acc[k][i] = gv[k][i] = (P)0;
+    if (p < npk) load_pack<T, W>(gain + (size_t)p * W, gv[k]);
+  }
+
+  auto fetch = [&](V (&xs)[NV], V (&ds)[NV], size_t base) {
+    size_t row = base + sub;
+    row = row < last ? row : last;
+    const T* xr = x + row * n;
+    const T* dr = dy + row * n;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      const size_t at = (size_t)(p < npk ? p : 0) * W;
+      xs[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(xr + at));
+      ds[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(dr + at));
+    }
+  };
+  auto finish = [&](const V (&xs)[NV], const V (&ds)[NV], size_t base, P (*sl)[ANY_MAX_ROWS][NW]) {
+    const size_t row = base + sub;
+    const bool live = row < m;
+    P xv[NV][W], dv[NV][W];
+    P ss = (P)0, c = (P)0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const bool inside = k * G + lane < npk;
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        xv[k][i] = inside ? (P)xs[k][i] : (P)0;
+        dv[k][i] = inside ? (P)ds[k][i] : (P)0;
+        ss += xv[k][i] * xv[k][i];
+        c += dv[k][i] * gv[k][i] * xv[k][i];
+      }
+    }
+    ss = wave_allreduce<AddOP>(ss);
+    c = wave_allreduce<AddOP>(c);
+    if ((lane & (WAVE - 1)) == 0) {
+      sl[0][sub][lane / WAVE] = ss;
+      sl[1][sub][lane / WAVE] = c;
+    }
+    lds_barrier();
+    const int slot = lane & (NW - 1);
+    ss = fold_partials<AddOP, NW>(slot < gw ? sl[0][sub][slot] : (P)0);
+    c = fold_partials<AddOP, NW>(slot < gw ? sl[1][sub][slot] : (P)0);
+    const P r = rsqrt_of(ss / (P)n + eps);
+    const P cc = c / (P)n * r * r;
+    if (live) {
+      T* out_row = dx + row * n;
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        const int p = k * G + lane;
+        if (p < npk) {
+          P out[W];
+#pragma unroll
+          for (int i = 0; i < W; ++i) {
+            out[i] = r * (dv[k][i] * gv[k][i] - xv[k][i] * cc);
+            acc[k][i] += dv[k][i] * xv[k][i] * r;
+          }
+          if constexpr (BLEND) {
+            P old[W];
+            load_pack<T, W>(out_row + (size_t)p * W, old);
+#pragma unroll
+            for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+          }
+          store_pack_nt<T, W>(out_row + (size_t)p * W, out);
+        }
+      }
+    }
+  };
+
+  V ax[NV], ad[NV], bx[NV], bd[NV];
+  size_t base = (size_t)blockIdx.x * RPB;
+  fetch(ax, ad, base);
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) settle(gv[k][i]);
+  for (; base < m; base += 2 * stride) {
+    fetch(bx, bd, base + stride);
+    __builtin_amdgcn_sched_barrier(0);
+    finish(ax, ad, base, slots[0]);
+    fetch(ax, ad, base + 2 * stride);
+    __builtin_amdgcn_sched_barrier(0);
+    finish(bx, bd, base + stride, slots[1]);
+  }
+
+  /* one partial row per workgroup: the groups' sums meet in LDS */
+  const int row_slots = G * NV * W;
+#pragma unroll
+  for (int k = 0; k < NV; ++k)
+#pragma unroll
+    for (int i = 0; i < W; ++i) comb[sub * row_slots + (k * G + lane) * W + i] = acc[k][i];
+  __syncthreads();
+  P* mine = partials + (size_t)blockIdx.x * n;
+  for (size_t col = threadIdx.x; col < n; col += blockDim.x) {
+    P t = (P)0;
+    for (int s2 = 0; s2 < RPB; ++s2) t += comb[s2 * row_slots + col];
+    mine[col] = t;
+  }
+}
+
 /* ------------------------------------------------------------------ streaming reverse */
 
 /* Rows too long to keep x and dy in registers: they are read twice (the second read mostly from
@@ -1160,6 +1289,23 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
     /* two register sets of x and dy beside the gain and the dg sums: up to eight registers an array
      * fit the 128 of a 1024-thread workgroup without spills */
     constexpr bool pairs_fit = NV * W * (int)(sizeof(P) / 4) <= 8;
+    /* rows of 257 ... 447 packs leave a 512-thread group more than an eighth idle and two such groups
+     * a workgroup: five or six wavefronts a row and three or two rows a workgroup instead (interleaved
+     * repeats: r16 n = 2560 4.30 -> 5.43 TB/s, 3072 5.03 -> 5.48; r32 n = 1280 5.09 -> 5.50, 1536 5.40 ->
+     * 5.95). Wider rows gain nothing from shedding their idle wavefronts (n = 5120 r16: 4.80 -> 4.87,
+     * with two such workgroups a CU 4.73) and keep the power-of-two groups. */
+    if constexpr (!LOOSE && G == 512 && NV == 1 && pairs_fit) {
+      const int gw = (int)((packs + WAVE - 1) / WAVE);
+      if (row_regime_override() == REGIME_AUTO && packs * 8 < (size_t)G * 7 && gw >= NORM_BLOCK / WAVE / ANY_MAX_ROWS) {
+        const int rpb = NORM_BLOCK / (gw * WAVE);
+        const size_t need_any = (m + rpb - 1) / rpb, one_per_cu = (size_t)compute_units();
+        rows = (unsigned)(need_any < one_per_cu ? need_any : one_per_cu);
+        const dim3 grid(rows), block(rpb * gw * WAVE);
+        if (blend) rmsnorm_rev_paired_any<T, W, NV, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
+        else rmsnorm_rev_paired_any<T, W, NV, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
+        return;
+      }
+    }
     if constexpr (!LOOSE && G > WAVE && pairs_fit) {
       /* aligned rows of whole packs in groups of more than a wavefront: rows in pairs, the next
        * row's loads in flight behind the current row's reduction, one workgroup per CU */

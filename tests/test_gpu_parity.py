@@ -802,6 +802,35 @@ def test_rmsnorm_reverse_rows_held_at_three_packs_a_thread(dtype):
                 b.check("rmsnorm rev odd plan")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rmsnorm_reverse_rows_on_five_or_six_wavefronts(dtype):
+    """Rows of 257 ... 447 packs (r16 n = 2560, 3072; r32 n = 1280, 1536): five or six wavefronts a
+    row, three or two rows a workgroup. Whole problem against the oracle, both blends, row counts
+    that are not a multiple of the rows a workgroup holds, and one that leaves workgroups idle."""
+    r = rng(67)
+    per_pack = 16 // torch.empty((), dtype=dtype).element_size()
+    for packs in (257, 320, 384, 447):
+        n = packs * per_pack
+        for m in (1, 37, 1000):
+            for alpha in (0.0, -0.5):
+                G.say(f"rmsnorm rev wavefront groups dtype={dtype} ({m},{n}) alpha={alpha}")
+                x = G.dev(r.normal(0, 1, (m, n)), dtype)
+                g = G.dev(r.normal(1, 0.02, n), dtype)
+                dy = G.dev(r.normal(0, 1, (m, n)), dtype)
+                dx = G.dev(r.normal(0, 1, (m, n)), dtype)
+                dg = G.dev(r.normal(0, 1, n), dtype)
+                hdx, hdg = G.host(dx.t).copy(), G.host(dg.t).copy()
+                scratch, _ = G.rmsnorm_scratch(dtype, m, n)
+                G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, 1e-6, alpha)
+                xh, gh, dyh = G.host(x.t), G.host(g.t), G.host(dy.t)
+                rdx, rdg = O.rmsnorm_ij_j_reverse(xh, gh, dyh, 1e-6, hdx if alpha else None, hdg if alpha else None, alpha)
+                sdx, sdg = G.rmsnorm_reverse_scales(xh, gh, dyh, 1e-6, hdx if alpha else None, hdg if alpha else None, alpha)
+                G.compare(dx.t, rdx, dtype, f"rmsnorm rev wavefront groups dx ({m},{n}) alpha {alpha}", scale=sdx)
+                G.compare(dg.t, rdg, dtype, f"rmsnorm rev wavefront groups dg ({m},{n}) alpha {alpha}", rowwise=False, scale=sdg)
+                for b in (x, g, dy, dx, dg, scratch):
+                    b.check("rmsnorm rev wavefront groups")
+
+
 def test_rmsnorm_reverse_long_rows_in_place():
     # dx written over dy: the shared-row path must not be taken
     r = rng(63)
