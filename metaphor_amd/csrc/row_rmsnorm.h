@@ -577,7 +577,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
  * not on sixteen). The group's width is a kernel argument, not a template parameter: one kernel
  * per (type, packs a thread, blend) serves every width. Sums of a group fold over sixteen slots of
  * which the ones past gw read as zero. */
-constexpr int ANY_MAX_ROWS = 4; /* groups per workgroup the LDS below is sized for: widths from 4 wavefronts */
+constexpr int ANY_MAX_ROWS = 8; /* groups per workgroup the LDS below is sized for: widths from 2 wavefronts */
 
 template <class T, int W, int NV, bool BLEND>
 __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
@@ -1289,12 +1289,13 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
     /* two register sets of x and dy beside the gain and the dg sums: up to eight registers an array
      * fit the 128 of a 1024-thread workgroup without spills */
     constexpr bool pairs_fit = NV * W * (int)(sizeof(P) / 4) <= 8;
-    /* rows of 257 ... 447 packs leave a 512-thread group more than an eighth idle and two such groups
-     * a workgroup: five or six wavefronts a row and three or two rows a workgroup instead (interleaved
-     * repeats: r16 n = 2560 4.30 -> 5.43 TB/s, 3072 5.03 -> 5.48; r32 n = 1280 5.09 -> 5.50, 1536 5.40 ->
-     * 5.95). Wider rows gain nothing from shedding their idle wavefronts (n = 5120 r16: 4.80 -> 4.87,
-     * with two such workgroups a CU 4.73) and keep the power-of-two groups. */
-    if constexpr (!LOOSE && G == 512 && NV == 1 && pairs_fit) {
+    /* rows of 129 ... 223 and 257 ... 447 packs leave a 256- or 512-thread group more than an eighth
+     * idle: three to six wavefronts a row and as many rows a workgroup as fit 1024 threads instead
+     * (interleaved repeats: r16 n = 1152 4.01 -> 4.72 TB/s, 1280 4.59 -> 5.17, 2560 4.30 -> 5.43, 3072
+     * 5.03 -> 5.48; r32 n = 576 4.78 -> 5.39, 1280 5.09 -> 5.50, 1536 5.40 -> 5.95). Wider rows gain nothing
+     * from shedding their idle wavefronts (n = 5120 r16: 4.80 -> 4.87, with two such workgroups a CU
+     * 4.73) and keep the power-of-two groups. */
+    if constexpr (!LOOSE && (G == 512 || G == 256) && NV == 1 && pairs_fit) {
       const int gw = (int)((packs + WAVE - 1) / WAVE);
       if (row_regime_override() == REGIME_AUTO && packs * 8 < (size_t)G * 7 && gw >= NORM_BLOCK / WAVE / ANY_MAX_ROWS) {
         const int rpb = NORM_BLOCK / (gw * WAVE);
