@@ -126,6 +126,70 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
   }
 }
 
+/* The resident forward for aligned rows of whole packs held by `gw` wavefronts a row, any number
+ * from 2 to 16 (a kernel argument), and as many rows a workgroup as the launch gives it threads
+ * for: rows that a power of two of wavefronts would leave partly idle. Sums of a group fold over
+ * sixteen slots of which the ones past gw read as zero. */
+constexpr int ANY_MAX_ROWS = 8; /* groups per workgroup the LDS of the wavefront-group kernels is sized for */
+
+template <class T, int W, int NV>
+__global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_fwd_any(
+    const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n, int gw) {
+  using P = typename precision<T>::type;
+  constexpr int NW = NORM_BLOCK / WAVE;
+  __shared__ P slots[2][ANY_MAX_ROWS][NW];
+  const int G = gw * WAVE, RPB = (int)blockDim.x / G;
+  const int sub = threadIdx.x / G, lane = threadIdx.x % G;
+  const int npk = (int)(n / W);
+
+  P gv[NV][W];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = k * G + lane;
+#pragma unroll
+    for (int i = 0; i < W; ++i) gv[k][i] = (P)0;
+    if (p < npk) load_pack<T, W>(gain + (size_t)p * W, gv[k]);
+  }
+  int parity = 0;
+  for (size_t base = (size_t)blockIdx.x * RPB; base < m; base += (size_t)gridDim.x * RPB, parity ^= 1) {
+    const size_t row = base + sub;
+    const bool live = row < m; /* uniform per wavefront; dead groups still meet the barrier */
+    const T* xr = x + (live ? row : 0) * n;
+    P xv[NV][W];
+    P ss = (P)0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = k * G + lane;
+      if (live && p < npk) {
+        load_pack_nt<T, W>(xr + (size_t)p * W, xv[k]);
+      } else {
+#pragma unroll
+        for (int i = 0; i < W; ++i) xv[k][i] = (P)0;
+      }
+#pragma unroll
+      for (int i = 0; i < W; ++i) ss += xv[k][i] * xv[k][i];
+    }
+    ss = wave_allreduce<AddOP>(ss);
+    if ((lane & (WAVE - 1)) == 0) slots[parity][sub][lane / WAVE] = ss;
+    __syncthreads();
+    const int slot = lane & (NW - 1);
+    ss = fold_partials<AddOP, NW>(slot < gw ? slots[parity][sub][slot] : (P)0);
+    const P r = rsqrt_of(ss / (P)n + eps);
+    if (live) {
+      T* yr = y + row * n;
+#pragma unroll
+      for (int k = 0; k < NV; ++k) {
+        const int p = k * G + lane;
+        if (p < npk) {
+#pragma unroll
+          for (int i = 0; i < W; ++i) xv[k][i] *= r * gv[k][i];
+          store_pack_nt<T, W>(yr + (size_t)p * W, xv[k]);
+        }
+      }
+    }
+  }
+}
+
 /* ------------------------------------------------------------------ streaming forward */
 
 /* The packs of a row start where x's alignment puts them; the gain's, and with APART (y not
@@ -577,7 +641,6 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
  * not on sixteen). The group's width is a kernel argument, not a template parameter: one kernel
  * per (type, packs a thread, blend) serves every width. Sums of a group fold over sixteen slots of
  * which the ones past gw read as zero. */
-constexpr int ANY_MAX_ROWS = 8; /* groups per workgroup the LDS below is sized for: widths from 2 wavefronts */
 
 template <class T, int W, int NV, bool BLEND>
 __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
@@ -1229,6 +1292,24 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
    * of two does not idle half of a group twice as wide (r32 n = 257: 4.1 -> 5.1 TB/s, n = 130: 3.8 -> 4.9) */
   const int nv_target = sizeof(T) == 2 || loose ? 2 : 1;
   const RowPlan shot = plan_row(packs, MAXNV, nv_target, 8);
+  /* aligned rows that leave the planned group more than an eighth idle and need at most five
+   * wavefronts at the planned packs a thread: persistent workgroups of three to eight such rows
+   * (interleaved repeats: r16 n = 1152 4.44 -> 5.31 TB/s, 1280 4.99 -> 5.74, 2560 5.20 -> 5.86; r32
+   * n = 576 5.20 -> 6.14, 640 5.57 -> 6.22, 1280 5.84 -> 6.19; one-shot workgroups of the same groups: -4 ... +7 %;
+   * six wavefronts a row: -2 ... +2 %, left with the power-of-two groups) */
+  if (!loose && !mismatch && row_regime_override() == REGIME_AUTO && shot.G >= 128 && shot.G <= 512 && shot.NV <= 2 &&
+      packs * 8 < (size_t)shot.G * shot.NV * 7) {
+    const int gw = (int)((packs + (size_t)WAVE * shot.NV - 1) / ((size_t)WAVE * shot.NV));
+    if (gw >= 2 && gw <= 5) {
+      const int rpb = NORM_BLOCK / WAVE / gw;
+      const size_t need = (m + rpb - 1) / rpb;
+      const dim3 grid((unsigned)(need < cap ? need : cap)), block(rpb * gw * WAVE);
+      if (shot.NV == 1) rmsnorm_fwd_any<T, W, 1><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
+      else rmsnorm_fwd_any<T, W, 2><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
+      MP_CHECK_LAUNCH();
+      return;
+    }
+  }
   const bool take_shot = row_regime_override() == REGIME_AUTO && shot.G > 0 && shot.G <= ONESHOT &&
                          (sizeof(T) != 2 || packs >= 32);
   if (take_shot) {

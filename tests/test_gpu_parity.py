@@ -672,6 +672,29 @@ def test_rmsnorm_forward_unaligned_and_in_place(dtype, regime):
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rmsnorm_forward_rows_on_two_to_five_wavefronts(dtype):
+    """Aligned rows that would leave a power-of-two group more than an eighth idle (r16 n = 1152, 1280,
+    2560, 5120; r32 n = 576, 640, 1280): groups of two to five wavefronts, three to eight rows a
+    persistent workgroup. Row counts around the rows a workgroup holds, and in place."""
+    r = rng(68)
+    per_pack = 16 // torch.empty((), dtype=dtype).element_size()
+    for packs in (129, 144, 160, 223, 257, 300, 320, 447, 520, 640):
+        n = packs * per_pack
+        for m in (1, 7, 37, 2100):
+            G.say(f"rmsnorm fwd wavefront groups dtype={dtype} ({m},{n})")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype)
+            g = G.dev(r.normal(1, 0.02, n), dtype)
+            y = G.Guarded((m, n), dtype)
+            G.rmsnorm(x.t, g.t, y.t, 1e-6)
+            ref = O.rmsnorm_ij_j(G.host(x.t), G.host(g.t), 1e-6)
+            G.compare(y.t, ref, dtype, f"rmsnorm fwd wavefront groups ({m},{n})")
+            G.rmsnorm(x.t, g.t, x.t, 1e-6)
+            G.compare(x.t, ref, dtype, f"rmsnorm fwd wavefront groups in place ({m},{n})")
+            for b in (x, g, y):
+                b.check("rmsnorm fwd wavefront groups")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 @pytest.mark.parametrize("packs,spin", [(0, 1 << 22), (64, 1 << 22), (3, 1 << 22), (64, 0), (1000, 2)],
                          ids=["default", "64packs", "3packs", "64packs-nowait", "1000packs-2polls"])
 def test_rmsnorm_forward_cluster_path(dtype, packs, spin):
