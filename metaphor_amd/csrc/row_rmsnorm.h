@@ -1376,6 +1376,22 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
      * 5.03 -> 5.48; r32 n = 576 4.78 -> 5.39, 1280 5.09 -> 5.50, 1536 5.40 -> 5.95). Wider rows gain nothing
      * from shedding their idle wavefronts (n = 5120 r16: 4.80 -> 4.87, with two such workgroups a CU
      * 4.73) and keep the power-of-two groups. */
+    /* rows of 513 ... 895 packs on one 1024-thread group at a pack a thread: where two packs a thread
+     * fit the paired kernel's registers (r32, r64), five to seven wavefronts a row at two packs a
+     * thread and three or two rows a workgroup (r32 n = 2176: 4.75 -> 5.79 TB/s, 2560: 5.38 -> 6.00, 3328:
+     * 5.25 -> 5.85; 3072: equal) */
+    if constexpr (!LOOSE && G == 1024 && NV == 1 && 2 * W * (int)(sizeof(P) / 4) <= 8) {
+      const int gw = (int)((packs + 2 * WAVE - 1) / (2 * WAVE));
+      if (row_regime_override() == REGIME_AUTO && packs * 8 < (size_t)G * 7 && gw >= 2) {
+        const int rpb = NORM_BLOCK / (gw * WAVE);
+        const size_t need_any = (m + rpb - 1) / rpb, one_per_cu = (size_t)compute_units();
+        rows = (unsigned)(need_any < one_per_cu ? need_any : one_per_cu);
+        const dim3 grid(rows), block(rpb * gw * WAVE);
+        if (blend) rmsnorm_rev_paired_any<T, W, 2, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
+        else rmsnorm_rev_paired_any<T, W, 2, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
+        return;
+      }
+    }
     if constexpr (!LOOSE && (G == 512 || G == 256) && NV == 1 && pairs_fit) {
       const int gw = (int)((packs + WAVE - 1) / WAVE);
       if (row_regime_override() == REGIME_AUTO && packs * 8 < (size_t)G * 7 && gw >= NORM_BLOCK / WAVE / ANY_MAX_ROWS) {
