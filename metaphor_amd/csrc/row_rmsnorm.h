@@ -650,20 +650,24 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
   using V = typename vec_of<T, W>::type;
   constexpr int NW = NORM_BLOCK / WAVE;
   __shared__ P slots[2][2][ANY_MAX_ROWS][NW];
-  __shared__ P comb[NORM_BLOCK * NV * W];
+  constexpr int COMB = NORM_BLOCK * (NV * W < 8 ? NV * W : 8); /* one row of dg sums: the launcher keeps G * NV * W within it */
+  __shared__ P comb[COMB];
 
   const int G = gw * WAVE, RPB = (int)blockDim.x / G;
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
   const int npk = (int)(n / W);
   const size_t last = m - 1, stride = (size_t)gridDim.x * RPB;
 
-  P gv[NV][W], acc[NV][W];
+  /* the gain stays in the storage type like x and dy and is widened where it is used: for two-byte
+   * types that is what lets two packs a thread fit beside the two register sets */
+  V gv[NV];
+  P acc[NV][W];
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
     const int p = k * G + lane;
 #pragma unroll
-    for (int i = 0; i < W; ++i) acc[k][i] = gv[k][i] = (P)0;
-    if (p < npk) load_pack<T, W>(gain + (size_t)p * W, gv[k]);
+    for (int i = 0; i < W; ++i) acc[k][i] = (P)0;
+    gv[k] = *reinterpret_cast<const V*>(gain + (size_t)(p < npk ? p : 0) * W);
   }
 
   auto fetch = [&](V (&xs)[NV], V (&ds)[NV], size_t base) {
@@ -682,17 +686,16 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
   auto finish = [&](const V (&xs)[NV], const V (&ds)[NV], size_t base, P (*sl)[ANY_MAX_ROWS][NW]) {
     const size_t row = base + sub;
     const bool live = row < m;
-    P xv[NV][W], dv[NV][W];
     P ss = (P)0, c = (P)0;
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
-      const bool inside = k * G + lane < npk;
+      if (k * G + lane < npk) { /* a pack beyond the row was loaded from its start and is dropped */
 #pragma unroll
-      for (int i = 0; i < W; ++i) {
-        xv[k][i] = inside ? (P)xs[k][i] : (P)0;
-        dv[k][i] = inside ? (P)ds[k][i] : (P)0;
-        ss += xv[k][i] * xv[k][i];
-        c += dv[k][i] * gv[k][i] * xv[k][i];
+        for (int i = 0; i < W; ++i) {
+          const P xv = (P)xs[k][i];
+          ss += xv * xv;
+          c += (P)ds[k][i] * (P)gv[k][i] * xv;
+        }
       }
     }
     ss = wave_allreduce<AddOP>(ss);
@@ -716,8 +719,9 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
           P out[W];
 #pragma unroll
           for (int i = 0; i < W; ++i) {
-            out[i] = r * (dv[k][i] * gv[k][i] - xv[k][i] * cc);
-            acc[k][i] += dv[k][i] * xv[k][i] * r;
+            const P xv = (P)xs[k][i], dv = (P)ds[k][i];
+            out[i] = r * (dv * (P)gv[k][i] - xv * cc);
+            acc[k][i] += dv * xv * r;
           }
           if constexpr (BLEND) {
             P old[W];
@@ -735,9 +739,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
   size_t base = (size_t)blockIdx.x * RPB;
   fetch(ax, ad, base);
 #pragma unroll
-  for (int k = 0; k < NV; ++k)
-#pragma unroll
-    for (int i = 0; i < W; ++i) settle(gv[k][i]);
+  for (int k = 0; k < NV; ++k) settle(gv[k]); /* the gain is waited for here, not inside the loop */
   for (; base < m; base += 2 * stride) {
     fetch(bx, bd, base + stride);
     __builtin_amdgcn_sched_barrier(0);
@@ -747,19 +749,21 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
     finish(bx, bd, base + stride, slots[1]);
   }
 
-  /* one partial row per workgroup: the groups' sums meet in LDS */
-  const int row_slots = G * NV * W;
+  /* one partial row per workgroup: the groups add their sums into one row in LDS, one after the other */
+  for (int turn = 0; turn < RPB; ++turn) {
+    if (sub == turn) {
 #pragma unroll
-  for (int k = 0; k < NV; ++k)
+      for (int k = 0; k < NV; ++k)
 #pragma unroll
-    for (int i = 0; i < W; ++i) comb[sub * row_slots + (k * G + lane) * W + i] = acc[k][i];
-  __syncthreads();
-  P* mine = partials + (size_t)blockIdx.x * n;
-  for (size_t col = threadIdx.x; col < n; col += blockDim.x) {
-    P t = (P)0;
-    for (int s2 = 0; s2 < RPB; ++s2) t += comb[s2 * row_slots + col];
-    mine[col] = t;
+        for (int i = 0; i < W; ++i) {
+          P& cell = comb[(k * G + lane) * W + i];
+          cell = turn == 0 ? acc[k][i] : cell + acc[k][i];
+        }
+    }
+    __syncthreads();
   }
+  P* mine = partials + (size_t)blockIdx.x * n;
+  for (size_t col = threadIdx.x; col < n; col += blockDim.x) mine[col] = comb[col];
 }
 
 /* ------------------------------------------------------------------ streaming reverse */
@@ -1376,13 +1380,16 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
      * 5.03 -> 5.48; r32 n = 576 4.78 -> 5.39, 1280 5.09 -> 5.50, 1536 5.40 -> 5.95). Wider rows gain nothing
      * from shedding their idle wavefronts (n = 5120 r16: 4.80 -> 4.87, with two such workgroups a CU
      * 4.73) and keep the power-of-two groups. */
-    /* rows of 513 ... 895 packs on one 1024-thread group at a pack a thread: where two packs a thread
-     * fit the paired kernel's registers (r32, r64), five to seven wavefronts a row at two packs a
-     * thread and three or two rows a workgroup (r32 n = 2176: 4.75 -> 5.79 TB/s, 2560: 5.38 -> 6.00, 3328:
-     * 5.25 -> 5.85; 3072: equal) */
-    if constexpr (!LOOSE && G == 1024 && NV == 1 && 2 * W * (int)(sizeof(P) / 4) <= 8) {
+    /* rows of 513 ... 896 packs on one 1024-thread group at a pack a thread: five to seven wavefronts
+     * a row at two packs a thread and three or two rows a workgroup. r32 and r64 hold the widened
+     * packs; r16 would not fit them twice over, so the kernel keeps x, dy and gain as loaded and
+     * widens on use (r32 n = 2176: 4.75 -> 5.79 TB/s, 2560: 5.38 -> 6.00, 3328: 5.25 -> 5.85, 3584:
+     * 5.31 -> 5.89, 3072: equal; r16 n = 4352: 4.26 -> 5.67, 5120: 4.80 -> 5.91, 6144: 5.49 -> 6.15,
+     * 6656: 5.07 -> 5.73, 7168: 4.88 -> 5.69). Seven eighths of a 512- or 256-thread group: -2 ... +3 %,
+     * left with the power-of-two groups. */
+    if constexpr (!LOOSE && G == 1024 && NV == 1 && (2 * W * (int)(sizeof(P) / 4) <= 8 || sizeof(T) == 2)) {
       const int gw = (int)((packs + 2 * WAVE - 1) / (2 * WAVE));
-      if (row_regime_override() == REGIME_AUTO && packs * 8 < (size_t)G * 7 && gw >= 2) {
+      if (row_regime_override() == REGIME_AUTO && packs * 8 <= (size_t)G * 7 && gw >= 2 && gw * WAVE * 2 * W <= NORM_BLOCK * 8) {
         const int rpb = NORM_BLOCK / (gw * WAVE);
         const size_t need_any = (m + rpb - 1) / rpb, one_per_cu = (size_t)compute_units();
         rows = (unsigned)(need_any < one_per_cu ? need_any : one_per_cu);
