@@ -511,8 +511,10 @@ __device__ __forceinline__ void group_allreduce_sum2_lds(P& a, P& b, P* slots_a,
  * both are dropped), and reductions behind a barrier that does not wait for global loads. One
  * workgroup per CU then moves what two of the unpaired kernel move (r32 [8192, 4096]: 66.4 -> 63.9 us,
  * against 63.1 for a plain two-reads-one-write pass over the same bytes), and leaves half as
- * many partial rows. EXACT: every thread's NV packs lie inside the row (n == G * NV * W). */
-template <class T, int W, int G, int NV, bool BLEND, bool EXACT>
+ * many partial rows. EXACT: every thread's NV packs lie inside the row (n == G * NV * W).
+ * DEPTH 3: three register sets, two rows on their way while a third is reduced; the launcher says
+ * where that pays. */
+template <class T, int W, int G, int NV, bool BLEND, bool EXACT, int DEPTH = 2>
 __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
@@ -520,7 +522,8 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
   using V = typename vec_of<T, W>::type;
   static_assert(G > WAVE && G <= NORM_BLOCK, "groups of 128 ... 1024 threads");
   constexpr int RPB = NORM_BLOCK / G;
-  __shared__ P slots[2][2][RPB][G / WAVE];
+  static_assert(DEPTH == 2 || DEPTH == 3, "two or three register sets");
+  __shared__ P slots[DEPTH][2][RPB][G / WAVE];
   __shared__ P comb[RPB > 1 ? NORM_BLOCK * NV * W : 1];
 
   const int sub = threadIdx.x / G, lane = threadIdx.x % G;
@@ -595,17 +598,33 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
   V ax[NV], ad[NV], bx[NV], bd[NV];
   size_t base = (size_t)blockIdx.x * RPB;
   fetch(ax, ad, base);
+  if constexpr (DEPTH == 3) fetch(bx, bd, base + stride);
 #pragma unroll
   for (int k = 0; k < NV; ++k)
 #pragma unroll
     for (int i = 0; i < W; ++i) settle(gv[k][i]); /* the gain is waited for here, not inside the loop */
-  for (; base < m; base += 2 * stride) {
-    fetch(bx, bd, base + stride);
-    __builtin_amdgcn_sched_barrier(0);
-    finish(ax, ad, base, slots[0]);
-    fetch(ax, ad, base + 2 * stride);
-    __builtin_amdgcn_sched_barrier(0);
-    finish(bx, bd, base + stride, slots[1]);
+  if constexpr (DEPTH == 3) { /* two rows on their way while a third is reduced and written */
+    V cx[NV], cd[NV];
+    for (; base < m; base += 3 * stride) {
+      fetch(cx, cd, base + 2 * stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(ax, ad, base, slots[0]);
+      fetch(ax, ad, base + 3 * stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(bx, bd, base + stride, slots[1]);
+      fetch(bx, bd, base + 4 * stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(cx, cd, base + 2 * stride, slots[DEPTH - 1]);
+    }
+  } else {
+    for (; base < m; base += 2 * stride) {
+      fetch(bx, bd, base + stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(ax, ad, base, slots[0]);
+      fetch(ax, ad, base + 2 * stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(bx, bd, base + stride, slots[1]);
+    }
   }
 
   /* one partial row per workgroup */
@@ -642,14 +661,14 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
  * per (type, packs a thread, blend) serves every width. Sums of a group fold over sixteen slots of
  * which the ones past gw read as zero. */
 
-template <class T, int W, int NV, bool BLEND>
+template <class T, int W, int NV, bool BLEND, int DEPTH = 2>
 __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n, int gw) {
   using P = typename precision<T>::type;
   using V = typename vec_of<T, W>::type;
   constexpr int NW = NORM_BLOCK / WAVE;
-  __shared__ P slots[2][2][ANY_MAX_ROWS][NW];
+  __shared__ P slots[DEPTH][2][ANY_MAX_ROWS][NW];
   constexpr int COMB = NORM_BLOCK * (NV * W < 8 ? NV * W : 8); /* one row of dg sums: the launcher keeps G * NV * W within it */
   __shared__ P comb[COMB];
 
@@ -738,15 +757,31 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
   V ax[NV], ad[NV], bx[NV], bd[NV];
   size_t base = (size_t)blockIdx.x * RPB;
   fetch(ax, ad, base);
+  if constexpr (DEPTH == 3) fetch(bx, bd, base + stride);
 #pragma unroll
   for (int k = 0; k < NV; ++k) settle(gv[k]); /* the gain is waited for here, not inside the loop */
-  for (; base < m; base += 2 * stride) {
-    fetch(bx, bd, base + stride);
-    __builtin_amdgcn_sched_barrier(0);
-    finish(ax, ad, base, slots[0]);
-    fetch(ax, ad, base + 2 * stride);
-    __builtin_amdgcn_sched_barrier(0);
-    finish(bx, bd, base + stride, slots[1]);
+  if constexpr (DEPTH == 3) {
+    V cx[NV], cd[NV];
+    for (; base < m; base += 3 * stride) {
+      fetch(cx, cd, base + 2 * stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(ax, ad, base, slots[0]);
+      fetch(ax, ad, base + 3 * stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(bx, bd, base + stride, slots[1]);
+      fetch(bx, bd, base + 4 * stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(cx, cd, base + 2 * stride, slots[DEPTH - 1]);
+    }
+  } else {
+    for (; base < m; base += 2 * stride) {
+      fetch(bx, bd, base + stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(ax, ad, base, slots[0]);
+      fetch(ax, ad, base + 2 * stride);
+      __builtin_amdgcn_sched_barrier(0);
+      finish(bx, bd, base + stride, slots[1]);
+    }
   }
 
   /* one partial row per workgroup: the groups add their sums into one row in LDS, one after the other */
@@ -1406,8 +1441,15 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
         const size_t need_any = (m + rpb - 1) / rpb, one_per_cu = (size_t)compute_units();
         rows = (unsigned)(need_any < one_per_cu ? need_any : one_per_cu);
         const dim3 grid(rows), block(rpb * gw * WAVE);
-        if (blend) rmsnorm_rev_paired_any<T, W, NV, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
-        else rmsnorm_rev_paired_any<T, W, NV, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
+        /* a third register set for two-byte types and for the shortest rows of four-byte ones (interleaved
+         * repeats: r16 n = 1280 4.71 -> 5.99 TB/s, 3072 5.55 -> 5.87, 2560 equal; r32 n = 640 5.36 -> 5.71,
+         * 1280 equal, 1536 5.86 -> 5.68) */
+        const bool deep = sizeof(T) == 2 || (sizeof(T) == 4 && gw <= 4);
+        auto go = [&]<bool BLEND, int DEPTH>() {
+          rmsnorm_rev_paired_any<T, W, NV, BLEND, DEPTH><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
+        };
+        if (blend) { if (deep) go.template operator()<true, 3>(); else go.template operator()<true, 2>(); }
+        else { if (deep) go.template operator()<false, 3>(); else go.template operator()<false, 2>(); }
         return;
       }
     }
@@ -1418,8 +1460,13 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
       rows = (unsigned)(need < one_per_cu ? need : one_per_cu);
       const dim3 grid(rows), block(NORM_BLOCK);
       const bool exact = n == (size_t)G * NV * W;
+      /* a third register set where a row is short enough that two sets in flight do not cover the
+       * memory latency (interleaved repeats: r16 n = 1024 5.45 -> 6.09 TB/s, 2048 5.89 -> 6.08, 4096
+       * 5.89 -> 6.10, 8192 6.16 -> 6.06; r32 n = 512 5.81 -> 6.04, 1024 6.09 -> 5.97, 2048 6.04 -> 5.57,
+       * 4096 5.99 -> 5.81) */
+      constexpr int DEPTH = NV == 1 && ((sizeof(T) == 2 && G <= 512) || G == 128) ? 3 : 2;
       auto go = [&]<bool BLEND, bool EXACT>() {
-        rmsnorm_rev_paired<T, W, G, NV, BLEND, EXACT><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+        rmsnorm_rev_paired<T, W, G, NV, BLEND, EXACT, DEPTH><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
       };
       if (blend) { if (exact) go.template operator()<true, true>(); else go.template operator()<true, false>(); }
       else { if (exact) go.template operator()<false, true>(); else go.template operator()<false, false>(); }

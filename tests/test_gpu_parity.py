@@ -855,6 +855,38 @@ def test_rmsnorm_reverse_rows_on_three_to_six_wavefronts(dtype):
                     b.check("rmsnorm rev wavefront groups")
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_rmsnorm_reverse_three_rows_in_flight_ends_at_every_step(dtype):
+    """Short rows run with three register sets that take turns (two rows on their way while a third is
+    reduced): row counts that leave the three-step loop after each of its steps, after one to three
+    whole turns, on a power-of-two group (128 packs), a three-wavefront group (160) and, for r16, a
+    512-thread group (448 packs). Whole problem against the oracle, both blends."""
+    r = rng(71)
+    per_pack = 16 // torch.empty((), dtype=dtype).element_size()
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    for packs, rows_a_group in ((128, 8), (160, 5), (448, 2)):
+        n = packs * per_pack
+        step = cus * rows_a_group  # rows that one step of every workgroup covers
+        for m in (3 * step + 7, 4 * step + 1, 5 * step, 6 * step + step // 2, 9 * step - 1):
+            alpha = 0.0 if m % 2 else -0.5
+            G.say(f"rmsnorm rev three sets dtype={dtype} ({m},{n}) alpha={alpha}")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype)
+            g = G.dev(r.normal(1, 0.02, n), dtype)
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dx = G.dev(r.normal(0, 1, (m, n)), dtype)
+            dg = G.dev(r.normal(0, 1, n), dtype)
+            hdx, hdg = G.host(dx.t).copy(), G.host(dg.t).copy()
+            scratch, _ = G.rmsnorm_scratch(dtype, m, n)
+            G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, 1e-6, alpha)
+            xh, gh, dyh = G.host(x.t), G.host(g.t), G.host(dy.t)
+            rdx, rdg = O.rmsnorm_ij_j_reverse(xh, gh, dyh, 1e-6, hdx if alpha else None, hdg if alpha else None, alpha)
+            sdx, sdg = G.rmsnorm_reverse_scales(xh, gh, dyh, 1e-6, hdx if alpha else None, hdg if alpha else None, alpha)
+            G.compare(dx.t, rdx, dtype, f"rmsnorm rev three sets dx ({m},{n}) alpha {alpha}", scale=sdx)
+            G.compare(dg.t, rdg, dtype, f"rmsnorm rev three sets dg ({m},{n}) alpha {alpha}", rowwise=False, scale=sdg)
+            for b in (x, g, dy, dx, dg, scratch):
+                b.check("rmsnorm rev three sets")
+
+
 def test_rmsnorm_reverse_long_rows_in_place():
     # dx written over dy: the shared-row path must not be taken
     r = rng(63)
