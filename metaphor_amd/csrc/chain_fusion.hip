@@ -22,6 +22,7 @@
 
 #include <hip/hiprtc.h>
 
+#include <atomic>
 #include <map>
 #include <memory>
 #include <mutex>
@@ -352,18 +353,24 @@ bool compile(const std::string& source, std::vector<char>& code, std::string& er
 /* ---------------------------------------------------------------- the process-wide cache */
 
 struct Loaded {
+  std::atomic<bool> ready{false}; /* set after module and fn are written, read before they are used */
   hipModule_t module = nullptr;
   hipFunction_t fn[9] = {};
 };
 
+/* `build` is held while this chain is compiled or loaded on a device, so that neither holds up
+ * calls for other chains; `compiled` and Loaded::ready let calls for a chain that is ready pass
+ * without taking it. */
 struct Chain {
   int leaves = 0;
   std::string source;
+  std::mutex build;
+  std::atomic<bool> compiled{false};
   std::vector<char> code;
   Loaded on_device[MAX_DEVICES];
 };
 
-std::mutex cache_lock;
+std::mutex cache_lock; /* the map only: held for a lookup or an insertion, never for a compilation */
 std::map<std::pair<std::string, int>, std::unique_ptr<Chain>> cache; /* entries are never removed */
 
 /* The chain of (signature, dtype): its source on first sight, its code object when `compiled` is
@@ -383,23 +390,30 @@ Chain* chain_for(const char* signature, int dtype, bool compiled) {
   }
   std::string canonical;
   spell(e, e.root, canonical);
-  std::lock_guard<std::mutex> hold(cache_lock);
-  auto key = std::make_pair(canonical, dtype);
-  auto it = cache.find(key);
-  if (it == cache.end()) {
-    auto c = std::make_unique<Chain>();
-    c->leaves = e.leaves;
-    c->source = chain_source(e, dtype);
-    it = cache.emplace(std::move(key), std::move(c)).first;
-  }
-  Chain* c = it->second.get();
-  if (compiled && c->code.empty()) {
-    std::vector<char> code;
-    if (!compile(c->source, code, err)) {
-      fail(std::string("chain \"") + signature + "\": " + err);
-      return nullptr;
+  Chain* c = nullptr;
+  {
+    std::lock_guard<std::mutex> hold(cache_lock);
+    auto key = std::make_pair(canonical, dtype);
+    auto it = cache.find(key);
+    if (it == cache.end()) {
+      auto fresh = std::make_unique<Chain>();
+      fresh->leaves = e.leaves;
+      fresh->source = chain_source(e, dtype);
+      it = cache.emplace(std::move(key), std::move(fresh)).first;
     }
-    c->code = std::move(code);
+    c = it->second.get();
+  }
+  if (compiled && !c->compiled.load(std::memory_order_acquire)) {
+    std::lock_guard<std::mutex> hold(c->build);
+    if (!c->compiled.load(std::memory_order_relaxed)) {
+      std::vector<char> code;
+      if (!compile(c->source, code, err)) {
+        fail(std::string("chain \"") + signature + "\": " + err);
+        return nullptr;
+      }
+      c->code = std::move(code);
+      c->compiled.store(true, std::memory_order_release);
+    }
   }
   return c;
 }
@@ -411,9 +425,10 @@ const Loaded* loaded_here(Chain* c) {
     fail("no current device");
     return nullptr;
   }
-  std::lock_guard<std::mutex> hold(cache_lock);
   Loaded& l = c->on_device[dev];
-  if (l.module != nullptr) return &l;
+  if (l.ready.load(std::memory_order_acquire)) return &l;
+  std::lock_guard<std::mutex> hold(c->build);
+  if (l.ready.load(std::memory_order_relaxed)) return &l;
   hipModule_t module = nullptr;
   hipError_t r = hipModuleLoadData(&module, c->code.data());
   if (r != hipSuccess) {
@@ -432,6 +447,7 @@ const Loaded* loaded_here(Chain* c) {
       }
     }
   l.module = module;
+  l.ready.store(true, std::memory_order_release);
   return &l;
 }
 
@@ -488,6 +504,7 @@ extern "C" const void* mpChainCodeObject(const char* signature, int dtype, len_t
 }
 
 extern "C" int mpChainForward(const char* signature, int dtype, const void* const* x, void* out, len_t n, StreamContext stream) {
+  if (x == nullptr) return fail("no operand array");
   Chain* c = chain_for(signature, dtype, true);
   if (c == nullptr) return 1;
   void* outs[1] = {out};
@@ -496,6 +513,7 @@ extern "C" int mpChainForward(const char* signature, int dtype, const void* cons
 
 extern "C" int mpChainReverse(const char* signature, int dtype, const void* const* x, const void* out_grads, void* const* g,
                               double alpha, len_t n, StreamContext stream) {
+  if (x == nullptr || g == nullptr) return fail("no operand array");
   Chain* c = chain_for(signature, dtype, true);
   if (c == nullptr) return 1;
   const int k = c->leaves;
@@ -510,7 +528,7 @@ extern "C" int mpChainReverse(const char* signature, int dtype, const void* cons
 extern "C" len_t mpChainCacheSize(void) {
   std::lock_guard<std::mutex> hold(cache_lock);
   len_t n = 0;
-  for (const auto& kv : cache) n += kv.second->code.empty() ? 0 : 1;
+  for (const auto& kv : cache) n += kv.second->compiled.load(std::memory_order_acquire) ? 1 : 0;
   return n;
 }
 

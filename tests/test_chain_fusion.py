@@ -140,3 +140,39 @@ def test_the_fusion_library_exports_what_its_header_declares():
                                     "mpChainSource", "mpChainCodeObject", "mpChainCacheSize", "mpChainError"])
     for n in names:
         assert getattr(lib, n)
+
+
+def test_several_threads_compile_at_once():
+    """Eight threads ask for four new expressions, two threads an expression: every call succeeds, each
+    expression is compiled once, and a thread's error text is its own."""
+    import threading
+    lib = ffi.load_fusion()
+    exprs = [f"relu(shift(mul(0,1),{k}.25))".encode() for k in range(4)]
+    before = lib.mpChainCacheSize()
+    results = [None] * 8
+
+    def work(i):
+        if i == 7:  # one thread fails meanwhile; the others must not see its error
+            results[i] = (lib.mpChainCompile(b"foo(0)", 1), lib.mpChainError().decode())
+        else:
+            results[i] = (lib.mpChainCompile(exprs[i % 4], 1), lib.mpChainError().decode())
+
+    threads = [threading.Thread(target=work, args=(i,)) for i in range(8)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join()
+    assert [r[0] for r in results[:7]] == [0] * 7, results
+    assert results[7][0] != 0 and "unknown op" in results[7][1]
+    assert all("unknown op" not in r[1] for r in results[:7])
+    assert lib.mpChainCacheSize() == before + 4
+
+
+def test_missing_operand_arrays_are_refused():
+    """No array of leaf pointers: refused before anything touches a device."""
+    lib = ffi.load_fusion()
+    ctx = ffi.StreamContext()
+    assert lib.mpChainForward(b"add(0,1)", 1, None, None, 16, ctx) != 0
+    assert "operand array" in lib.mpChainError().decode()
+    assert lib.mpChainReverse(b"add(0,1)", 1, None, None, None, 0.0, 16, ctx) != 0
+    assert "operand array" in lib.mpChainError().decode()
