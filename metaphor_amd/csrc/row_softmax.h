@@ -608,6 +608,9 @@ template <class T> inline int cluster_size(size_t packs) {
    * two workgroups a row win or tie: n = 24576 6.10 against 5.76, 32768 equal; sixteen packs a thread
    * in 256 or 512 threads, an earlier choice, 5.78 / 5.37 / 5.58 / 5.70) */
   if (regime == REGIME_AUTO && sizeof(T) == 4 && packs > resident + 1 && packs <= 4096) return 0;
+  /* r16 rows of exactly 64 KiB as well (n = 32768: 5.51 -> 5.89 TB/s); every other length from 24576
+   * to 32000 ties or is better here */
+  if (regime == REGIME_AUTO && sizeof(T) == 2 && packs == 4096) return 0;
   constexpr size_t tile = (size_t)CLUSTER_THREADS * cluster_nv<T>();
   size_t ppb = (size_t)cluster_tuning().packs_per_block;
   if (ppb == 0) ppb = sizeof(T) == 2 ? tile : tile - CLUSTER_THREADS;
@@ -925,6 +928,9 @@ template <class T> inline int cluster_rev_size(size_t packs) {
   const int regime = row_regime_override();
   if (regime != REGIME_AUTO && regime != REGIME_CLUSTER) return 0;
   if (regime == REGIME_AUTO && packs <= (size_t)CLUSTER_THREADS * 2) return 0; /* one workgroup, two packs each */
+  /* r16 rows of exactly 64 KiB stay with one persistent workgroup at four packs a thread (interleaved
+   * repeats, n = 32768: 5.48 -> 5.75 TB/s; 24576 ... 32000: 1 ... 7 % better shared) */
+  if (regime == REGIME_AUTO && sizeof(T) == 2 && packs == 4096) return 0;
   constexpr size_t tile = (size_t)CLUSTER_THREADS * CLUSTER_REV_NV;
   size_t ppb = (size_t)cluster_tuning().packs_per_block;
   if (ppb == 0 || ppb > tile) ppb = tile;
