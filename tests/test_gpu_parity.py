@@ -346,7 +346,7 @@ def test_reference_example_reductions():
 # ------------------------------------------------------------------ softmax
 
 SOFTMAX_SHAPES = [(1, 1), (3, 7), (5, 64), (4, 65), (1031, 16), (9, 256), (7, 1000), (256, 1024), (6, 2048),
-                  (3, 5000), (5, 8192), (2, 20000), (2, 50257), (1, 151936), (1030, 33), (2051, 8), (515, 32)]
+                  (3, 5000), (5, 8192), (2, 20000), (3, 32768), (2, 50257), (3, 65536), (1, 151936), (1030, 33), (2051, 8), (515, 32)]
 
 
 def _softmax_inputs(r, m, n, dtype, masked):
