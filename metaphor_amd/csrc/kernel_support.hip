@@ -81,4 +81,12 @@ extern "C" void mpSetClusterTuning(len_t packs_per_block, len_t spin_limit) {
   mp::cluster_tuning().packs_per_block = (int)packs_per_block;
   mp::cluster_tuning().spin_limit = (unsigned)spin_limit;
 }
+
+// Diagnostic: which kernel the RMSNorm reverse runs on shared rows of four-byte types: 0 by the
+// launcher's rule (the pipelined kernel from 8193 packs a row on), 1 always the pipelined kernel,
+// 2 never. Tests use 1 to drive that kernel on small rows. Process-wide.
+extern "C" void mpSetClusterDeep(len_t which) {
+  mp::require(which <= 2, "mpSetClusterDeep: 0, 1 or 2");
+  mp::cluster_tuning().deep = (int)which;
+}
 #endif

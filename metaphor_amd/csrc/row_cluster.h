@@ -49,6 +49,7 @@ template <class Word> __global__ __launch_bounds__(256) void cluster_zero_slots(
 struct ClusterTuning {
   int packs_per_block = 0; /* 0: one pack per thread less than the register tile holds */
   unsigned spin_limit = 1u << 22;
+  int deep = 0; /* the RMSNorm reverse's shared rows: 0 by the launcher's rule, 1 always the pipelined kernel, 2 never */
 };
 #ifdef MP_DIAGNOSTICS
 inline ClusterTuning& cluster_tuning() {

@@ -1105,6 +1105,258 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
   }
 }
 
+/* The same as a pipeline over the rows of a slice. What the kernel above cannot hide is the exchange
+ * itself: a row's sums are published and then waited for, and until the partners' words arrive
+ * (another CU, often another XCD) the workgroup has nothing to do. Here the sums of row j + 2 are
+ * published and the words of row j + 1 read while row j is written back, so the partners' words of
+ * a row have had a whole iteration to arrive when they are asked for, and nobody waits while they
+ * are fetched; the chunk of row j + 3 is on its way meanwhile. Four register sets take turns
+ * (being written back, waiting for its totals, just reduced, loading).
+ * A wavefront's loads return in order, so a wavefront that polled behind loads of its own would
+ * wait for them first: the last wavefront of the workgroup holds no data and is the only one that
+ * publishes and polls, the other fifteen hold the chunk (960 lanes, two packs each), the gain
+ * chunk stays in registers and every barrier orders LDS only. One workgroup per CU. */
+constexpr int DEEP_LANES = CLUSTER_THREADS - WAVE; /* lanes of a workgroup that hold data */
+/* Which rows take it. Four-byte types only: the four register sets of r16 leave no room for its
+ * dg sums, which are four times as wide as its packs (kept in LDS instead, the kernel spills
+ * regardless and loses 12-21 % to the kernel above), and r64 spills. From 8193 packs a row on
+ * (interleaved repeats, r32: n = 50257 4.27 -> 5.10 TB/s, 65536 5.27 -> 5.44, 100352 4.74 -> 5.46,
+ * 131072 4.92 -> 5.40, 151936 4.44 -> 5.27, 262144 3.99 -> 5.26; below: n = 20480 equal, 24576 5.36 ->
+ * 4.77, 32768 5.53 -> 5.40). The test build can force either kernel. */
+template <class T> inline bool norm_rev_deep(size_t packs) {
+  if (sizeof(T) != 4) return false;
+#ifdef MP_DIAGNOSTICS
+  if (cluster_tuning().deep != 0) return cluster_tuning().deep == 1;
+#endif
+  return packs > 8192;
+}
+/* packs of a row that one workgroup of the shared-row reverse holds */
+template <class T> inline size_t norm_rev_cluster_tile(size_t packs) {
+  return norm_rev_deep<T>(packs) ? (size_t)DEEP_LANES * 2 : (size_t)CLUSTER_THREADS * norm_rev_cluster_nv<T>();
+}
+
+template <class T, int W, bool BLEND>
+__global__ __launch_bounds__(CLUSTER_THREADS) void rmsnorm_rev_cluster_deep(
+    const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
+    typename precision<T>::type eps, typename precision<T>::type alpha,
+    typename slot_word<typename precision<T>::type>::type* slots,
+    size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
+  using P = typename precision<T>::type;
+  using V = typename vec_of<T, W>::type;
+  using Word = typename slot_word<P>::type;
+  constexpr int G = CLUSTER_THREADS, D = DEEP_LANES, NV = 2, NW = G / WAVE;
+  /* the packs start at the row's first element whatever the alignment: the one variant serves
+   * aligned rows as well (built for aligned rows only it needs 17 registers more and spills) */
+  constexpr bool LOOSE = true;
+  __shared__ P red[2][2][NW]; /* [row parity][sum][wavefront]; the sixteenth wavefront's slot stays zero */
+  __shared__ P fb[2][NW];     /* the sums of a workgroup that folds a whole row itself */
+  __shared__ P bc[2][3];      /* [row parity]: the row totals and whether a partner was missing */
+  const int lane = threadIdx.x;
+  const bool messenger = lane >= D;
+  const int ml = lane - D;
+  const int rank = (int)(blockIdx.x % (unsigned)C);
+  const size_t slice = blockIdx.x / (unsigned)C, S = gridDim.x / (unsigned)C;
+  const RowPacks<T, W, LOOSE> rp(n);
+  const int lo = rank * packs_per_block;
+  const int hi = messenger ? 0 : (lo + packs_per_block < rp.npk ? lo + packs_per_block : rp.npk);
+
+  P acc[NV][W];
+  V gv[NV];
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+#pragma unroll
+    for (int i = 0; i < W; ++i) acc[k][i] = (P)0;
+    const int p = lo + k * D + lane;
+    gv[k] = p < hi ? rp.template raw<false>(gain, p) : V{};
+  }
+  if (lane < 2 * NW) (&red[0][0][0])[lane] = (&red[1][0][0])[lane] = (P)0;
+
+  auto fetch = [&](size_t row, V (&xs)[NV], V (&ds)[NV]) {
+    const size_t off = row * n;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * D + lane;
+      xs[k] = p < hi ? rp.template raw<true>(x + off, p) : V{};
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * D + lane;
+      ds[k] = p < hi ? rp.template raw<true>(dy + off, p) : V{};
+    }
+  };
+  /* this workgroup's sums of a row into red[parity]; no barrier */
+  auto sums = [&](V (&xv)[NV], V (&dv)[NV], int parity) {
+    P ss = (P)0, c = (P)0;
+#pragma unroll
+    for (int k = 0; k < NV; ++k)
+#pragma unroll
+      for (int i = 0; i < W; ++i) {
+        const P xf = (P)xv[k][i];
+        ss += xf * xf;
+        c += (P)dv[k][i] * (P)gv[k][i] * xf;
+      }
+    ss = wave_allreduce<AddOP>(ss);
+    c = wave_allreduce<AddOP>(c);
+    if (!messenger && (lane & (WAVE - 1)) == 0) {
+      red[parity][0][lane / WAVE] = ss;
+      red[parity][1][lane / WAVE] = c;
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) { /* no widened copy lives on */
+      forget(xv[k]);
+      forget(dv[k]);
+    }
+  };
+  unsigned patience = spin_limit; /* after the first wait that runs out, no later row is waited for */
+  /* the messenger, between the two barriers of an iteration: the sums in red[parity] go out as row
+   * `ahead`'s (when there is one), the words of row `now` come in */
+  auto exchange = [&](bool has_ahead, size_t ahead, int parity, bool has_now, size_t now, int now_parity) {
+    if (!messenger) return;
+    if (has_ahead) {
+      P mine[2] = {fold_partials<AddOP, NW>(red[parity][0][ml & (NW - 1)]), fold_partials<AddOP, NW>(red[parity][1][ml & (NW - 1)])};
+      if (ml == 0) {
+        Word* words = slots + ahead * (size_t)C * 2;
+#pragma unroll
+        for (int v = 0; v < 2; ++v) {
+          const P part = mine[v] == (P)0 ? -(P)0 : mine[v];
+          __hip_atomic_store(words + (size_t)rank * 2 + v, __builtin_bit_cast(Word, part), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+      }
+    }
+    if (has_now) {
+      Word* words = slots + now * (size_t)C * 2;
+      Word w[2] = {0, 0};
+      bool heard = true;
+      if (ml < C) {
+        for (unsigned spins = 0;; ++spins) {
+          heard = true;
+#pragma unroll
+          for (int v = 0; v < 2; ++v) {
+            w[v] = __hip_atomic_load(words + (size_t)ml * 2 + v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            heard = heard && w[v] != 0;
+          }
+          if (heard || spins >= patience) break;
+          __builtin_amdgcn_s_sleep(4);
+        }
+      }
+      const P missing = wave_allreduce<AddOP>(heard ? (P)0 : (P)1);
+      P total[2];
+#pragma unroll
+      for (int v = 0; v < 2; ++v) total[v] = wave_allreduce<AddOP>(ml < C && heard ? __builtin_bit_cast(P, w[v]) : (P)0);
+      if (ml == 0) {
+        bc[now_parity][0] = total[0];
+        bc[now_parity][1] = total[1];
+        bc[now_parity][2] = missing;
+      }
+    }
+  };
+  /* row totals from bc, then this chunk of dx and of the dg sums */
+  auto finish = [&](size_t row, int parity, V (&xv)[NV], V (&dv)[NV]) {
+    const size_t off = row * n;
+    P ss = bc[parity][0], c = bc[parity][1];
+    if (bc[parity][2] != (P)0) { /* a partner was not heard from: both sums over the whole row here */
+      patience = 0;
+      P s2 = (P)0, c2 = (P)0;
+      for (int p = lane; p < rp.npk; p += G) {
+        P u[W], d[W], g[W];
+        rp.template load<false>(x + off, p, u);
+        rp.template load<false>(dy + off, p, d);
+        rp.template load<false>(gain, p, g);
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+          s2 += u[i] * u[i];
+          c2 += d[i] * g[i] * u[i];
+        }
+      }
+      s2 = wave_allreduce<AddOP>(s2);
+      c2 = wave_allreduce<AddOP>(c2);
+      if ((lane & (WAVE - 1)) == 0) {
+        fb[0][lane / WAVE] = s2;
+        fb[1][lane / WAVE] = c2;
+      }
+      __syncthreads();
+      ss = fold_partials<AddOP, NW>(fb[0][lane & (NW - 1)]);
+      c = fold_partials<AddOP, NW>(fb[1][lane & (NW - 1)]);
+      __syncthreads(); /* fb is free again */
+    }
+    const P r = rsqrt_of(ss / (P)n + eps);
+    const P cc = c / (P)n * r * r;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+      const int p = lo + k * D + lane;
+      if (p < hi) {
+        P out[W];
+#pragma unroll
+        for (int i = 0; i < W; ++i) {
+          const P xf = (P)xv[k][i], df = (P)dv[k][i];
+          out[i] = r * (df * (P)gv[k][i] - xf * cc);
+          acc[k][i] += df * xf * r;
+        }
+        if constexpr (BLEND) {
+          P old[W];
+          rp.template load<false>(dx + off, p, old);
+#pragma unroll
+          for (int i = 0; i < W; ++i) out[i] += alpha * old[i];
+        }
+        rp.store(dx + off, p, out);
+      }
+    }
+  };
+  /* one iteration, between two barriers: row `row` (parity `parity`) is written back from `fx, fd`
+   * with the totals that came in one iteration ago, while the messenger sends the sums of row + 2
+   * (reduced from `sx, sd` just before) and reads the words of row + 1; row + 3 is asked for into
+   * `lx, ld`. The set of row + 1 is not touched. */
+  auto iteration = [&](size_t row, int parity, V (&fx)[NV], V (&fd)[NV], V (&sx)[NV], V (&sd)[NV], V (&lx)[NV], V (&ld)[NV]) {
+    const bool has_one = row + S < m, has_two = row + 2 * S < m;
+    if (row + 3 * S < m) fetch(row + 3 * S, lx, ld);
+    __builtin_amdgcn_sched_barrier(0);
+    if (has_two) sums(sx, sd, parity);
+    lds_barrier();
+    exchange(has_two, row + 2 * S, parity, has_one, row + S, parity ^ 1);
+    finish(row, parity, fx, fd);
+    lds_barrier();
+  };
+
+  V ax[NV], ad[NV], bx[NV], bd[NV], cx[NV], cd[NV], ex[NV], ed[NV];
+  if (slice < m) fetch(slice, ax, ad);
+  if (slice + S < m) fetch(slice + S, bx, bd);
+  if (slice + 2 * S < m) fetch(slice + 2 * S, cx, cd);
+#pragma unroll
+  for (int k = 0; k < NV; ++k) settle(gv[k]);
+  __syncthreads(); /* the zeroed slots */
+  if (slice < m) { /* the sums of the first two rows go out, the totals of the first come in, before the loop */
+    sums(ax, ad, 0);
+    lds_barrier();
+    exchange(true, slice, 0, false, 0, 0);
+    lds_barrier();
+    const bool has_one = slice + S < m;
+    if (has_one) sums(bx, bd, 1);
+    lds_barrier();
+    exchange(has_one, slice + S, 1, true, slice, 0);
+    lds_barrier();
+  }
+  for (size_t row = slice; row < m; row += 4 * S) { /* four rows a turn: their parities are 0, 1, 0, 1 */
+    iteration(row, 0, ax, ad, cx, cd, ex, ed);
+    if (row + S >= m) break;
+    iteration(row + S, 1, bx, bd, ex, ed, ax, ad);
+    if (row + 2 * S >= m) break;
+    iteration(row + 2 * S, 0, cx, cd, ax, ad, bx, bd);
+    if (row + 3 * S >= m) break;
+    iteration(row + 3 * S, 1, ex, ed, bx, bd, cx, cd);
+  }
+
+  P* mine = partials + slice * n;
+#pragma unroll
+  for (int k = 0; k < NV; ++k) {
+    const int p = lo + k * D + lane;
+    if (p < hi) {
+#pragma unroll
+      for (int i = 0; i < W; ++i)
+        if (i < rp.valid(p)) mine[(size_t)p * W + i] = acc[k][i];
+    }
+  }
+}
+
 /* Workgroups per row when the reverse shares rows; 0 when it does not. */
 template <class T> inline int rmsnorm_rev_cluster_size(size_t n) {
   constexpr int W = PACK_BYTES / (int)sizeof(T);
@@ -1113,7 +1365,7 @@ template <class T> inline int rmsnorm_rev_cluster_size(size_t n) {
   if (regime != REGIME_AUTO && regime != REGIME_CLUSTER) return 0;
   constexpr size_t resident = (size_t)NORM_BLOCK * max_nv_for<T>(16); /* what the resident reverse holds */
   if (regime == REGIME_AUTO && packs <= resident) return 0;
-  constexpr size_t tile = (size_t)CLUSTER_THREADS * norm_rev_cluster_nv<T>();
+  const size_t tile = norm_rev_cluster_tile<T>(packs);
   size_t ppb = (size_t)cluster_tuning().packs_per_block;
   if (ppb == 0 || ppb > tile) ppb = tile;
   const size_t c = (packs + ppb - 1) / ppb;
@@ -1510,20 +1762,31 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
   bool shared = false;
   if (!resident && C >= 1) {
     using Word = typename slot_word<P>::type;
-    size_t S = (size_t)compute_units() * norm_rev_cluster_per_cu<T>() / (size_t)C; /* every workgroup resident at once */
+    const bool deep = norm_rev_deep<T>(packs);
+    size_t S = (size_t)compute_units() * (deep ? 1 : norm_rev_cluster_per_cu<T>()) / (size_t)C; /* every workgroup resident at once */
     if (S > m) S = m;
     if (S == 0) S = 1;
     rows = (unsigned)S;
-    const int ppb = cluster_chunk_packs(packs, C, (size_t)CLUSTER_THREADS * norm_rev_cluster_nv<T>());
-    require(ppb <= CLUSTER_THREADS * norm_rev_cluster_nv<T>(), "rmsnorm reverse: cluster chunk exceeds the register tile");
+    const int ppb = cluster_chunk_packs(packs, C, norm_rev_cluster_tile<T>(packs));
+    require((size_t)ppb <= norm_rev_cluster_tile<T>(packs), "rmsnorm reverse: cluster chunk exceeds the register tile");
     Word* slots = reinterpret_cast<Word*>(partials + rmsnorm_reverse_partial_rows(m) * n);
-    if (C > 1) {
+    if (C > 1 || deep) { /* the pipelined kernel hands its sums over through the words also when a row is one chunk (test build only) */
       const size_t words = m * (size_t)C * 2;
       cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
     }
     const dim3 grid((unsigned)(S * C)), block(CLUSTER_THREADS);
-    if (blend) rmsnorm_rev_cluster<T, W, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
-    else rmsnorm_rev_cluster<T, W, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+    bool launched = false;
+    if constexpr (sizeof(T) == 4) {
+      if (deep) {
+        if (blend) rmsnorm_rev_cluster_deep<T, W, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+        else rmsnorm_rev_cluster_deep<T, W, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+        launched = true;
+      }
+    }
+    if (!launched) {
+      if (blend) rmsnorm_rev_cluster<T, W, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+      else rmsnorm_rev_cluster<T, W, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+    }
     shared = true;
   }
   if (!resident && !shared) {

@@ -43,7 +43,7 @@ def lib():
 ROW_STEMS = ("softmax_ij_j", "softmax_ij_j_reverse", "rmsnorm_ij_j", "rmsnorm_ij_j_reverse")
 ROW_SIZE_FNS = ("mpSoftmaxScratchBytes", "mpSoftmaxReverseScratchBytes", "mpRmsnormScratchBytes",
                 "mpRmsnormReverseScratchBytes")
-_diag = {"lib": None, "regime": 0, "tuned": False}
+_diag = {"lib": None, "regime": 0, "tuned": False, "deep": 0}
 
 
 def diag_lib():
@@ -65,12 +65,14 @@ def diag_lib():
         d.mpSetRowRegime.restype = None
         d.mpSetClusterTuning.argtypes = [ffi.len_t, ffi.len_t]
         d.mpSetClusterTuning.restype = None
+        d.mpSetClusterDeep.argtypes = [ffi.len_t]
+        d.mpSetClusterDeep.restype = None
         _diag["lib"] = d
     return _diag["lib"]
 
 
 def _override_active():
-    return _diag["regime"] != 0 or _diag["tuned"]
+    return _diag["regime"] != 0 or _diag["tuned"] or _diag["deep"] != 0
 
 
 def row_size(fn, dtype, m, n):
@@ -392,6 +394,13 @@ def set_cluster_tuning(packs_per_block=0, spin_limit=1 << 22):
     """Chunk size and poll limit of the shared-row kernels in the test build (defaults restore it)."""
     diag_lib().mpSetClusterTuning(int(packs_per_block), int(spin_limit))
     _diag["tuned"] = not (int(packs_per_block) == 0 and int(spin_limit) == 1 << 22)
+
+
+def set_cluster_deep(which=0):
+    """Which kernel the RMSNorm reverse runs on shared r32 rows in the test build: 0 by the launcher's
+    rule, 1 always the pipelined one, 2 never."""
+    diag_lib().mpSetClusterDeep(int(which))
+    _diag["deep"] = int(which)
 
 
 def permutate(src, dst, alpha=0.0):

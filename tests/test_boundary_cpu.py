@@ -48,11 +48,11 @@ def test_shipped_libraries_export_no_process_wide_switches():
         flags = ["-D", "--defined-only"] if name.endswith(".so") else ["--defined-only"]
         out = subprocess.run(["nm"] + flags + [os.path.join(ffi.LIB_DIR, name)],
                              capture_output=True, text=True, check=True).stdout
-        assert "mpSetRowRegime" not in out and "mpSetClusterTuning" not in out, name
+        assert "mpSetRowRegime" not in out and "mpSetClusterTuning" not in out and "mpSetClusterDeep" not in out, name
         assert "row_regime_override" not in out and "cluster_tuning" not in out, name
     diag = subprocess.run(["nm", "-D", "--defined-only", os.path.join(ffi.LIB_DIR, "libmp_kernels_diag.so")],
                           capture_output=True, text=True, check=True).stdout
-    assert " T mpSetRowRegime" in diag and " T mpSetClusterTuning" in diag
+    assert " T mpSetRowRegime" in diag and " T mpSetClusterTuning" in diag and " T mpSetClusterDeep" in diag
 
 
 def test_dispatch_arrays_are_r16_r32_r64_in_scalar_tag_order():

@@ -20,9 +20,11 @@ REGIMES = [0, 1, 2, 3, 4, 5, 6, 7, 8, 9]  # auto, G = 64..1024, stream, cluster 
 def _auto_regime():
     G.set_regime(0)
     G.set_cluster_tuning()
+    G.set_cluster_deep()
     yield
     G.set_regime(0)
     G.set_cluster_tuning()
+    G.set_cluster_deep()
     torch.cuda.synchronize()
 
 
@@ -794,6 +796,44 @@ def test_rmsnorm_reverse_cluster_path(dtype, packs, spin):
                       rowwise=False, scale=sdg)
             for gd in (x, g, dy, dx, dg, scratch):
                 gd.check("rmsnorm rev cluster")
+
+
+@pytest.mark.parametrize("packs,spin", [(0, 1 << 22), (64, 1 << 22), (64, 0), (1000, 2), (300, 1 << 22)],
+                         ids=["default", "64packs", "64packs-nowait", "1000packs-2polls", "300packs"])
+def test_rmsnorm_reverse_pipelined_shared_rows(packs, spin):
+    """The r32 kernel that publishes the sums of row j + 2 and reads the words of row j + 1 while it
+    writes back row j (four register sets, the last wavefront polling), forced onto rows of every
+    length: one to more rows than a slice gets through in four iterations, rows of one chunk, rows
+    that are not whole packs, operands off their alignment; with a poll limit of 0 or 2 workgroups
+    stop waiting and fold whole rows themselves."""
+    r = rng(68)
+    dtype = torch.float32
+    G.set_regime(CLUSTER)
+    G.set_cluster_tuning(packs, spin)
+    G.set_cluster_deep(1)
+    eps = 1e-6
+    for (m, n, shift) in [(1, 8, 0), (2, 64, 0), (3, 1000, 0), (4, 2048, 0), (5, 5000, 0), (6, 5000, 0), (7, 5000, 1),
+                          (9, 776, 0), (700, 2048, 0), (3000, 1001, 0), (2, 50264, 0), (3, 151936, 0), (3, 50257, 0),
+                          (2, 70001, 1), (33, 5000, 1)]:
+        for alpha in (0.0, 1.0):
+            G.say(f"rmsnorm rev pipelined packs={packs} spin={spin} shape=({m},{n}) shift={shift} alpha={alpha}")
+            x = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            g = G.dev(r.normal(1, 0.02, n), dtype, shift)
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            dx = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            dg = G.dev(r.normal(0, 1, n), dtype)
+            hdx, hdg = G.host(dx.t).copy(), G.host(dg.t).copy()
+            scratch, nbytes = G.rmsnorm_scratch(dtype, m, n)
+            G.rmsnorm_reverse(x.t, g.t, dy.t, dx.t, dg.t, scratch.t, eps, alpha)
+            rdx, rdg = O.rmsnorm_ij_j_reverse(G.host(x.t), G.host(g.t), G.host(dy.t), eps,
+                                              hdx if alpha else None, hdg if alpha else None, alpha)
+            sdx, sdg = G.rmsnorm_reverse_scales(G.host(x.t), G.host(g.t), G.host(dy.t), eps,
+                                                hdx if alpha else None, hdg if alpha else None, alpha)
+            G.compare(dx.t, rdx, dtype, f"rmsnorm rev pipelined dx ({m},{n}) packs {packs} spin {spin}", scale=sdx)
+            G.compare(dg.t, rdg, dtype, f"rmsnorm rev pipelined dg ({m},{n}) packs {packs} spin {spin}",
+                      rowwise=False, scale=sdg)
+            for gd in (x, g, dy, dx, dg, scratch):
+                gd.check("rmsnorm rev pipelined")
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.float64], ids=["r32", "r64"])
