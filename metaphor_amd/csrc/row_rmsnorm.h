@@ -1119,7 +1119,9 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
 constexpr int DEEP_LANES = CLUSTER_THREADS - WAVE; /* lanes of a workgroup that hold data */
 /* Which rows take it. Four-byte types only: the four register sets of r16 leave no room for its
  * dg sums, which are four times as wide as its packs (kept in LDS instead, the kernel spills
- * regardless and loses 12-21 % to the kernel above), and r64 spills. From 8193 packs a row on
+ * regardless and loses 12-21 % to the kernel above; as 512 threads at four packs a lane in 255
+ * registers it spills nothing and runs at the rate of the kernel above, -5 ... +4 %), and r64
+ * spills. From 8193 packs a row on
  * (interleaved repeats, r32: n = 50257 4.27 -> 5.10 TB/s, 65536 5.27 -> 5.44, 100352 4.74 -> 5.46,
  * 131072 4.92 -> 5.40, 151936 4.44 -> 5.27, 262144 3.99 -> 5.26; below: n = 20480 equal, 24576 5.36 ->
  * 4.77, 32768 5.53 -> 5.40). The test build can force either kernel. */
