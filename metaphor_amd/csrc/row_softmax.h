@@ -916,6 +916,13 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
    * the reverse. */
   constexpr bool FIT = sizeof(T) == 2;
   if (FIT && plan.G == 1024 && plan.NV == 2) plan = plan_row_fit(packs, MAXNV < 8 ? MAXNV : 8, 2, 16);
+  /* and r16 rows that fill a narrower group at two packs a thread to eleven sixteenths or less run
+   * on half the group at four (interleaved repeats: n = 1280 128 x 2 -> 64 x 4 5.63 -> 5.96 TB/s, 2560
+   * 256 x 2 -> 128 x 4 5.88 -> 6.11, 4608 5.51 -> 6.11, 5120 512 x 2 -> 256 x 4 5.71 -> 6.18, 5632 5.91 ->
+   * 6.06; fuller rows equal) */
+  else if (FIT && row_regime_override() == REGIME_AUTO && plan.NV == 2 && plan.G >= 128 && plan.G <= 512 && MAXNV >= 4 &&
+           packs * 16 <= (size_t)plan.G * 2 * 11)
+    plan = RowPlan{plan.G / 2, 4};
   const bool resident = for_row_plan<MAXNV, true, FIT>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
@@ -1007,7 +1014,10 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   constexpr int MAXNV = max_nv_for<T>(32);
   /* two packs a thread up to 256 packs a row, one from 512 on (interleaved repeats: r32 n = 2048
    * 512 x 1 6.25 TB/s against 256 x 2 5.95, r16 n = 4096 6.37 against 6.15, n = 8192 6.40 against 6.27) */
-  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, packs >= 512 ? 1 : 2, 16);
+  /* a pack a thread from 512 packs a row on; r16 rows of up to 768 packs stay at two on 512 threads
+   * rather than one on a 1024-thread group they fill to three quarters or less (interleaved repeats:
+   * n = 4608 5.23 -> 6.06 TB/s, 5120 5.51 -> 6.16, 5632 5.82 -> 6.16, 6144 and 6656 equal) */
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, packs >= (sizeof(T) == 2 ? 769 : 512) ? 1 : 2, 16);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) {

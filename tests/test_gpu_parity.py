@@ -479,6 +479,39 @@ def test_softmax_forward_r16_rows_held_at_three_or_five_packs_a_thread():
             y.check("y")
 
 
+def test_softmax_r16_rows_on_half_the_group():
+    """r16 rows that would fill a group at two packs a thread to eleven sixteenths or less run on half
+    the group at four (forward: n = 1280, 2560, 2816, 5120, 5632), and rows of 513 ... 768 packs stay at
+    two packs a thread on 512 threads in the reverse; with a ragged end and one element off alignment;
+    forward (masked and plain) and reverse (both blends) against the oracle."""
+    r = rng(37)
+    dtype = torch.float16
+    for (m, n, shift) in [(9, 1280, 0), (9, 2560, 0), (5, 2816, 0), (7, 5120, 0), (5, 5632, 0), (3, 6144, 0),
+                          (5, 5121, 0), (5, 5120, 1), (4, 2563, 1), (300, 4608, 0)]:
+        for masked in (False, True):
+            G.say(f"softmax r16 half group ({m},{n}) shift={shift} masked={masked}")
+            x = G.dev(_softmax_inputs(r, m, n, dtype, masked), dtype, shift)
+            y = G.Guarded((m, n), dtype, shift)
+            G.softmax(x.t, y.t)
+            G.compare(y.t, O.softmax_ij_j(G.host(x.t)), dtype, f"softmax r16 half group ({m},{n})", **G.softmax_tol(dtype))
+            if masked:
+                assert bool((y.t[torch.isinf(x.t)] == 0).all())
+            x.check("x")
+            y.check("y")
+        for alpha in (0.0, 0.5):
+            G.say(f"softmax rev r16 half group ({m},{n}) shift={shift} alpha={alpha}")
+            yv = G.dev(O.softmax_ij_j(_softmax_inputs(r, m, n, dtype, False)), dtype, shift)
+            dy = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            dx = G.dev(r.normal(0, 1, (m, n)), dtype, shift)
+            before = G.host(dx.t).copy()
+            G.softmax_reverse(yv.t, dy.t, dx.t, alpha)
+            ref = O.softmax_ij_j_reverse(G.host(yv.t), G.host(dy.t), before if alpha else None, alpha)
+            scale = G.softmax_reverse_scale(G.host(yv.t), G.host(dy.t), before if alpha else None, alpha)
+            G.compare(dx.t, ref, dtype, f"softmax rev r16 half group ({m},{n}) alpha {alpha}", scale=scale)
+            for g in (yv, dy, dx):
+                g.check("softmax rev r16 half group")
+
+
 def test_softmax_long_rows_without_scratch_take_the_two_pass_kernel():
     r = rng(33)
     for (m, n) in [(3, 151936), (4, 50257)]:
