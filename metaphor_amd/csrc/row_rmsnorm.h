@@ -1620,6 +1620,18 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
    * (interleaved repeats: r16 n = 1152 4.44 -> 5.31 TB/s, 1280 4.99 -> 5.74, 2560 5.20 -> 5.86; r32
    * n = 576 5.20 -> 6.14, 640 5.57 -> 6.22, 1280 5.84 -> 6.19; one-shot workgroups of the same groups: -4 ... +7 %;
    * six wavefronts a row: -2 ... +2 %, left with the power-of-two groups) */
+  /* r16 rows of 129 ... 223 packs (128 x 2 planned): persistent workgroups of eight such rows that load
+   * after they have written beat both the wavefront-group kernel and one-shot workgroups there
+   * (interleaved repeats: n = 1152 4.78 -> 5.34 TB/s, 1280 5.06 -> 5.54, 1408 5.21 -> 5.68, 1536 5.42 -> 5.71) */
+  const bool eight_rows = !loose && !mismatch && sizeof(T) == 2 && row_regime_override() == REGIME_AUTO &&
+                          shot.G == 128 && shot.NV == 2 && packs > 128 && packs * 8 < (size_t)shot.G * shot.NV * 7;
+  if (eight_rows) {
+    const size_t need = (m + NORM_BLOCK / 128 - 1) / (NORM_BLOCK / 128);
+    const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
+    rmsnorm_fwd_resident<T, W, 128, 2, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+    MP_CHECK_LAUNCH();
+    return;
+  }
   if (!loose && !mismatch && row_regime_override() == REGIME_AUTO && shot.G >= 128 && shot.G <= 512 && shot.NV <= 2 &&
       packs * 8 < (size_t)shot.G * shot.NV * 7) {
     const int gw = (int)((packs + (size_t)WAVE * shot.NV - 1) / ((size_t)WAVE * shot.NV));
@@ -1688,6 +1700,15 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
    * one pack a thread the wide group stays (n = 3072: 1024 x 1 6.00 against 256 x 3 5.85), and the
    * forward loses by the same change at every length tried (n = 5120: 5.68 -> 5.49) */
   if (plan.NV >= 2) plan = plan_row_fit(packs, MAXNV, 1, 8);
+  /* aligned r32 rows of 129 ... 239 and 257 ... 479 packs: 128-thread groups at two or four packs a
+   * thread, eight rows a workgroup (two packs: the paired kernel; four: the unpaired one, two
+   * workgroups a CU), not a group of twice or four times the width at a pack a thread that they
+   * would not fill (interleaved repeats against that and the wavefront-group kernel: n = 704 5.65 ->
+   * 5.83 TB/s, 832 5.74 -> 5.98, 1152 5.43 -> 5.93, 1408 5.62 -> 5.95, 1664 5.21 -> 5.90, 1792 5.53 -> 5.85;
+   * rows that fill the wide group lose, n = 1024 6.03 -> 5.82, 2048 6.02 -> 5.57, and keep it) */
+  if (!LOOSE && sizeof(T) == 4 && !force_shared && row_regime_override() == REGIME_AUTO && packs > 128 && packs <= 512 && MAXNV >= 4 &&
+      packs * 16 < (size_t)(packs <= 256 ? 256 : 512) * 15)
+    plan = RowPlan{128, packs <= 256 ? 2 : 4};
   const bool resident = for_row_plan<MAXNV, true, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     /* two register sets of x and dy beside the gain and the dg sums: up to eight registers an array
@@ -1720,7 +1741,11 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
     }
     if constexpr (!LOOSE && (G == 512 || G == 256) && NV == 1 && pairs_fit) {
       const int gw = (int)((packs + WAVE - 1) / WAVE);
-      if (row_regime_override() == REGIME_AUTO && packs * 8 < (size_t)G * 7 && gw >= NORM_BLOCK / WAVE / ANY_MAX_ROWS) {
+      /* r16: only rows that fill the group to less than eleven sixteenths; fuller ones are better off on
+       * the power-of-two group since it keeps three register sets (n = 1536: 5.55 -> 6.03 TB/s, 3072:
+       * 5.79 -> 6.05) */
+      const bool idle_enough = sizeof(T) == 2 ? packs * 16 < (size_t)G * 11 : packs * 8 < (size_t)G * 7;
+      if (row_regime_override() == REGIME_AUTO && idle_enough && gw >= NORM_BLOCK / WAVE / ANY_MAX_ROWS) {
         const int rpb = NORM_BLOCK / (gw * WAVE);
         const size_t need_any = (m + rpb - 1) / rpb, one_per_cu = (size_t)compute_units();
         rows = (unsigned)(need_any < one_per_cu ? need_any : one_per_cu);

@@ -902,8 +902,10 @@ def test_rmsnorm_reverse_rows_held_at_three_packs_a_thread(dtype):
 def test_rmsnorm_reverse_rows_on_three_to_six_wavefronts(dtype):
     """Rows of 129 ... 223, 257 ... 447 and (at two packs a thread) 513 ... 896 packs (r16 n = 1280, 2560,
     3072, 5120, 7168; r32 n = 640, 1280, 1536, 2560, 3584): three to seven wavefronts a row, five to two
-    rows a workgroup. Whole problem against the oracle, both blends, row counts that are not a
-    multiple of the rows a workgroup holds, and one that leaves workgroups idle."""
+    rows a workgroup; r32 rows of up to 479 packs run on 128-thread groups at two or four packs a
+    thread instead, r16 rows that fill a power-of-two group to eleven sixteenths or more on that
+    group. Whole problem against the oracle, both blends, row counts that are not a multiple of the
+    rows a workgroup holds, and one that leaves workgroups idle."""
     r = rng(67)
     per_pack = 16 // torch.empty((), dtype=dtype).element_size()
     for packs in (129, 160, 223, 257, 320, 384, 447, 513, 640, 832, 895, 896):
