@@ -601,7 +601,7 @@ template <class T> inline int cluster_size(size_t packs) {
   /* up to two packs per thread a resident workgroup is the better kernel; measured exceptions: r32
    * rows of exactly 2048 packs (n = 8192: 5.8 resident, 6.1 here), and r16 chunks want the whole
    * register tile (n = 49152: 5.4 -> 5.7 TB/s) where r32 is better one pack per thread below it */
-  const size_t resident = (size_t)CLUSTER_THREADS * 2 - (sizeof(T) >= 4 ? 1 : 0);
+  const size_t resident = (size_t)CLUSTER_THREADS * 2 - (sizeof(T) == 4 ? 1 : 0); /* r64 at 2048 packs: 3.66 here, 5.8 resident */
   if (regime == REGIME_AUTO && packs <= resident) return 0;
   /* r32 rows of 32 ... 64 KiB stay with one workgroup of 1024 threads at four packs a thread
    * (interleaved repeats, 2^28 elements: n = 12288 6.12 TB/s against 5.94 shared, 16384 equal; above,
