@@ -26,13 +26,15 @@ sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0
 SETS = {"cfg1": 16, "cfg2": 4, "cfg3": 2, "cfg4": 2, "cfg5a": 3, "cfg5b": 3, "copy": 2, "permutate": 2, "gemm": 2,
-        "chain": 2}
+        "chain": 2, "normvocab": 3}
+ON_REQUEST = {"normvocab"}  # workloads outside BASELINE's configurations: run with --workload, not beside the headline
 MFMA_PEAK_TFLOPS = {"gemm": 2500.0}  # dense fp16 matrix rate of the MI355X
 
 
 PROFILE_OF = {"cfg1": "cfg1_softmax", "cfg2": "cfg2_rmsnorm", "cfg3": "cfg3_softmax_r16",
               "cfg4": "cfg4_fused_chain", "cfg5a": "cfg5a_softmax_vocab", "cfg5b": "cfg5b_softmax_vocab",
-              "permutate": "permutate_transpose", "gemm": "gemm_rocblas_r16"}
+              "permutate": "permutate_transpose", "gemm": "gemm_rocblas_r16",
+              "chain": "chain_runtime_fused", "normvocab": "normvocab_rmsnorm_shared_rows"}
 
 
 def traffic_from_profile(name, direction=None):
@@ -443,7 +445,7 @@ def main():
     if not args.no_extra:
         extra = {}
         for other in sorted(SETS):
-            if other == name:
+            if other == name or other in ON_REQUEST:
                 continue
             osets = make_sets(other)
             o = osets[0]

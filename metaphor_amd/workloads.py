@@ -409,7 +409,21 @@ class Gemm(Workload):
         inner_product("ji_jk_ik", self.a, self.gc, 1.0, self.gb, 1.0, n, m, k)
 
 
-WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b, Copy, Permutate, Gemm, RuntimeChain)}
+class NormVocab(Cfg2):
+    """RMSNorm over rows as long as cfg5a's: every row shared by several workgroups, in both
+    directions (no BASELINE configuration; here so that those kernels can be traced)."""
+    name = "normvocab"
+    shape = (512, 151936)
+
+    def __init__(self, seed=0, shape=None):
+        super().__init__(seed, shape)
+        self.fwd_scratch = rmsnorm_scratch(torch.float32, *self.shape)
+
+    def forward(self):
+        rmsnorm_forward(self.x, self.gain, self.y, self.eps, self.fwd_scratch)
+
+
+WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b, Copy, Permutate, Gemm, RuntimeChain, NormVocab)}
 
 DESCRIPTION = {
     "cfg1": "softmax fwd r32 [256,1024]",
@@ -419,6 +433,7 @@ DESCRIPTION = {
     "cfg5a": "vocabulary softmax fwd (+rev) r32 [512,151936]",
     "cfg5b": "vocabulary softmax fwd (+rev) r32 [2048,50257]",
     "chain": "relu((a-b)*(c+d)) fwd+rev r32 flat 2^28, an expression no build listed, compiled at run time",
+    "normvocab": "RMSNorm fwd+rev r32 [512,151936]: rows shared by several workgroups (not a BASELINE configuration)",
     "copy": "plain copy r32 flat 2^28 (calibration)",
     "permutate": "transpose r32 [16384,16384], reverse = accumulating transpose",
     "gemm": "matrix product r16 (fp32 accumulate) 8192^3 on rocBLAS, reverse = its two gradient products",
