@@ -310,8 +310,11 @@ __global__ __launch_bounds__(LANES * SLICES) void reduce_cols_kernel(
 constexpr size_t SHORT_MATRIX_ROWS = 256; /* up to here the column sum takes four slices a workgroup */
 
 /* Lanes (packs) of a row per workgroup: as many as a narrow matrix has, so that no lane idles
- * (measured on r32 [4M, 4]: 0.4 TB/s with 8 lanes); 8 lanes x one pack = 128 bytes, one cache
- * line, of every aligned row (many strips, so narrow matrices still spread); a wavefront per
+ * (measured on r32 [4M, 4]: 0.4 TB/s with 8 lanes); 32 lanes x one pack = 512 bytes of every
+ * aligned row of a wider one: strips of one 128-byte line a row, the first choice, leave a
+ * quarter of what the memory gives on the table (interleaved repeats, 8 -> 32 lanes: r32
+ * [16384, 16384] 5.47 -> 6.43 TB/s, [65536, 4096] 5.76 -> 6.16, [262144, 1024] 5.60 -> 6.43; r16 5.32 -> 6.06,
+ * 5.29 -> 5.93, 5.13 -> 6.10; 64 lanes: the same for r32, r16 [65536, 4096] 4.05); a wavefront per
  * kilobyte of a row for wide rows that are not aligned, because a misaligned 128-byte segment
  * would touch two lines for the data of one (measured on r32 [20000, 50257]: 3.4 TB/s with 8
  * lanes, one element per lane 4.3). */
@@ -322,9 +325,9 @@ template <class T> inline size_t reduce_cols_lanes(size_t n, bool loose) {
   if (packs <= 2) return 2;
   if (packs <= 4) return 4;
   if (packs <= 8) return 8;
-  if (loose && packs <= 16) return 16;
-  if (loose && packs <= 32) return 32;
-  return loose ? 64 : 8;
+  if (packs <= 16) return 16;
+  if (packs <= 32) return 32;
+  return loose ? 64 : 32;
 }
 
 /* Row chunks of the two-stage column sum: enough workgroups to fill the GPU when the matrix is
@@ -390,12 +393,22 @@ inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, do
     MP_CHECK_LAUNCH();
     return;
   }
-  const size_t lanes = reduce_cols_lanes<T>(n, loose); /* under 8 lanes the kernel is always the loose one */
-  const size_t blocks = ((n + W - 1) / W + lanes - 1) / lanes;
+  size_t lanes = reduce_cols_lanes<T>(n, loose); /* other than 8 lanes the kernel is always the loose one */
+  size_t blocks = ((n + W - 1) / W + lanes - 1) / lanes;
   require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
   size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;
   const size_t fit = scratch_bytes / (n * sizeof(P)); /* partial rows the workspace holds */
   if (chunks > fit) chunks = fit;
+  /* without a workspace the strips are all the workgroups there are: an aligned matrix too narrow
+   * to give every CU one at 32 lanes goes back to strips of a line */
+  const bool too_few = chunks <= 1 && blocks < (size_t)compute_units();
+  /* and the weighted sum of r16 rows keeps them as well (a vector times an r16 matrix, 32 lanes against 8:
+   * [16384, 16384] 5.32 -> 4.95 TB/s, [65536, 4096] 5.23 -> 4.76; r32 gains there like the plain sum) */
+  const bool weighted_r16 = weight != nullptr && sizeof(T) == 2;
+  if (!loose && lanes == 32 && (too_few || weighted_r16)) {
+    lanes = 8;
+    blocks = ((n + W - 1) / W + lanes - 1) / lanes;
+  }
   if (chunks > 1) {
     const size_t chunk = (m + chunks - 1) / chunks;
     P* partials = static_cast<P*>(scratch);
