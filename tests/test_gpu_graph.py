@@ -31,6 +31,16 @@ def test_replays_of_a_captured_forward_and_reverse_sequence_match_eager():
     p, dp, dl = torch.empty_like(logits), rnd(lm, ln), torch.empty_like(logits)
     fs, rs = W.softmax_scratch(f32, lm, ln), W.softmax_reverse_scratch(f32, lm, ln)
     assert fs is not None and rs is not None
+    # RMSNorm over the same long rows: the shared-row forward and the pipelined shared-row reverse
+    lgain = 1 + 0.02 * rnd(ln)
+    ly, ldx, ldg = torch.empty_like(logits), torch.empty_like(logits), torch.empty_like(lgain)
+    lf, lr = W.rmsnorm_scratch(f32, lm, ln), W.rmsnorm_reverse_scratch(f32, lm, ln)
+    assert lf is not None
+    # column sums of a tall matrix through a workspace (partial rows, then the fixed-order finish)
+    tall = rnd(3000, 512)
+    sums = torch.empty(512, device="cuda", dtype=f32)
+    kernels, _ = G.lib()
+    cs = torch.empty(max(int(kernels.mpReduceScratchBytes(G.KEY[f32], 3000, 512)), 16), dtype=torch.uint8, device="cuda")
     a, b, c, d = (torch.rand(10007, generator=gen, device="cuda", dtype=f32) * 4 - 2 for _ in range(4))
     e = torch.empty_like(a)
     # an expression compiled at run time: its first (eager) call compiles and loads it, which a
@@ -46,11 +56,14 @@ def test_replays_of_a_captured_forward_and_reverse_sequence_match_eager():
         W.rmsnorm_reverse(x, gain, dy, dx, dg, nscratch, 1e-6)
         W.softmax_forward(logits, p, fs)
         W.softmax_reverse(p, dp, dl, 0.0, rs)
+        W.rmsnorm_forward(logits, lgain, ly, 1e-6, lf)
+        W.rmsnorm_reverse(logits, lgain, dp, ldx, ldg, lr, 1e-6)
+        W._launch("reduce_ij_j_scratch", f32, tall.data_ptr(), sums.data_ptr(), cs.data_ptr(), 0.0, 3000, 512)
         W.fused_forward(a, b, c, d, e)
         assert G.chain_forward(chain, [a, b, c, d], e2) == 0, G.chain_error()
         assert G.chain_reverse(chain, [a, b, c, d], up, grads, 0.0) == 0, G.chain_error()
 
-    outputs = (y, dx, dg, p, dl, e, e2, *grads)
+    outputs = (y, dx, dg, p, dl, ly, ldx, ldg, sums, e, e2, *grads)
     G.say("eager sequence")
     sequence()
     torch.cuda.synchronize()
