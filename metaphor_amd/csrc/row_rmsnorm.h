@@ -1171,7 +1171,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS) void rmsnorm_rev_cluster_deep(
     const int p = lo + k * D + lane;
     gv[k] = p < hi ? rp.template raw<false>(gain, p) : V{};
   }
-  if (lane < 2 * NW) (&red[0][0][0])[lane] = (&red[1][0][0])[lane] = (P)0;
+  if (lane < NW) red[0][0][lane] = red[0][1][lane] = red[1][0][lane] = red[1][1][lane] = (P)0;
 
   auto fetch = [&](size_t row, V (&xs)[NV], V (&ds)[NV]) {
     const size_t off = row * n;
