@@ -1014,12 +1014,15 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   constexpr int MAXNV = max_nv_for<T>(32);
   /* two packs a thread up to 256 packs a row, one from 512 on (interleaved repeats: r32 n = 2048
    * 512 x 1 6.25 TB/s against 256 x 2 5.95, r16 n = 4096 6.37 against 6.15, n = 8192 6.40 against 6.27) */
+  const bool one_pack = sizeof(T) == 2 ? (packs > 400 && packs <= 512) || packs > 768 : packs >= (sizeof(T) == 4 ? 129 : 512);
   /* a pack a thread from 512 packs a row on (r32: from 129; interleaved repeats against two packs on
    * half the group: n = 576 5.90 -> 6.23 TB/s, 832 5.67 -> 6.16, 1152 5.93 -> 6.25, 1408 5.89 -> 6.31, 1536
-   * 5.93 -> 6.20); r16 rows of up to 768 packs stay at two on 512 threads
+   * 5.93 -> 6.20); r16 rows of 513 ... 768 packs stay at two on 512 threads
    * rather than one on a 1024-thread group they fill to three quarters or less (interleaved repeats:
-   * n = 4608 5.23 -> 6.06 TB/s, 5120 5.51 -> 6.16, 5632 5.82 -> 6.16, 6144 and 6656 equal) */
-  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, packs >= (sizeof(T) == 2 ? 769 : sizeof(T) == 4 ? 129 : 512) ? 1 : 2, 16);
+   * n = 4608 5.23 -> 6.06 TB/s, 5120 5.51 -> 6.16, 5632 5.82 -> 6.16, 6144 and 6656 equal), and r16 rows of
+   * 401 ... 512 packs take one pack on 512 threads (against two on 256: n = 3584 6.02 -> 6.25, 3840 5.98 ->
+   * 6.46, 4096 6.10 -> 6.33; 3328 equal, 3072 better at two) */
+  const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, one_pack ? 1 : 2, 16);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (ragged) {
