@@ -665,7 +665,7 @@ def test_softmax_short_rows_any_length_and_alignment(dtype):
 # ------------------------------------------------------------------ RMSNorm
 
 NORM_SHAPES = [(1, 1), (3, 7), (17, 64), (1031, 16), (259, 128), (33, 256), (64, 4096), (5, 1000), (300, 1024), (3, 50257),
-               (2, 70001), (1025, 128), (40, 8192), (3, 32768), (2, 300000), (2051, 8), (515, 32)]
+               (2, 70001), (1025, 128), (40, 8192), (5, 16384), (3, 32768), (2, 300000), (2051, 8), (515, 32)]
 
 
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
