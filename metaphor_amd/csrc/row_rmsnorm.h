@@ -1723,7 +1723,8 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
      * (interleaved repeats: r16 n = 1152 4.01 -> 4.72 TB/s, 1280 4.59 -> 5.17, 2560 4.30 -> 5.43, 3072
      * 5.03 -> 5.48; r32 n = 576 4.78 -> 5.39, 1280 5.09 -> 5.50, 1536 5.40 -> 5.95). Wider rows gain nothing
      * from shedding their idle wavefronts (n = 5120 r16: 4.80 -> 4.87, with two such workgroups a CU
-     * 4.73) and keep the power-of-two groups. */
+     * 4.73) and keep the power-of-two groups. Aligned r32 rows of these lengths no longer come here:
+     * the plan above puts them on 128-thread groups, which beat this path in turn. */
     /* rows of 513 ... 896 packs on one 1024-thread group at a pack a thread: five to seven wavefronts
      * a row at two packs a thread and three or two rows a workgroup. r32 and r64 hold the widened
      * packs; r16 would not fit them twice over, so the kernel keeps x, dy and gain as loaded and
