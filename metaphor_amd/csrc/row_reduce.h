@@ -317,7 +317,8 @@ constexpr size_t SHORT_MATRIX_ROWS = 256; /* up to here the column sum takes fou
  * 5.29 -> 5.93, 5.13 -> 6.10; 64 lanes: the same for r32, r16 [65536, 4096] 4.05); a wavefront per
  * kilobyte of a row for wide rows that are not aligned, because a misaligned 128-byte segment
  * would touch two lines for the data of one (measured on r32 [20000, 50257]: 3.4 TB/s with 8
- * lanes, one element per lane 4.3). */
+ * lanes, one element per lane 4.3); two-byte types stay at 32 lanes there as well (64 -> 32: r16
+ * [20000, 50257] 4.76 -> 4.92 TB/s, [65536, 4099] 4.25 -> 4.88; r32 loses 6-11 % by it). */
 template <class T> inline size_t reduce_cols_lanes(size_t n, bool loose) {
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   const size_t packs = (n + W - 1) / W;
@@ -327,7 +328,7 @@ template <class T> inline size_t reduce_cols_lanes(size_t n, bool loose) {
   if (packs <= 8) return 8;
   if (packs <= 16) return 16;
   if (packs <= 32) return 32;
-  return loose ? 64 : 32;
+  return loose && sizeof(T) >= 4 ? 64 : 32;
 }
 
 /* Row chunks of the two-stage column sum: enough workgroups to fill the GPU when the matrix is
