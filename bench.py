@@ -1,18 +1,30 @@
 #!/usr/bin/env python3
 """Benchmark of the row-reduction / elementwise hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload cfg2] [--no-extra] [--no-cpu] [--no-ceilings]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--regions R] [--workload cfg2]
+                    [--no-extra] [--no-cpu] [--no-ceilings] [--strict]
 
 A step is one pass of the hot path over one batch of the headline workload (cfg2: RMSNorm
 forward + reverse, r32, [8192, 4096]) with all inputs resident in HBM. Successive steps
 rotate over several buffer sets, and the reverse of a step works on a different set than its
-forward, so the 256 MiB memory-side cache cannot serve repeats. One JSON line is printed:
-whole-step throughput (`value`, GB/s of algorithmic bytes), the roofline of the dominant
-launcher measured with events on the launch stream inside the timed region, the CPU oracle
-timed on the host cores with the measured parity of the GPU results against it, and (unless
---no-extra) forward/reverse rates and roofline objects of the other workloads. Every roofline
-object also carries the rate of a plain pass with the same reads, writes and footprint
-(`copy_ceiling`, from lib/libmp_probe.so), timed in the same run.
+forward, so the 256 MiB memory-side cache cannot serve repeats.
+
+Timing: W untimed warm-up steps, then a pre-warm of the same steps for a stated wall time (a
+GPU that has idled runs its first milliseconds below its sustained clocks; `prewarm_ms` and
+`prewarm_steps` are in the line), then R regions of EXACTLY K steps each, every region bracketed
+by synchronisations. `value` is the median region's K * bytes / time, `ms_per_step` that
+region's time / K; all R per-region values are in the line (`region_values_GBps`), the first
+among them. Inside each region one launch of the dominant launcher is bracketed by a pair of
+events on the launch stream (`in_region_launch_ms`: it includes the cost of the pair itself,
+2-3 us); the roofline object's launch duration comes from groups of 8 back-to-back launches of
+that launcher between one pair, timed right after the regions, which takes the pair's cost out.
+
+One JSON line is printed: whole-step throughput, the roofline of the dominant launcher, and for
+every workload its forward/reverse rates, roofline objects, the CPU oracle timed on the host
+cores over a bounded sample of the same inputs, and the measured parity of the GPU results
+against that oracle on the sample. Every roofline object also carries the rate of a plain pass
+with the same reads, writes and footprint (`copy_ceiling`, from lib/libmp_probe.so), timed in
+the same run.
 """
 import argparse
 import json
@@ -70,66 +82,87 @@ def make_sets(name, count=None):
     return [W.WORKLOADS[name](seed=i) for i in range(count or SETS[name])]
 
 
-EVENT_EVERY = 8  # a pair of events costs ~2-5 us of stream time: sample launches, not every one
+BATCH = 8  # launches between a pair of events: a pair costs 2-3 us of stream time, shared by the group
 
 
-def time_steps(sets, steps, warmup):
-    """K timed steps. Returns (seconds, durations in ms of the dominant launcher sampled with
-    events inside the timed region on the launch stream)."""
+def _step(sets, i):
+    S = len(sets)
+    sets[i % S].forward()
+    if sets[0].has_reverse:
+        sets[(i + S // 2) % S].reverse()
+
+
+def time_regions(sets, steps, warmup, regions=7, prewarm_s=0.25):
+    """W warm-up steps, a pre-warm of the same steps for prewarm_s of wall time, then `regions`
+    regions of exactly `steps` steps, each between two synchronisations. Returns the list of
+    region times in seconds, the durations in ms of the one launch of the dominant launcher
+    bracketed by events inside each region, and what the pre-warm took."""
     import torch
     S = len(sets)
-    rev_of = lambda i: sets[(i + S // 2) % S]
     has_rev = sets[0].has_reverse
     for s in sets:  # every set's forward output exists before any reverse consumes it
         s.forward()
     for i in range(warmup):
-        sets[i % S].forward()
-        if has_rev:
-            rev_of(i).reverse()
-    every = EVENT_EVERY if steps >= 4 * EVENT_EVERY else 1
-    sampled = list(range(0, steps, every))
-    ev = {i: _events(2) for i in sampled}
+        _step(sets, i)
     torch.cuda.synchronize()
-    t0 = time.perf_counter()
-    for i in range(steps):
-        if has_rev:
-            sets[i % S].forward()
-            if i in ev:
-                ev[i][0].record()
-            rev_of(i).reverse()
-            if i in ev:
-                ev[i][1].record()
-        else:
-            if i in ev:
-                ev[i][0].record()
-            sets[i % S].forward()
-            if i in ev:
-                ev[i][1].record()
-    torch.cuda.synchronize()
-    dt = time.perf_counter() - t0
-    return dt, [ev[i][0].elapsed_time(ev[i][1]) for i in sampled]
+    t0, n_pre = time.perf_counter(), 0
+    while time.perf_counter() - t0 < prewarm_s:
+        for i in range(steps):
+            _step(sets, i)
+        torch.cuda.synchronize()
+        n_pre += steps
+    prewarm = {"prewarm_ms": round((time.perf_counter() - t0) * 1e3, 1), "prewarm_steps": n_pre}
+    times, pairs = [], []
+    mid = steps // 2
+    for _ in range(regions):
+        a, b = _events(2)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(steps):
+            if i != mid:
+                _step(sets, i)
+            elif has_rev:
+                sets[i % S].forward()
+                a.record()
+                sets[(i + S // 2) % S].reverse()
+                b.record()
+            else:
+                a.record()
+                sets[i % S].forward()
+                b.record()
+        torch.cuda.synchronize()
+        times.append(time.perf_counter() - t0)
+        pairs.append((a, b))
+    return times, [a.elapsed_time(b) for a, b in pairs], prewarm
 
 
-def time_each(sets, iters):
-    """Per-launcher medians outside the headline region: (forward ms list, reverse ms list)."""
+def time_each(sets, iters, batch=BATCH):
+    """Per-launch durations in ms of the forward and of the reverse launcher: groups of `batch`
+    back-to-back launches (rotating over the buffer sets) between one pair of events, one value
+    per group. A reverse works on the set half a rotation away from the last forward's."""
     import torch
     S = len(sets)
     has_rev = sets[0].has_reverse
+    groups = max(3, iters // batch)
     fwd, rev = [], []
-    for i in range(iters):
+    k = 0
+    for _ in range(groups):
         a, b = _events(2)
         a.record()
-        sets[i % S].forward()
+        for _ in range(batch):
+            sets[k % S].forward()
+            k += 1
         b.record()
         fwd.append((a, b))
         if has_rev:
             c, d = _events(2)
             c.record()
-            sets[(i + S // 2) % S].reverse()
+            for j in range(batch):
+                sets[(k + j + S // 2) % S].reverse()
             d.record()
             rev.append((c, d))
     torch.cuda.synchronize()
-    return [a.elapsed_time(b) for a, b in fwd], [a.elapsed_time(b) for a, b in rev]
+    return [a.elapsed_time(b) / batch for a, b in fwd], [a.elapsed_time(b) / batch for a, b in rev]
 
 
 def graph_forward_ms(sets, replays=50):
@@ -208,8 +241,12 @@ def roofline_of(name, direction, nbytes, launch_ms, ceiling=None):
            "frac": round(achieved / HBM_PEAK_GBPS, 4),
            "traffic": traffic_from_profile(name, direction),
            "kernel": f"{name} {direction} launcher", "bytes_per_launch": nbytes,
-           "avg_launch_ms": round(avg_ms, 5), "launches_timed": len(kept),
-           "host_stalls_dropped": len(launch_ms) - len(kept)}
+           "avg_launch_ms": round(avg_ms, 5), "launches_timed": len(kept) * BATCH,
+           "timing": f"{len(kept)} groups of {BATCH} back-to-back launches, one event pair a group",
+           "host_stalls_dropped": len(launch_ms) - len(kept),
+           # nothing filtered: every group counts, the slowest one shown
+           "avg_launch_ms_all": round(sum(launch_ms) / len(launch_ms), 5),
+           "max_launch_ms": round(max(launch_ms), 5)}
     if ceiling:
         out["copy_ceiling"] = ceiling
         out["frac_of_copy_ceiling"] = round(achieved / ceiling["GBps"], 4)
@@ -237,12 +274,12 @@ def probe_lib():
     return _probe["lib"]
 
 
-def copy_ceiling(mix, stream_bytes, iters=20, row_pairs=None):
+def copy_ceiling(mix, stream_bytes, iters=24, row_pairs=None):
     """Rate of a plain pass that reads mix[0] streams and writes mix[1] streams of stream_bytes
     each: one-shot workgroups of 64 and of 256 threads, a 16-byte pack per lane and stream, and
     (row_pairs = (rows, workgroups), 16 KiB rows) the structure of the paired RMSNorm reverse
     without its arithmetic. Buffer sets rotate so that the memory-side cache cannot serve a
-    repeat; timed like the launchers, one event pair per launch, median. Best shape is reported."""
+    repeat; timed like the launchers (groups of back-to-back launches between one event pair), median. Best shape is reported."""
     import ctypes
     import torch
     from metaphor_amd import ffi
@@ -261,15 +298,17 @@ def copy_ceiling(mix, stream_bytes, iters=20, row_pairs=None):
     def run(tag, launch):
         for i in range(3):
             launch(bufs[i % sets])
-        pairs = []
-        for i in range(iters):
+        pairs, k = [], 0
+        for _ in range(max(3, iters // BATCH)):  # timed like the launchers: groups of back-to-back launches
             a, b = _events(2)
             a.record()
-            launch(bufs[i % sets])
+            for _ in range(BATCH):
+                launch(bufs[k % sets])
+                k += 1
             b.record()
             pairs.append((a, b))
         torch.cuda.synchronize()
-        ms = _median([a.elapsed_time(b) for a, b in pairs])
+        ms = _median([a.elapsed_time(b) / BATCH for a, b in pairs])
         shapes[tag] = round((nr + nw) * stream_bytes / (ms * 1e-3) / 1e9, 1)
 
     for block in (64, 256):
@@ -309,54 +348,140 @@ def ceilings_for(w):
     return fwd, rev
 
 
-def cpu_baseline_cfg2(w, budget_s=12.0):
-    """The fp64 oracle on the host cores over the same bytes: whole cfg2 passes (forward, then
-    the row-parallel reverse) until about `budget_s` seconds are spent. Also returns the
-    parity of the GPU results of this buffer set against that oracle."""
+def _numbers(got, ref, dtype, rowwise=True, scale=None, atol=None):
+    """n, max_abs, max_rel, violations of one comparison under this path's bound (tests/gpu_lib.py)."""
+    import gpu_lib as G
+    st = G.parity_stats(got, ref, dtype, rowwise=rowwise, scale=scale, atol=atol)
+    return {"n": st["n"], "max_abs": float(f"{st['max_abs']:.3e}"), "max_rel": float(f"{st['max_rel']:.3e}"),
+            "violations": st["violations"]}
+
+
+BOUND_TEXT = {
+    "r32": "|got - ref| <= 1e-5 * max(|ref|, RMS(ref row or tensor)); softmax outputs: <= 1e-6 absolute",
+    "r16": "|got - ref| <= 2e-3 * max(|ref|, RMS(ref row)) + 2^-24",
+}
+
+
+def cpu_and_parity(name, w, budget_s):
+    """The fp64 oracle (oracle/mp_oracle.c, OpenMP) on the host cores over a bounded sample of the
+    workload's own input bytes, repeated until about budget_s seconds are spent, and the measured
+    parity of the GPU results of this buffer set against the oracle on that sample. The sample:
+    cfg1 and cfg2 whole; cfg3 the first four 2048-row blocks; cfg4 / chain the first 2^22 elements;
+    cfg5a the first 32 rows, cfg5b the first 96. Returns (cpu_baseline, parity); every comparison
+    also raises when an entry is outside its bound."""
     import numpy as np
     import oracle_lib as O
     import gpu_lib as G
     import torch
 
-    cores = min(O.threads(), 16)
-    O.set_threads(cores)
-    x, g, dy = w.x.cpu().numpy(), w.gain.cpu().numpy(), w.dy.cpu().numpy()
-    passes, spent = 0, 0.0
+    avail = os.cpu_count() or 1
+    used = min(O.threads(), avail)  # OMP_NUM_THREADS where the box sets it (its share of the host per GPU)
+    O.set_threads(used)
+    w.forward()
+    if w.has_reverse:
+        w.reverse()
+    torch.cuda.synchronize()
+    dt = w.dtype
+    tol = G.softmax_tol(dt)
+    parity = {"reference": "fp64 oracle (oracle/mp_oracle.c) on the same input bytes",
+              "bound": BOUND_TEXT["r16" if dt == torch.float16 else "r32"]}
+
+    if name == "cfg2":
+        x, g, dy = w.x.cpu().numpy(), w.gain.cpu().numpy(), w.dy.cpu().numpy()
+        sample, units = f"whole problem, all {w.rows} rows, forward + reverse", w.rows
+        nbytes = w.fwd_bytes + w.rev_bytes
+
+        def once():
+            return O.rmsnorm_ij_j(x, g, w.eps), O.rmsnorm_ij_j_reverse_mt(x, g, dy, w.eps)
+
+        def check(res):
+            y, (dx, dg) = res
+            sdx, _ = G.rmsnorm_reverse_scales(x, g, dy, w.eps)
+            G.compare(w.y, y, dt, "bench cfg2 y")
+            G.compare(w.dx, dx, dt, "bench cfg2 dx", scale=sdx)
+            G.compare(w.dgain, dg, dt, "bench cfg2 dgain", rowwise=False)
+            parity.update({"y": _numbers(w.y, y, dt), "dx": _numbers(w.dx, dx, dt),
+                           "dgain": _numbers(w.dgain, dg, dt, rowwise=False),
+                           "dx_with_cancellation_scale": _numbers(w.dx, dx, dt, scale=sdx)})
+    elif name in ("cfg1", "cfg3", "cfg5a", "cfg5b"):
+        m, n = w.shape
+        rows = {"cfg1": m, "cfg3": min(m, 4 * w.block) if name == "cfg3" else 0, "cfg5a": 32, "cfg5b": 96}[name]
+        rows = min(rows, m)
+        x = w.x[:rows].cpu().numpy()
+        es = w.x.element_size()
+        units = rows
+        if w.has_reverse:
+            yg, dy = w.y[:rows].cpu().numpy(), w.dy[:rows].cpu().numpy()
+            sample = f"rows 0..{rows - 1} of {m}, forward + reverse (the reverse reads the GPU's own forward output)"
+            nbytes = 5 * rows * n * es
+
+            def once():
+                return O.softmax_ij_j(x), O.softmax_ij_j_reverse(yg, dy)
+
+            def check(res):
+                y, dx = res
+                sc = G.softmax_reverse_scale(yg, dy)
+                G.compare(w.y[:rows], y, dt, f"bench {name} y", **tol)
+                G.compare(w.dx[:rows], dx, dt, f"bench {name} dx", scale=sc)
+                parity.update({"y": _numbers(w.y[:rows], y, dt, **tol), "dx": _numbers(w.dx[:rows], dx, dt),
+                               "dx_with_cancellation_scale": _numbers(w.dx[:rows], dx, dt, scale=sc)})
+        else:
+            sample = f"rows 0..{rows - 1} of {m}, forward"
+            nbytes = 2 * rows * n * es
+
+            def once():
+                return O.softmax_ij_j(x)
+
+            def check(y):
+                G.compare(w.y[:rows], y, dt, f"bench {name} y", **tol)
+                parity.update({"y": _numbers(w.y[:rows], y, dt, **tol)})
+    elif name in ("cfg4", "chain"):
+        k = min(w.n, 1 << 22)
+        ins = [t[:k].cpu().numpy() for t in (w.a, w.b, w.c, w.d)]
+        de = w.de[:k].cpu().numpy()
+        sample, units, nbytes = f"elements 0..{k - 1} of {w.n}, forward + reverse", k, 56 * k
+        if name == "cfg4":
+            def once():
+                return O.fused_selu_hadamard_add_add(*ins), O.fused_selu_hadamard_add_add_reverse(*ins, de)
+        else:  # relu((a - b) * (c + d)) and its gradients in fp64 (relu's convention: zero counts as positive)
+            def once():
+                a64, b64, c64, d64 = (t.astype(np.float64) for t in ins)
+                u, v = a64 - b64, c64 + d64
+                p = u * v
+                g = de.astype(np.float64) * (p >= 0)
+                return np.where(p >= 0, p, 0.0), (g * v, -(g * v), g * u, g * u)
+
+        def check(res):
+            e, grads = res
+            G.compare(w.e[:k], e, dt, f"bench {name} e", rowwise=False)
+            parity["e"] = _numbers(w.e[:k], e, dt, rowwise=False)
+            for tag, got, ref in zip("abcd", (w.da, w.db, w.dc, w.dd), grads):
+                G.compare(got[:k], ref, dt, f"bench {name} d{tag}", rowwise=False)
+                parity["d" + tag] = _numbers(got[:k], ref, dt, rowwise=False)
+    else:
+        return None, None
+
+    passes, spent, res = 0, 0.0, None
     while True:
         t0 = time.perf_counter()
-        y = O.rmsnorm_ij_j(x, g, w.eps)
-        dx, dg = O.rmsnorm_ij_j_reverse_mt(x, g, dy, w.eps)
+        res = once()
         spent += time.perf_counter() - t0
         passes += 1
-        if spent >= budget_s or passes >= 4000:
+        if spent >= budget_s or passes >= 100000:
             break
-    gbps = passes * (w.fwd_bytes + w.rev_bytes) / spent / 1e9
-    w.forward()
-    w.reverse()
-    torch.cuda.synchronize()
-    sdx, sdg = G.rmsnorm_reverse_scales(x, g, dy, w.eps)
-    G.compare(w.y, y, torch.float32, "bench cfg2 y")
-    G.compare(w.dx, dx, torch.float32, "bench cfg2 dx", scale=sdx)
-    G.compare(w.dgain, dg, torch.float32, "bench cfg2 dgain", rowwise=False)
+    check(res)
+    if name == "chain":  # numpy stands in for the oracle here: a parity check, not a baseline
+        parity["reference"] = "numpy fp64 on the same input bytes"
+        return None, parity
+    cpu = {"value": round(passes * nbytes / spent / 1e9, 3), "unit": "GB/s", "cores": used, "kind": "port",
+           "threads_used": used, "cores_available": avail,
+           "rows_per_s": round(passes * units / spent, 1),
+           "sample": f"{passes} passes over {sample}; {spent:.1f} s on {used} OpenMP threads "
+                     f"({avail} logical cores visible; the thread count is the box's OMP_NUM_THREADS, its share of the host per GPU)"}
+    return cpu, parity
 
-    def numbers(got, ref, rowwise, scale=None):
-        st = G.parity_stats(got, ref, torch.float32, rowwise=rowwise, scale=scale)
-        return {"n": st["n"], "max_abs": float(f"{st['max_abs']:.3e}"), "max_rel": float(f"{st['max_rel']:.3e}"),
-                "violations": st["violations"]}
 
-    parity = {
-        "reference": "fp64 oracle (oracle/mp_oracle.c) on the same input bytes, whole [8192, 4096] problem",
-        "bound": "|got - ref| <= 1e-5 * max(|ref|, RMS(ref row)); dgain: RMS of the whole vector; "
-                 "max_rel is the largest |got - ref| / max(|ref|, RMS)",
-        "y": numbers(w.y, y, True),
-        "dx": numbers(w.dx, dx, True),
-        "dgain": numbers(w.dgain, dg, False),
-        "dx_with_cancellation_scale": numbers(w.dx, dx, True, sdx),
-    }
-    return {"value": round(gbps, 3), "unit": "GB/s", "cores": cores, "kind": "port",
-            "rows_per_s": round(passes * w.rows / spent, 1),
-            "sample": f"{passes} full passes of cfg2 (forward + reverse, all {w.rows} rows), "
-                      f"{spent:.1f} s on {cores} OpenMP threads"}, parity
+CPU_BUDGET_S = {"cfg2": 10.0, "cfg1": 1.5, "cfg3": 3.0, "cfg4": 3.0, "chain": 1.5, "cfg5a": 3.0, "cfg5b": 3.0}
 
 
 def main():
@@ -364,10 +489,12 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--regions", type=int, default=7, help="timed regions of --steps steps each; value = the median one")
     ap.add_argument("--workload", default="cfg2", choices=sorted(SETS))
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity check")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the plain-copy ceilings of each stream mix")
+    ap.add_argument("--strict", action="store_true", help="exit 1 when a recorded check fails (a run-time chain slower than the build-time one)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this path has no multi-GPU leg (rows shard without "
@@ -381,20 +508,23 @@ def main():
     ffi.load()  # raises if the HIP libraries are not built; there is no fallback
     torch.cuda.set_device(0)
 
+    import contextlib
     name = args.workload
     sets = make_sets(name)
     w = sets[0]
-    dt, dom_ms = time_steps(sets, args.steps, args.warmup)
+    times, in_region_ms, prewarm = time_regions(sets, args.steps, args.warmup, args.regions)
     step_bytes = w.fwd_bytes + w.rev_bytes
+    region_values = [args.steps * step_bytes / t / 1e9 for t in times]
+    dt = _median(times)  # the median region: `value` and `ms_per_step` describe the same region
     value = args.steps * step_bytes / dt / 1e9
-    fwd_ms, rev_ms = time_each(sets, max(20, min(args.steps, 100)))
+    fwd_ms, rev_ms = time_each(sets, max(24, min(args.steps, 96)))
 
-    dom_bytes, dom_name = (w.rev_bytes, "reverse") if w.has_reverse else (w.fwd_bytes, "forward")
+    dom_bytes, dom_name, dom_ms = (w.rev_bytes, "reverse", rev_ms) if w.has_reverse else (w.fwd_bytes, "forward", fwd_ms)
+    checks_failed = []
     cpu_line = parity = None
-    if not args.no_cpu and name == "cfg2":
-        import contextlib
+    if not args.no_cpu:
         with contextlib.redirect_stdout(sys.stderr):  # stdout carries the one JSON line only
-            cpu_line, parity = cpu_baseline_cfg2(w)
+            cpu_line, parity = cpu_and_parity(name, w, CPU_BUDGET_S.get(name, 3.0))
     per_workload = rates(w, fwd_ms, rev_ms)
     del sets
     torch.cuda.empty_cache()
@@ -415,12 +545,19 @@ def main():
         "data": "synthetic",
         "config": {"workload": f"{name}: {W.DESCRIPTION[name]}", "buffer_sets": SETS[name],
                    "bytes_per_step": step_bytes},
+        # how `value` was taken: median of `regions` regions of `steps` steps each, after the warm-up
+        # steps and a disclosed pre-warm of the same steps; the first region is region_values_GBps[0]
+        "regions": args.regions,
+        "region_values_GBps": [round(v, 1) for v in region_values],
+        **prewarm,
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "rows_per_s": round(args.steps * w.rows / dt, 1),
-        # the dominant launcher, from events sampled inside the timed region
+        # the dominant launcher: groups of back-to-back launches between event pairs, right after the regions
         "roofline": roofline_of(name, dom_name, dom_bytes, dom_ms, rev_ceiling if w.has_reverse else fwd_ceiling),
         name: per_workload,
     }
+    # one launch of the dominant launcher inside each timed region, events around it (pair included)
+    line["roofline"]["in_region_launch_ms"] = [round(t, 5) for t in in_region_ms]
     if w.has_reverse:
         line[name]["roofline_fwd"] = roofline_of(name, "forward", w.fwd_bytes, fwd_ms, fwd_ceiling)
     avg_ms = line["roofline"]["avg_launch_ms"]
@@ -438,7 +575,9 @@ def main():
                                  "unit": "TFLOP/s", "frac": round(tf / MFMA_PEAK_TFLOPS[name], 4),
                                  "flops_per_launch": w.rev_flops})
     if cpu_line is not None:
-        line["cpu_baseline"], line["parity"] = cpu_line, parity
+        line["cpu_baseline"] = cpu_line
+    if parity is not None:
+        line["parity"] = parity
     del w
     torch.cuda.empty_cache()
 
@@ -449,8 +588,9 @@ def main():
                 continue
             osets = make_sets(other)
             o = osets[0]
-            k = max(10, min(args.steps, 40 if other in ("cfg3", "cfg4", "chain") else 100))
-            time_steps(osets, 5, 2)
+            k = max(24, min(args.steps, 40 if other in ("cfg3", "cfg4", "chain") else 96))
+            for i in range(5):
+                _step(osets, i)
             f_ms, r_ms = time_each(osets, k)
             extra[other] = rates(o, f_ms, r_ms)
             extra[other]["workload"] = W.DESCRIPTION[other]
@@ -460,6 +600,13 @@ def main():
                 extra[other]["fwd_graph_GBps"] = round(o.fwd_bytes / (g_ms * 1e-3) / 1e9, 1)
                 extra[other]["fwd_graph_matches_eager"] = same
                 extra[other]["native_caller"] = native_launch_cost()
+            if not args.no_cpu and other in CPU_BUDGET_S:
+                with contextlib.redirect_stdout(sys.stderr):
+                    o_cpu, o_parity = cpu_and_parity(other, o, CPU_BUDGET_S[other])
+                if o_cpu is not None:
+                    extra[other]["cpu_baseline"] = o_cpu
+                if o_parity is not None:
+                    extra[other]["parity"] = o_parity
             del osets
             torch.cuda.empty_cache()
             if other.startswith("cfg") or other == "chain":  # the same roofline object as the headline workload carries
@@ -471,9 +618,23 @@ def main():
                     extra[other]["roofline"] = roofline_of(other, "forward", o.fwd_bytes, f_ms, f_ceil)
             del o
             torch.cuda.empty_cache()
+        # an expression compiled at run time must run at the rate of the build-time chain with the
+        # same streams (same engine, same launch plan): within 10 % in both directions
+        if "chain" in extra and "cfg4" in extra:
+            c, f = extra["chain"], extra["cfg4"]
+            ratio = {"fwd": round(c["fwd_ms"] / f["fwd_ms"], 4), "rev": round(c["rev_ms"] / f["rev_ms"], 4)}
+            ok = all(v <= 1.10 for v in ratio.values())
+            extra["chain"]["runtime_vs_buildtime_ms_ratio"] = {**ratio, "bound": 1.10, "ok": ok}
+            if not ok:
+                checks_failed.append(f"run-time chain slower than the build-time chain: {ratio}")
         line["other_workloads"] = extra
+    line["checks_failed"] = checks_failed
 
     print(json.dumps(line), flush=True)
+    for msg in checks_failed:
+        print(f"bench.py: CHECK FAILED: {msg}", file=sys.stderr)
+    if checks_failed and args.strict:
+        sys.exit(1)
 
 
 if __name__ == "__main__":
