@@ -89,4 +89,12 @@ extern "C" void mpSetClusterDeep(len_t which) {
   mp::require(which <= 2, "mpSetClusterDeep: 0, 1 or 2");
   mp::cluster_tuning().deep = (int)which;
 }
+
+// Diagnostic: where the stamped exchange words of the shared-row softmax kernels live: 1 (as
+// shipped) in the library's own device memory where a region is to be had, 0 always in the
+// caller's workspace, which is then cleared in front of every launch. Process-wide.
+extern "C" void mpSetClusterWords(len_t own) {
+  mp::require(own <= 1, "mpSetClusterWords: 0 or 1");
+  mp::cluster_tuning().own_words = (int)own;
+}
 #endif

@@ -10,6 +10,10 @@
 
 #include "row_dispatch.h"
 
+#ifdef MP_HOST_SIDE
+#include <mutex>
+#endif
+
 #if defined(__cplusplus) && defined(__HIPCC__)
 
 namespace mp {
@@ -50,6 +54,7 @@ struct ClusterTuning {
   int packs_per_block = 0; /* 0: one pack per thread less than the register tile holds */
   unsigned spin_limit = 1u << 22;
   int deep = 0; /* the RMSNorm reverse's shared rows: 0 by the launcher's rule, 1 always the pipelined kernel, 2 never */
+  int own_words = 1; /* stamped exchange words: 1 in the library's own memory where a region is to be had, 0 always in the caller's workspace */
 };
 #ifdef MP_DIAGNOSTICS
 inline ClusterTuning& cluster_tuning() {
@@ -141,6 +146,154 @@ __device__ __forceinline__ bool cluster_exchange_sums(typename slot_word<P>::typ
 #pragma unroll
     for (int v = 0; v < NVAL; ++v) {
       const P total = wave_allreduce<AddOP>(lane < C && heard ? __builtin_bit_cast(P, w[v]) : (P)0);
+      if (lane == 0) bc[v] = total;
+    }
+    if (lane == 0) bc[NVAL] = missing;
+  }
+  __syncthreads();
+#pragma unroll
+  for (int v = 0; v < NVAL; ++v) vals[v] = bc[v];
+  return bc[NVAL] == (P)0;
+}
+
+/* ---------------------------------------------------------------------------------------
+ * Stamped exchange words: the hand-over above without the clearing launch in front.
+ *
+ * A word is 64 bits: a stamp in the high half, 32 bits of a value in the low half (a value of
+ * precision<T> takes one word for fp32, two for fp64). Workgroup `rank` of a row owns
+ * WPS = values * parts consecutive words. At its start it reads the stamp its own first word
+ * carries from the launch before (zero in memory nobody has written yet), adds one, and that is
+ * the stamp of this launch: it publishes its values under it and takes a partner's words for
+ * published when all of them carry it. Every workgroup of a row publishes exactly once per
+ * launch, whether it later stops waiting or not, so the words of a row move from one stamp to
+ * the next in step and a word left by an earlier launch can never carry the stamp being waited
+ * for; nothing has to be cleared between launches, and launches recorded into a graph and
+ * replayed are as good as fresh ones, since the stamp lives on the device.
+ *
+ * That needs words that only this protocol ever writes and that are tied to one launch geometry.
+ * They live in device memory of the library (share_arena), handed out by share_region(): one
+ * region per (caller's workspace address, rows, workgroups a row, words a workgroup), never taken
+ * back. The caller's workspace is the key because launches that may overlap in time must have
+ * different workspaces anyway, so they never meet in a region, while launches through one
+ * workspace are ordered by the caller already. When the arena or the table is full, or a problem
+ * needs more than the arena holds, the words are taken from the caller's workspace instead, which
+ * the launcher then clears with cluster_zero_slots first (every stamp is 1 then): same kernels.
+ * ------------------------------------------------------------------------------------- */
+
+typedef unsigned long long share_word;
+constexpr size_t SHARE_ARENA_WORDS = (size_t)(4u << 20) / sizeof(share_word);
+constexpr int SHARE_REGIONS = 64;
+static __device__ __align__(256) share_word share_arena[SHARE_ARENA_WORDS];
+
+template <class P> constexpr int share_parts() { return (int)(sizeof(P) / 4); }
+
+#ifdef MP_HOST_SIDE
+struct ShareTable {
+  struct Entry { uintptr_t workspace; size_t rows, offset; int per_row, wps; };
+  std::mutex lock;
+  Entry entries[SHARE_REGIONS];
+  int count = 0;
+  size_t used = 0;
+};
+static ShareTable share_table;
+
+/* Offset (in words) of the region for this key inside share_arena; -1: none to be had, use the
+ * caller's workspace. */
+inline long long share_region(const void* workspace, size_t rows, int per_row, int wps) {
+#ifdef MP_DIAGNOSTICS
+  if (!cluster_tuning().own_words) return -1;
+#endif
+  const uintptr_t key = reinterpret_cast<uintptr_t>(workspace);
+  const size_t need = rows * (size_t)per_row * (size_t)wps;
+  std::lock_guard<std::mutex> hold(share_table.lock);
+  for (int i = 0; i < share_table.count; ++i) {
+    const ShareTable::Entry& e = share_table.entries[i];
+    if (e.workspace == key && e.rows == rows && e.per_row == per_row && e.wps == wps) return (long long)e.offset;
+  }
+  const size_t start = (share_table.used + 31) / 32 * 32; /* regions start on 256-byte lines */
+  if (share_table.count == SHARE_REGIONS || start + need > SHARE_ARENA_WORDS) return -1;
+  share_table.entries[share_table.count++] = ShareTable::Entry{key, rows, start, per_row, wps};
+  share_table.used = start + need;
+  return (long long)start;
+}
+#endif
+
+/* The words of the launch: the caller's (cleared by the launcher) when given, else the region at
+ * `offset` of the library's arena. */
+__device__ __forceinline__ share_word* share_words(share_word* callers, size_t offset) {
+  return callers != nullptr ? callers : share_arena + offset;
+}
+
+/* The stamp of this launch for a workgroup whose first word is `mine`: asked for by the
+ * workgroup's first lane before it loads its chunk, read (share_stamp_of) when it publishes.
+ * Only wave 0 may use the result. */
+__device__ __forceinline__ share_word share_peek(const share_word* mine, int lane) {
+  share_word old = 0;
+  if (lane == 0) old = __hip_atomic_load(mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return old;
+}
+__device__ __forceinline__ unsigned share_stamp_of(share_word peeked) {
+  const unsigned old = (unsigned)(peeked >> 32);
+  return (unsigned)__builtin_amdgcn_readfirstlane((int)(old + 1u)); /* lane 0's, for every lane of wave 0 */
+}
+
+template <int NVAL, class P>
+__device__ __forceinline__ void share_publish(share_word* mine, unsigned stamp, const P (&vals)[NVAL]) {
+  constexpr int PARTS = share_parts<P>();
+  typedef unsigned bits_t __attribute__((ext_vector_type(PARTS)));
+#pragma unroll
+  for (int v = 0; v < NVAL; ++v) {
+    const bits_t b = __builtin_bit_cast(bits_t, vals[v]);
+#pragma unroll
+    for (int q = 0; q < PARTS; ++q)
+      __hip_atomic_store(mine + v * PARTS + q, ((share_word)stamp << 32) | b[q], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+}
+
+/* One look at a partner's words; true when every one carries the stamp (vals are then its values). */
+template <int NVAL, class P>
+__device__ __forceinline__ bool share_read(const share_word* theirs, unsigned stamp, P (&vals)[NVAL]) {
+  constexpr int PARTS = share_parts<P>();
+  typedef unsigned bits_t __attribute__((ext_vector_type(PARTS)));
+  share_word w[NVAL * PARTS];
+#pragma unroll
+  for (int i = 0; i < NVAL * PARTS; ++i) w[i] = __hip_atomic_load(theirs + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  bool ok = true;
+#pragma unroll
+  for (int v = 0; v < NVAL; ++v) {
+    bits_t b;
+#pragma unroll
+    for (int q = 0; q < PARTS; ++q) {
+      ok = ok && (unsigned)(w[v * PARTS + q] >> 32) == stamp;
+      b[q] = (unsigned)w[v * PARTS + q];
+    }
+    vals[v] = __builtin_bit_cast(P, b);
+  }
+  return ok;
+}
+
+/* cluster_exchange_sums on stamped words. `row_words` points at the row's C * NVAL * parts words,
+ * `peeked` is share_peek() of this workgroup's first word, taken before the chunk was loaded. */
+template <int NVAL, class P>
+__device__ __forceinline__ bool share_exchange_sums(share_word* row_words, int C, int rank, share_word peeked,
+                                                    P (&vals)[NVAL], unsigned spin_limit, P* bc, int lane) {
+  constexpr int WPS = NVAL * share_parts<P>();
+  if (lane < WAVE) { /* wave 0: lane r waits for workgroup r of this row */
+    const unsigned stamp = share_stamp_of(peeked);
+    if (lane == 0) share_publish<NVAL>(row_words + (size_t)rank * WPS, stamp, vals);
+    P got[NVAL];
+    bool heard = true;
+    if (lane < C) {
+      for (unsigned spins = 0;; ++spins) {
+        heard = share_read<NVAL>(row_words + (size_t)lane * WPS, stamp, got);
+        if (heard || spins >= spin_limit) break;
+        __builtin_amdgcn_s_sleep(4);
+      }
+    }
+    const P missing = wave_allreduce<AddOP>(heard ? (P)0 : (P)1); /* every lane takes part */
+#pragma unroll
+    for (int v = 0; v < NVAL; ++v) {
+      const P total = wave_allreduce<AddOP>(lane < C && heard ? got[v] : (P)0);
       if (lane == 0) bc[v] = total;
     }
     if (lane == 0) bc[NVAL] = missing;

@@ -405,9 +405,9 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
  * two agent-scope atomic words in caller-owned scratch, waits for the other C-1, and writes its
  * chunk: the row is still read once and written once.
  *
- * A published word is never zero (a maximum of +0 is stored as -0; the sum of a chunk without a
- * finite entry is stored as 1 and ignored through its -inf maximum), so "non-zero" means
- * "published" and the scratch only has to be zero when the kernel starts (cluster_zero_slots).
+ * The words are stamped (row_cluster.h): a word counts as published when it carries the stamp of
+ * this launch, which a workgroup derives from what its own word carried before, so no launch in
+ * front has to clear anything when the words are the library's own.
  *
  * Waiting is bounded. Workgroups of one row have consecutive indices and a workgroup publishes
  * before it waits, so with in-order dispatch the wait is short; if spin_limit polls pass
@@ -425,16 +425,17 @@ template <class T> constexpr int cluster_nv() {
 
 template <class T, int W>
 __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
-    const T* x, T* y, typename slot_word<typename precision<T>::type>::type* slots,
+    const T* x, T* y, share_word* callers_words, size_t region,
     size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
   using P = typename precision<T>::type;
-  using Word = typename slot_word<P>::type;
-  constexpr int G = CLUSTER_THREADS, NV = cluster_nv<T>();
+  constexpr int G = CLUSTER_THREADS, NV = cluster_nv<T>(), WPS = 2 * share_parts<P>();
   __shared__ P red[4][G / WAVE];
   __shared__ P bc[3];
   const int lane = threadIdx.x;
   const size_t row = blockIdx.x / (unsigned)C;
   const int rank = (int)(blockIdx.x % (unsigned)C);
+  share_word* row_words = share_words(callers_words, region) + row * (size_t)C * WPS;
+  const share_word peeked = C > 1 ? share_peek(row_words + (size_t)rank * WPS, lane) : 0; /* on its way while the chunk loads */
   const T* xr = x + row * n;
   T* yr = y + row * n;
   const RowGeom<T, W> g(xr, n, true);
@@ -520,31 +521,24 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
   }
   P M = mx, S = s;
   if (C > 1) {
-    Word* mine = slots + ((size_t)row * C + rank) * 2;
-    if (lane == 0) {
-      const P pm = mx == (P)0 ? -(P)0 : mx;
-      const P ps = mx > neg_inf<P>() ? s : (P)1;
-      __hip_atomic_store(mine + 0, __builtin_bit_cast(Word, pm), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      __hip_atomic_store(mine + 1, __builtin_bit_cast(Word, ps), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    }
     if (lane < WAVE) { /* wave 0: lane b waits for workgroup b of this row */
-      P om = neg_inf<P>(), os = (P)0;
+      const unsigned stamp = share_stamp_of(peeked);
+      if (lane == 0) { /* the sum of a chunk without a finite entry is ignored through its -inf maximum */
+        const P mine[2] = {mx, s};
+        share_publish<2>(row_words + (size_t)rank * WPS, stamp, mine);
+      }
+      P theirs[2] = {neg_inf<P>(), (P)0};
       bool ok = true;
       if (lane < C) {
-        Word* theirs = slots + ((size_t)row * C + lane) * 2;
-        Word a = 0, b = 0;
         for (unsigned spins = 0;; ++spins) {
-          a = __hip_atomic_load(theirs + 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          b = __hip_atomic_load(theirs + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          if ((a != 0 && b != 0) || spins >= spin_limit) break;
+          ok = share_read<2>(row_words + (size_t)lane * WPS, stamp, theirs);
+          if (ok || spins >= spin_limit) break;
           __builtin_amdgcn_s_sleep(4);
         }
-        ok = a != 0 && b != 0;
-        om = __builtin_bit_cast(P, a);
-        os = __builtin_bit_cast(P, b);
       }
+      const P om = theirs[0], os = theirs[1];
       const P all_ok = wave_allreduce<AddOP>(ok ? (P)0 : (P)1); /* every lane takes part */
-      const P gm = wave_allreduce<MaxOP>(ok ? om : neg_inf<P>());
+      const P gm = wave_allreduce<MaxOP>(lane < C && ok ? om : neg_inf<P>());
       const P part = (lane < C && ok && om > neg_inf<P>()) ? os * exp_shifted(om, shift_of(gm)) : (P)0;
       const P gs = wave_allreduce<AddOP>(part);
       if (lane == 0) {
@@ -626,7 +620,7 @@ template <class T> inline size_t softmax_scratch_bytes(size_t m, size_t n) {
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   const size_t c = cluster_size_for_scratch(cluster_size<T>((n + W - 1) / W));
-  return m * c * 2 * sizeof(P);
+  return m * c * 2 * share_parts<P>() * sizeof(share_word); /* (max, sum) as stamped words */
 }
 
 /* ------------------------------------------------------------------ streaming reverse */
@@ -720,8 +714,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_rev_stream(
 /* ------------------------------------------------------------------ cluster reverse */
 
 /* The reverse of a long row, shared like the forward: each of C consecutive workgroups keeps its
- * chunk of y and dy in registers, publishes its part of dot(y, dy) as one agent-scope atomic word
- * (a part of exactly +0 is stored as -0, so a published word is never zero), waits for the
+ * chunk of y and dy in registers, publishes its part of dot(y, dy) as a stamped word, waits for the
  * others with the same bounded poll, and writes its chunk of dx: y and dy are read once. A
  * workgroup that stops waiting reads the whole row again for the dot product, which is why the
  * shared path is not taken when dx overwrites y or dy. */
@@ -735,17 +728,18 @@ constexpr int CLUSTER_REV_NV = 4;
 template <class T, int W, bool BLEND>
 __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_rev_cluster(
     const T* y, const T* dy, T* dx, typename precision<T>::type alpha,
-    typename slot_word<typename precision<T>::type>::type* slots,
+    share_word* callers_words, size_t region,
     size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
   using P = typename precision<T>::type;
-  using Word = typename slot_word<P>::type;
-  constexpr int G = CLUSTER_THREADS, NV = CLUSTER_REV_NV;
+  constexpr int G = CLUSTER_THREADS, NV = CLUSTER_REV_NV, WPS = share_parts<P>();
   using V = typename vec_of<T, W>::type;
   __shared__ P red[2][G / WAVE];
   __shared__ P bc[2];
   const int lane = threadIdx.x;
   const size_t row = blockIdx.x / (unsigned)C;
   const int rank = (int)(blockIdx.x % (unsigned)C);
+  share_word* row_words = share_words(callers_words, region) + row * (size_t)C * WPS;
+  const share_word peeked = C > 1 ? share_peek(row_words + (size_t)rank * WPS, lane) : 0; /* on its way while the chunk loads */
   const T* yr = y + row * n;
   const T* gr = dy + row * n;
   T* dr = dx + row * n;
@@ -798,7 +792,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_rev_cluster(
 
   if (C > 1) {
     P sums[1] = {dot};
-    const bool complete = cluster_exchange_sums<1>(slots + (size_t)row * C, C, rank, sums, spin_limit, bc, lane);
+    const bool complete = share_exchange_sums<1>(row_words, C, rank, peeked, sums, spin_limit, bc, lane);
     dot = sums[0];
     if (!complete) { /* gave up waiting: the whole row's dot product here */
       P d = (P)0;
@@ -893,16 +887,24 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
    * overwrote: shared rows need distinct buffers */
   const bool shareable = scratch != nullptr && !ranges_overlap(x, y, m * n * sizeof(T));
   if (C >= 1 && (C == 1 || shareable) && m * (size_t)C < 0x7fffffffull) {
-    using Word = typename slot_word<P>::type;
-    Word* slots = static_cast<Word*>(scratch);
     const int ppb = cluster_chunk_packs(packs, C, (size_t)CLUSTER_THREADS * cluster_nv<T>(), CLUSTER_SKEW_MAX);
     require(ppb <= CLUSTER_THREADS * cluster_nv<T>(), "softmax: cluster chunk exceeds the register tile");
+    /* the stamped words of the rows: a region of the library's own for this workspace and geometry,
+     * or (none to be had) the caller's workspace, cleared first */
+    constexpr int WPS = 2 * share_parts<P>();
+    share_word* callers = nullptr;
+    long long region = 0;
     if (C > 1) {
-      const size_t words = m * (size_t)C * 2;
-      cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
+      region = share_region(scratch, m, C, WPS);
+      if (region < 0) {
+        callers = static_cast<share_word*>(scratch);
+        region = 0;
+        const size_t words = m * (size_t)C * WPS;
+        cluster_zero_slots<share_word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(callers, words);
+      }
     }
     softmax_fwd_cluster<T, W><<<dim3((unsigned)(m * C)), dim3(CLUSTER_THREADS), 0, stream>>>(
-        x, y, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+        x, y, callers, (size_t)region, m, n, C, ppb, cluster_tuning().spin_limit);
     MP_CHECK_LAUNCH();
     return;
   }
@@ -955,7 +957,7 @@ template <class T> inline size_t softmax_reverse_scratch_bytes(size_t m, size_t 
   using P = typename precision<T>::type;
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   const size_t c = cluster_size_for_scratch(cluster_rev_size<T>((n + W - 1) / W));
-  return m * c * sizeof(P);
+  return m * c * share_parts<P>() * sizeof(share_word); /* the part of the dot product as stamped words */
 }
 
 template <class T>
@@ -996,17 +998,23 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   const int C = cluster_rev_size<T>(packs);
   const bool distinct = !ranges_overlap(dx, y, m * n * sizeof(T)) && !ranges_overlap(dx, dy, m * n * sizeof(T));
   if (C >= 1 && (C == 1 || (scratch != nullptr && distinct)) && m * (size_t)C < 0x7fffffffull) {
-    using Word = typename slot_word<P>::type;
-    Word* slots = static_cast<Word*>(scratch);
     const int ppb = cluster_chunk_packs(packs, C, (size_t)CLUSTER_THREADS * CLUSTER_REV_NV, CLUSTER_SKEW_MAX);
     require(ppb <= CLUSTER_THREADS * CLUSTER_REV_NV, "softmax reverse: cluster chunk exceeds the register tile");
-    if (C > 1) {
-      const size_t words = m * (size_t)C;
-      cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
+    constexpr int WPS = share_parts<P>();
+    share_word* callers = nullptr;
+    long long region = 0;
+    if (C > 1) { /* as in the forward: the library's own words for this workspace and geometry, else the caller's, cleared */
+      region = share_region(scratch, m, C, WPS);
+      if (region < 0) {
+        callers = static_cast<share_word*>(scratch);
+        region = 0;
+        const size_t words = m * (size_t)C * WPS;
+        cluster_zero_slots<share_word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(callers, words);
+      }
     }
     const dim3 grid((unsigned)(m * C)), block(CLUSTER_THREADS);
-    if (blend) softmax_rev_cluster<T, W, true><<<grid, block, 0, stream>>>(y, dy, dx, al, slots, m, n, C, ppb, cluster_tuning().spin_limit);
-    else softmax_rev_cluster<T, W, false><<<grid, block, 0, stream>>>(y, dy, dx, al, slots, m, n, C, ppb, cluster_tuning().spin_limit);
+    if (blend) softmax_rev_cluster<T, W, true><<<grid, block, 0, stream>>>(y, dy, dx, al, callers, (size_t)region, m, n, C, ppb, cluster_tuning().spin_limit);
+    else softmax_rev_cluster<T, W, false><<<grid, block, 0, stream>>>(y, dy, dx, al, callers, (size_t)region, m, n, C, ppb, cluster_tuning().spin_limit);
     MP_CHECK_LAUNCH();
     return;
   }

@@ -43,7 +43,7 @@ def lib():
 ROW_STEMS = ("softmax_ij_j", "softmax_ij_j_reverse", "rmsnorm_ij_j", "rmsnorm_ij_j_reverse")
 ROW_SIZE_FNS = ("mpSoftmaxScratchBytes", "mpSoftmaxReverseScratchBytes", "mpRmsnormScratchBytes",
                 "mpRmsnormReverseScratchBytes")
-_diag = {"lib": None, "regime": 0, "tuned": False, "deep": 0}
+_diag = {"lib": None, "regime": 0, "tuned": False, "deep": 0, "own_words": 1}
 
 
 def diag_lib():
@@ -67,12 +67,14 @@ def diag_lib():
         d.mpSetClusterTuning.restype = None
         d.mpSetClusterDeep.argtypes = [ffi.len_t]
         d.mpSetClusterDeep.restype = None
+        d.mpSetClusterWords.argtypes = [ffi.len_t]
+        d.mpSetClusterWords.restype = None
         _diag["lib"] = d
     return _diag["lib"]
 
 
 def _override_active():
-    return _diag["regime"] != 0 or _diag["tuned"] or _diag["deep"] != 0
+    return _diag["regime"] != 0 or _diag["tuned"] or _diag["deep"] != 0 or _diag["own_words"] != 1
 
 
 def row_size(fn, dtype, m, n):
@@ -401,6 +403,13 @@ def set_cluster_deep(which=0):
     rule, 1 always the pipelined one, 2 never."""
     diag_lib().mpSetClusterDeep(int(which))
     _diag["deep"] = int(which)
+
+
+def set_cluster_words(own=1):
+    """Where the shared-row softmax kernels of the test build keep their exchange words: 1 in the
+    library's own memory (as shipped), 0 in the caller's workspace, cleared before every launch."""
+    diag_lib().mpSetClusterWords(int(own))
+    _diag["own_words"] = int(own)
 
 
 def permutate(src, dst, alpha=0.0):

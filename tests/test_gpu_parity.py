@@ -430,6 +430,98 @@ def test_softmax_forward_cluster_path(dtype, packs, spin):
                 y.check("y")
 
 
+@pytest.mark.parametrize("own", [1, 0], ids=["library-words", "caller-words"])
+def test_shared_row_softmax_launch_after_launch(own):
+    """The stamped exchange words of the shared-row softmax kernels: launch after launch through one
+    workspace with fresh inputs every time (a word left by the launch before must not pass for a
+    result), two geometries taking turns through the same workspace, more workspaces than the
+    library has regions for, forward and reverse, in the library's own words (the library as
+    shipped) and in the caller's workspace (test build), whole outputs against the oracle."""
+    r = rng(37)
+    f32 = torch.float32
+    G.set_cluster_words(own)
+    try:
+        shapes = [(6, 50257), (3, 151936)]
+        big = max(G.row_size("mpSoftmaxScratchBytes", f32, m, n) for m, n in shapes)
+        bigr = max(G.row_size("mpSoftmaxReverseScratchBytes", f32, m, n) for m, n in shapes)
+        assert big > 0 and bigr > 0
+        fs, rs = G.Guarded((big,), torch.uint8), G.Guarded((bigr,), torch.uint8)
+        for launch in range(6):
+            m, n = shapes[launch % 2]
+            x = G.dev(r.normal(0, 3, (m, n)) + launch, f32)
+            dy = G.dev(r.normal(0, 1, (m, n)), f32)
+            y, dx = G.Guarded((m, n), f32), G.Guarded((m, n), f32)
+            G.say(f"shared rows own={own} launch {launch} ({m},{n})")
+            G.softmax(x.t, y.t, scratch=fs.t)
+            G.softmax_reverse(y.t, dy.t, dx.t, 0.0, scratch=rs.t)
+            yh, dyh = G.host(y.t), G.host(dy.t)
+            G.compare(y.t, O.softmax_ij_j(G.host(x.t)), f32, f"shared rows launch {launch}", atol=1e-6)
+            G.compare(dx.t, O.softmax_ij_j_reverse(yh, dyh), f32, f"shared rows rev launch {launch}",
+                      scale=G.softmax_reverse_scale(yh, dyh))
+            for b in (y, dx, fs, rs):
+                b.check("shared rows")
+        # 70 workspaces at different addresses (the table has 64 regions): the ones beyond fall back
+        m, n = 2, 50257
+        need = G.row_size("mpSoftmaxScratchBytes", f32, m, n)
+        pool = torch.zeros(70 * (need + 256), dtype=torch.uint8, device="cuda")
+        x = G.dev(r.normal(0, 3, (m, n)), f32)
+        ref = O.softmax_ij_j(G.host(x.t))
+        for i in range(70):
+            y = G.Guarded((m, n), f32)
+            ws = pool[i * (need + 256):(i + 1) * (need + 256)]
+            G.say(f"shared rows own={own} workspace {i}")
+            G.softmax(x.t, y.t, scratch=ws)
+            if i % 10 == 0 or i > 60:
+                G.compare(y.t, ref, f32, f"shared rows workspace {i}", atol=1e-6)
+                y.check("y")
+    finally:
+        G.set_cluster_words(1)
+
+
+def test_shared_row_softmax_replayed_from_a_graph_with_fresh_inputs():
+    """A captured forward + reverse over shared rows, replayed with other inputs each time: the stamp
+    of a launch is read on the device, so a replay is as good as a fresh launch."""
+    r = rng(38)
+    f32 = torch.float32
+    m, n = 5, 50257
+    x = torch.empty((m, n), dtype=f32, device="cuda")
+    dy = torch.empty((m, n), dtype=f32, device="cuda")
+    y, dx = torch.empty_like(x), torch.empty_like(x)
+    fs = torch.empty(G.row_size("mpSoftmaxScratchBytes", f32, m, n), dtype=torch.uint8, device="cuda")
+    rs = torch.empty(G.row_size("mpSoftmaxReverseScratchBytes", f32, m, n), dtype=torch.uint8, device="cuda")
+
+    def fresh(k):
+        x.copy_(torch.from_numpy(r.normal(0, 3, (m, n)) + k).to(f32))
+        dy.copy_(torch.from_numpy(r.normal(0, 1, (m, n))).to(f32))
+
+    def sequence():
+        G.softmax(x, y, scratch=fs)
+        G.softmax_reverse(y, dy, dx, 0.0, scratch=rs)
+
+    fresh(0)
+    G.say("shared rows graph: eager")
+    sequence()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        sequence()
+    for k in range(1, 5):
+        fresh(k)
+        y.fill_(float("nan"))
+        dx.fill_(float("nan"))
+        torch.cuda.synchronize()
+        G.say(f"shared rows graph: replay {k}")
+        graph.replay()
+        torch.cuda.synchronize()
+        yh, dyh = G.host(y), G.host(dy)
+        G.compare(y, O.softmax_ij_j(G.host(x)), f32, f"shared rows replay {k}", atol=1e-6)
+        G.compare(dx, O.softmax_ij_j_reverse(yh, dyh), f32, f"shared rows rev replay {k}",
+                  scale=G.softmax_reverse_scale(yh, dyh))
+        if k == 2:  # eager work through the same workspaces between replays
+            sequence()
+            torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("dtype", [torch.float16, torch.float32], ids=["r16", "r32"])
 def test_shared_rows_starting_at_every_offset_from_a_128_byte_line(dtype):
     """Rows of 16 bytes more than a multiple of 128: nine consecutive rows start at each of the
