@@ -11,8 +11,9 @@
  * constant as second argument, scale (the reference's dilate: x * c) and shift (its translate:
  * x + c), with its leaves written as 0, 1, ... (or x0, x1, ...) and numbered in order of first
  * appearance; a leaf may appear more than once. Examples: "selu(mul(add(0,1),add(2,3)))",
- * "relu(scale(mul(0,1),0.125))". At most 8 leaves, 64 nodes. A constant is part of the expression:
- * another value is another expression, compiled separately.
+ * "relu(scale(mul(0,1),0.125))". At most 8 leaves, 8 constants, 64 nodes. The constants are
+ * arguments of the kernels, read from the text at every call: an expression is compiled once,
+ * whatever the values (a learning rate that changes every step costs nothing).
  * dtype is MP_R16, MP_R32 or MP_R64 (tensor_types.h).
  *
  * The first use of an (expression, dtype) in a process compiles it (about half a second, with
@@ -58,8 +59,12 @@ EXTERN_C const char* mpChainSource(const char* expression, int dtype);
  * chain_forward_<l>, chain_reverse_overwrite_<l>, chain_reverse_blend_<l> with l = 0 (all operands
  * 16-byte aligned), 1 (operands that share a place in a 128-byte line) or 2 (any alignment). */
 EXTERN_C const void* mpChainCodeObject(const char* expression, int dtype, len_t* bytes);
-/* How many (expression, dtype) pairs this process has compiled. */
+/* How many (expression, dtype) pairs this process has compiled (expressions that differ in their
+ * constants only are one). */
 EXTERN_C len_t mpChainCacheSize(void);
+/* How many compilations this process has started, failed ones included. A compilation that failed is
+ * not tried again: later calls for that (expression, dtype) fail at once with the same reason. */
+EXTERN_C len_t mpChainCompilations(void);
 /* Why the calling thread's last failing call failed. Valid until that thread's next failure. */
 EXTERN_C const char* mpChainError(void);
 

@@ -1,7 +1,8 @@
 /*
  * Elementwise expressions fused at run time: mpChainForward / mpChainReverse take an expression
  * over add, sub, mul, neg, relu, selu, scale(x, c) and shift(x, c) as text, and run it as ONE kernel of the flat elementwise
- * engine (elementwise.h) and its reverse as ONE kernel that writes every leaf gradient. The first
+ * engine (elementwise.h) and its reverse as ONE kernel that writes every leaf gradient. The constants
+ * of scale and shift are kernel arguments, so an expression is compiled once whatever their values. The first
  * call for an (expression, dtype) writes the three functors (forward, reverse that overwrites,
  * reverse that blends), compiles them with hiprtc against the very headers this library is built
  * from (their text is embedded at build time) and keeps the code object for the life of the
@@ -38,7 +39,7 @@
 
 namespace {
 
-constexpr int MAX_LEAVES = 8, MAX_NODES = 64, MAX_DEVICES = 64;
+constexpr int MAX_LEAVES = 8, MAX_NODES = 64, MAX_CONSTANTS = 8, MAX_DEVICES = 64;
 
 enum Op { LEAF, ADD, SUB, MUL, NEG, RELU, SELU, SCALE, SHIFT };
 
@@ -47,13 +48,23 @@ struct Node {
   int leaf;    /* LEAF: its number */
   int arg[2];  /* indices into Expr::nodes */
   std::string name; /* the forward value's spelling in the generated code */
-  std::string constant; /* SCALE, SHIFT: the literal, as printf("%.17g") spells it */
+  int constant;     /* SCALE, SHIFT: which of the call's constants; -1 for the other ops */
 };
 
+/* The constants of an expression are not part of the kernel: the generated code reads them from its
+ * functor (c[0], c[1], ... in the order their ops close in the text), which every launch fills from
+ * the text it was given. One compilation serves every value. */
 struct Expr {
   std::vector<Node> nodes;
+  std::vector<double> constants;
   int root = -1;
   int leaves = 0;
+};
+
+/* What a chain's kernels take as their last argument: the generated functors begin with these members. */
+struct FunctorArgs {
+  double alpha;
+  double c[MAX_CONSTANTS];
 };
 
 thread_local std::string last_error;
@@ -70,6 +81,7 @@ struct Parser {
   Expr& e;
   std::string err;
   int next_leaf = 0; /* leaves must appear as 0, 1, 2, ... in order of first appearance */
+  int depth = 0;
 
   void skip() {
     while (*p == ' ' || *p == '\t') ++p;
@@ -83,12 +95,22 @@ struct Parser {
     ++p;
     return true;
   }
-  int node() {
-    skip();
-    if ((int)e.nodes.size() >= MAX_NODES) {
+  bool room() { /* before every node is added, and on the way down: a nest of unary ops adds none until it turns back */
+    if ((int)e.nodes.size() >= MAX_NODES || depth > MAX_NODES) {
       err = "more than 64 nodes";
-      return -1;
+      return false;
     }
+    return true;
+  }
+  int node() {
+    ++depth;
+    const int made = node_here();
+    --depth;
+    return made;
+  }
+  int node_here() {
+    skip();
+    if (!room()) return -1;
     const char* q = p;
     if (*q == 'x') ++q;
     if (*q >= '0' && *q <= '9') { /* a leaf: 3 or x3 */
@@ -104,7 +126,7 @@ struct Parser {
         err = "more than 8 leaves";
         return -1;
       }
-      e.nodes.push_back(Node{LEAF, v, {-1, -1}, "in[" + std::to_string(v) + "]", ""});
+      e.nodes.push_back(Node{LEAF, v, {-1, -1}, "in[" + std::to_string(v) + "]", -1});
       return (int)e.nodes.size() - 1;
     }
     std::string word;
@@ -130,7 +152,7 @@ struct Parser {
       b = node();
       if (b < 0) return -1;
     }
-    std::string constant;
+    int constant = -1;
     if (op == SCALE || op == SHIFT) { /* a literal second argument: scale(0,0.5) */
       if (!take(',')) return -1;
       skip();
@@ -141,11 +163,15 @@ struct Parser {
         return -1;
       }
       p = end;
-      char text[40];
-      snprintf(text, sizeof text, "%.17g", value);
-      constant = text;
+      if ((int)e.constants.size() >= MAX_CONSTANTS) {
+        err = "more than 8 constants";
+        return -1;
+      }
+      constant = (int)e.constants.size();
+      e.constants.push_back(value);
     }
     if (!take(')')) return -1;
+    if (!room()) return -1;
     e.nodes.push_back(Node{op, -1, {a, b}, "", constant});
     return (int)e.nodes.size() - 1;
   }
@@ -156,7 +182,7 @@ bool parse(const char* text, Expr& e, std::string& err) {
     err = "no expression";
     return false;
   }
-  Parser ps{text, e, "", 0};
+  Parser ps{text, e, "", 0, 0};
   e.root = ps.node();
   if (e.root < 0) {
     err = ps.err;
@@ -175,7 +201,8 @@ bool parse(const char* text, Expr& e, std::string& err) {
   return true;
 }
 
-/* The expression as the cache spells it: bare leaf numbers, no blanks ("add(x0, x1)" -> "add(0,1)"). */
+/* The expression as the cache spells it: bare leaf numbers, no blanks, "#" for a constant
+ * ("scale(add(x0, x1), 0.5)" -> "scale(add(0,1),#)"). */
 void spell(const Expr& e, int n, std::string& out) {
   static const char* const names[] = {"", "add", "sub", "mul", "neg", "relu", "selu", "scale", "shift"};
   const Node& node = e.nodes[n];
@@ -190,7 +217,7 @@ void spell(const Expr& e, int n, std::string& out) {
     out += ',';
     spell(e, node.arg[1], out);
   }
-  if (!node.constant.empty()) out += "," + node.constant;
+  if (node.constant >= 0) out += ",#";
   out += ')';
 }
 
@@ -212,8 +239,8 @@ void forward_lines(Expr& e, int n, int& counter, std::vector<std::string>& lines
     case NEG: rhs = "-" + a; break;
     case RELU: rhs = "mp::relu_value(" + a + ")"; break;
     case SELU: rhs = "mp::selu_value(" + a + ")"; break;
-    case SCALE: rhs = a + " * (P)(" + node.constant + ")"; break;
-    case SHIFT: rhs = a + " + (P)(" + node.constant + ")"; break;
+    case SCALE: rhs = a + " * (P)c[" + std::to_string(node.constant) + "]"; break;
+    case SHIFT: rhs = a + " + (P)c[" + std::to_string(node.constant) + "]"; break;
     default: break;
   }
   node.name = "t" + std::to_string(counter++);
@@ -251,7 +278,7 @@ void sweep(const Expr& e, int n, const std::string& adjoint, int& counter, std::
     case NEG: sweep(e, node.arg[0], fresh("-" + adjoint), counter, lines, leaf_terms); break;
     case RELU: sweep(e, node.arg[0], fresh(adjoint + " * mp::relu_slope(" + v0 + ")"), counter, lines, leaf_terms); break;
     case SELU: sweep(e, node.arg[0], fresh(adjoint + " * mp::selu_slope(" + v0 + ")"), counter, lines, leaf_terms); break;
-    case SCALE: sweep(e, node.arg[0], fresh(adjoint + " * (P)(" + node.constant + ")"), counter, lines, leaf_terms); break;
+    case SCALE: sweep(e, node.arg[0], fresh(adjoint + " * (P)c[" + std::to_string(node.constant) + "]"), counter, lines, leaf_terms); break;
     case SHIFT: sweep(e, node.arg[0], adjoint, counter, lines, leaf_terms); break;
     default: break;
   }
@@ -266,7 +293,7 @@ std::string join(const std::vector<std::string>& v, const char* sep) {
 const char* storage_type(int dtype) { return dtype == MP_R16 ? "_Float16" : dtype == MP_R32 ? "float" : "double"; }
 
 std::string functor(const char* name, int nin, int nout, const std::string& body) {
-  return std::string("struct ") + name + " {\n  double alpha;\n  template <class P> __device__ __forceinline__ void apply(const P (&in)[" +
+  return std::string("struct ") + name + " {\n  double alpha;\n  double c[" + std::to_string(MAX_CONSTANTS) + "];\n  template <class P> __device__ __forceinline__ void apply(const P (&in)[" +
          std::to_string(nin) + "], P (&out)[" + std::to_string(nout) + "]) const {\n" + body + "  }\n};\n\n";
 }
 
@@ -317,7 +344,13 @@ std::string chain_source(Expr& e, int dtype) {
 
 /* ---------------------------------------------------------------- source -> code object */
 
-bool compile(const std::string& source, std::vector<char>& code, std::string& err) {
+std::atomic<unsigned long> compilations{0}; /* hiprtc compilations this process has started */
+
+bool compile(const std::string& generated, std::vector<char>& code, std::string& err) {
+  compilations.fetch_add(1, std::memory_order_relaxed);
+  /* test hook: with MP_CHAIN_BREAK_COMPILE set in the environment every compilation fails, which no
+   * expression that parses can bring about by itself */
+  const std::string source = getenv("MP_CHAIN_BREAK_COMPILE") ? generated + "\n#error MP_CHAIN_BREAK_COMPILE is set\n" : generated;
   hiprtcProgram prog;
   hiprtcResult r = hiprtcCreateProgram(&prog, source.c_str(), "chain.hip", CHAIN_HEADER_COUNT, CHAIN_HEADER_TEXT, CHAIN_HEADER_NAMES);
   if (r != HIPRTC_SUCCESS) {
@@ -366,6 +399,8 @@ struct Chain {
   std::string source;
   std::mutex build;
   std::atomic<bool> compiled{false};
+  std::atomic<bool> failed{false}; /* a compilation that failed is not tried again: `failure` says why */
+  std::string failure;
   std::vector<char> code;
   Loaded on_device[MAX_DEVICES];
 };
@@ -374,9 +409,11 @@ std::mutex cache_lock; /* the map only: held for a lookup or an insertion, never
 std::map<std::pair<std::string, int>, std::unique_ptr<Chain>> cache; /* entries are never removed */
 
 /* The chain of (signature, dtype): its source on first sight, its code object when `compiled` is
- * asked for. NULL with last_error set when it cannot be had. A failure is not cached: it is as
- * cheap to find again as to look up. */
-Chain* chain_for(const char* signature, int dtype, bool compiled) {
+ * asked for. NULL with last_error set when it cannot be had. Text that does not parse is not
+ * cached (it is as cheap to find wrong again as to look up); a compilation that failed is, with its
+ * log, so that a caller who falls back to one launch per op does not pay for it on every call.
+ * constants: the values of this call's text, for the launch. */
+Chain* chain_for(const char* signature, int dtype, bool compiled, std::vector<double>* constants = nullptr) {
   if (dtype != MP_R16 && dtype != MP_R32 && dtype != MP_R64) {
     fail("dtype must be 0 (r16), 1 (r32) or 2 (r64)");
     return nullptr;
@@ -390,6 +427,7 @@ Chain* chain_for(const char* signature, int dtype, bool compiled) {
   }
   std::string canonical;
   spell(e, e.root, canonical);
+  if (constants) *constants = e.constants;
   Chain* c = nullptr;
   {
     std::lock_guard<std::mutex> hold(cache_lock);
@@ -405,10 +443,16 @@ Chain* chain_for(const char* signature, int dtype, bool compiled) {
   }
   if (compiled && !c->compiled.load(std::memory_order_acquire)) {
     std::lock_guard<std::mutex> hold(c->build);
+    if (c->failed.load(std::memory_order_relaxed)) {
+      fail(c->failure);
+      return nullptr;
+    }
     if (!c->compiled.load(std::memory_order_relaxed)) {
       std::vector<char> code;
       if (!compile(c->source, code, err)) {
-        fail(std::string("chain \"") + signature + "\": " + err);
+        c->failure = std::string("chain \"") + canonical + "\": " + err;
+        c->failed.store(true, std::memory_order_release);
+        fail(c->failure);
         return nullptr;
       }
       c->code = std::move(code);
@@ -455,7 +499,7 @@ int layout_index(int layout) { return layout == mp::EW_ALIGNED ? 0 : layout == m
 
 /* One launch: kind 0 forward, 1 reverse that overwrites, 2 reverse that blends. */
 int enqueue(Chain* c, int kind, int dtype, const void* const* in, int nin, void* const* out, int nout, double alpha,
-            size_t n, hipStream_t stream) {
+            const std::vector<double>& constants, size_t n, hipStream_t stream) {
   if (n == 0) return 0;
   for (int s = 0; s < nin; ++s)
     if (in[s] == nullptr) return fail("a NULL operand");
@@ -471,7 +515,10 @@ int enqueue(Chain* c, int kind, int dtype, const void* const* in, int nin, void*
   for (int s = 0; s < nin; ++s) ptrs[s] = in[s];
   for (int s = 0; s < nout; ++s) ptrs[nin + s] = out[s];
   unsigned head = plan.head;
-  void* params[4] = {ptrs, &n, &head, &alpha};
+  FunctorArgs args{};
+  args.alpha = alpha;
+  for (size_t i = 0; i < constants.size() && i < (size_t)MAX_CONSTANTS; ++i) args.c[i] = constants[i];
+  void* params[4] = {ptrs, &n, &head, &args};
   const hipError_t r = hipModuleLaunchKernel(l->fn[kind * 3 + layout_index(plan.layout)], plan.blocks, 1, 1, mp::EW_BLOCK, 1, 1,
                                              0, stream, params, nullptr);
   if (r != hipSuccess) return fail(std::string("hipModuleLaunchKernel: ") + hipGetErrorString(r));
@@ -505,24 +552,26 @@ extern "C" const void* mpChainCodeObject(const char* signature, int dtype, len_t
 
 extern "C" int mpChainForward(const char* signature, int dtype, const void* const* x, void* out, len_t n, StreamContext stream) {
   if (x == nullptr) return fail("no operand array");
-  Chain* c = chain_for(signature, dtype, true);
+  std::vector<double> constants;
+  Chain* c = chain_for(signature, dtype, true, &constants);
   if (c == nullptr) return 1;
   void* outs[1] = {out};
-  return enqueue(c, 0, dtype, x, c->leaves, outs, 1, 0.0, (size_t)n, get_stream(stream));
+  return enqueue(c, 0, dtype, x, c->leaves, outs, 1, 0.0, constants, (size_t)n, get_stream(stream));
 }
 
 extern "C" int mpChainReverse(const char* signature, int dtype, const void* const* x, const void* out_grads, void* const* g,
                               double alpha, len_t n, StreamContext stream) {
   if (x == nullptr || g == nullptr) return fail("no operand array");
-  Chain* c = chain_for(signature, dtype, true);
+  std::vector<double> constants;
+  Chain* c = chain_for(signature, dtype, true, &constants);
   if (c == nullptr) return 1;
   const int k = c->leaves;
   const void* in[2 * MAX_LEAVES + 1];
   for (int i = 0; i < k; ++i) in[i] = x[i];
   in[k] = out_grads;
-  if (alpha == 0.0) return enqueue(c, 1, dtype, in, k + 1, g, k, 0.0, (size_t)n, get_stream(stream));
+  if (alpha == 0.0) return enqueue(c, 1, dtype, in, k + 1, g, k, 0.0, constants, (size_t)n, get_stream(stream));
   for (int i = 0; i < k; ++i) in[k + 1 + i] = g[i];
-  return enqueue(c, 2, dtype, in, 2 * k + 1, g, k, alpha, (size_t)n, get_stream(stream));
+  return enqueue(c, 2, dtype, in, 2 * k + 1, g, k, alpha, constants, (size_t)n, get_stream(stream));
 }
 
 extern "C" len_t mpChainCacheSize(void) {
@@ -531,5 +580,7 @@ extern "C" len_t mpChainCacheSize(void) {
   for (const auto& kv : cache) n += kv.second->compiled.load(std::memory_order_acquire) ? 1 : 0;
   return n;
 }
+
+extern "C" len_t mpChainCompilations(void) { return (len_t)compilations.load(std::memory_order_relaxed); }
 
 extern "C" const char* mpChainError(void) { return last_error.c_str(); }

@@ -242,6 +242,21 @@ static int fused_chain(mp::Stream stream) {
     CHECK(R->launches == l + 2);
     dump("any_affine_da", ra.native_grad<float>()); dump("any_affine_dc", rc.native_grad<float>());
     CHECK(R->runtime_chains_.size() == 2);
+    /* the same expression with other constants (a step size that changes every step) is the same kernel
+     * with other arguments: nothing is compiled, no new shape is recorded */
+    {
+      const len_t compiled = mpChainCacheSize(), started = mpChainCompilations();
+      R->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+      l = R->launches;
+      mp::Tensor f5 = mp::ops::relu(mp::ops::translate(mp::ops::dilate(mp::ops::hadamard(ra, rc), -0.75), 0.25));
+      dump("any_affine2", f5.native<float>());
+      CHECK(R->launches == l + 1);
+      f5.reverse(mp::ReverseCleanup::free);
+      dump("any_affine2_da", ra.native_grad<float>()); dump("any_affine2_dc", rc.native_grad<float>());
+      CHECK(R->runtime_chains_.size() == 2);
+      CHECK(mpChainCacheSize() == compiled);
+      CHECK(mpChainCompilations() == started);
+    }
     /* a single op stays the op's own kernel and keeps its own reverse */
     l = R->launches;
     mp::Tensor s3 = mp::ops::sub(rc, rd);

@@ -320,21 +320,22 @@ static const char* pending_name(Pending op) {
 
 /* The expression below t, as the chain table spells it: pending nodes of this graph become
  * op(...), everything else a leaf numbered in order of first appearance (the same tensor keeps
- * its number). Gives up (returns false) beyond eight leaves or 64 nodes. */
-static bool spell(Graph* g, Tensor t, std::string& out, std::vector<Tensor>& leaves, int& budget) {
+ * its number). Gives up (returns false) beyond eight leaves or 64 nodes. shape_only: the constants of
+ * dilate and translate are spelled "#" (expressions that differ in them only are one kernel). */
+static bool spell(Graph* g, Tensor t, std::string& out, std::vector<Tensor>& leaves, int& budget, bool shape_only = false) {
   if (--budget < 0) return false;
   if (is_pending(t) && t.ptr == g) {
     const Graph::Node& node = g->nodes_[t.idx];
     out += pending_name(node.pending);
     out += '(';
-    if (!spell(g, node.in0, out, leaves, budget)) return false;
+    if (!spell(g, node.in0, out, leaves, budget, shape_only)) return false;
     if (node.pending == Pending::dilate || node.pending == Pending::translate) {
-      char text[40]; /* the constant as every generator of chains spells it */
+      char text[40]; /* the constant as every generator of chains spells it; "#" when only the shape is asked for */
       snprintf(text, sizeof text, ",%.17g", node.value);
-      out += text;
+      out += shape_only ? ",#" : text;
     } else if (node.pending != Pending::selu && node.pending != Pending::relu) {
       out += ',';
-      if (!spell(g, node.in1, out, leaves, budget)) return false;
+      if (!spell(g, node.in1, out, leaves, budget, shape_only)) return false;
     }
     out += ')';
     return true;
@@ -409,15 +410,21 @@ void materialise(Tensor t) {
         if (leaves[i].len() == 0) panic("materialise: an input of a pending node was freed");
         x[i] = leaves[i].data_ptr();
       }
+      { /* the shapes this graph had compiled: a constant that changes from call to call adds nothing */
+        std::string shape;
+        std::vector<Tensor> again;
+        int room = 64;
+        spell(g, t, shape, again, room, true);
+        size_t idx = 0;
+        while (idx < g->runtime_chains_.size() && g->runtime_chains_[idx] != shape) ++idx;
+        if (idx == g->runtime_chains_.size()) g->runtime_chains_.push_back(shape);
+      }
       void* out = take_buffer();
       if (mpChainForward(signature.c_str(), (int)key, x, out, (len_t)n, ctx) != 0) panic(mpChainError());
       g->launches++;
-      if (g->mode == Mode::train) {
-        size_t idx = 0;
-        while (idx < g->runtime_chains_.size() && g->runtime_chains_[idx] != signature) ++idx;
-        if (idx == g->runtime_chains_.size()) g->runtime_chains_.push_back(signature);
+      if (g->mode == Mode::train) { /* the reverse gets the text itself, constants included */
         std::vector<OpDatum> args(leaves.begin(), leaves.end());
-        args.push_back(OpDatum((double)idx));
+        args.push_back(OpDatum(signature));
         args.push_back(t);
         attach_op(t, runtime_chain_reverse, std::move(args));
       }
@@ -544,13 +551,12 @@ static void chain_reverse(const std::vector<OpDatum>& a) {
   g->launches++;
 }
 
-/* The same for an expression compiled at run time: args = leaves..., index into the graph's
- * runtime_chains_, output. */
+/* The same for an expression compiled at run time: args = leaves..., the expression's text, output. */
 static void runtime_chain_reverse(const std::vector<OpDatum>& a) {
   const size_t k = a.size() - 2;
   const Tensor out = a[k + 1].t;
   Graph* g = out.ptr;
-  const std::string& signature = g->runtime_chains_[(size_t)a[k].s];
+  const std::string& signature = a[k].e;
   bool any = false;
   for (size_t i = 0; i < k; ++i) any = any || a[i].t.has_grad();
   void* x[8];

@@ -202,7 +202,8 @@ class Graph {
   Mode mode = Mode::train;
   Stream stream = nullptr;
   Fusion fusion = Fusion::listed;
-  /* expressions this graph had compiled at run time; a reverse entry refers to them by index */
+  /* the shapes of the expressions this graph had compiled at run time (constants spelled "#": a value
+   * that changes from call to call is an argument of the same kernel) */
   std::vector<std::string> runtime_chains_;
 
   /* kernels enqueued through this graph so far (fusion is observable through it) */

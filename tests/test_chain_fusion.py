@@ -18,6 +18,20 @@ EXTRA = ["mul(add(x0,x0),x1)", "relu(sub(mul(x0,x1),neg(x0)))", "selu(selu(add(x
          "sub(mul(x0,x1),mul(x2,add(x3,add(x4,add(x5,add(x6,x7))))))"]
 
 
+def _literal_constants(expr):
+    """The constants of an expression in the order their ops close in the text, which is the order
+    the run-time generator numbers them in (c[0], c[1], ...)."""
+    return [m.group(1) for m in re.finditer(r",\s*([-+]?(?:\d+\.?\d*|\.\d+)(?:[eE][-+]?\d+)?)\s*\)", expr)
+            if True]
+
+
+def _with_literals(lines, expr):
+    """Lines of the run-time generator with each (P)c[i] replaced by the literal the build-time
+    generator writes in its place."""
+    values = [chaingen.constant_text(float(v)) for v in _literal_constants(expr)]
+    return [re.sub(r"\(P\)c\[(\d+)\]", lambda m: f"(P)({values[int(m.group(1))]})", l) for l in lines]
+
+
 def _functor_bodies(source):
     """{functor name: [stripped statement lines]} of a generated source."""
     out = {}
@@ -58,9 +72,12 @@ def test_the_runtime_generator_writes_the_build_time_generators_lines(expr):
     got = _functor_bodies(src.decode())
     want_f = _functor_bodies(chaingen.forward_source("c", expr))
     want_r = _functor_bodies(chaingen.reverse_source("c", expr))
-    assert got["ChainForward"] == want_f["CFn_Scalar"]
-    assert got["ChainReverseOverwrite"] == want_r["CReverseOverwriteFn_Scalar"]
-    assert got["ChainReverseBlend"] == want_r["CReverseBlendFn_Scalar"]
+    # the run-time kernels take their constants as arguments (c[i]); with the literals put back the
+    # arithmetic is the build-time generator's, line for line
+    assert _with_literals(got["ChainForward"], expr) == want_f["CFn_Scalar"]
+    assert _with_literals(got["ChainReverseOverwrite"], expr) == want_r["CReverseOverwriteFn_Scalar"]
+    assert _with_literals(got["ChainReverseBlend"], expr) == want_r["CReverseBlendFn_Scalar"]
+    assert "double c[8];" in src.decode()
 
 
 def test_random_expressions_differentiate_like_autograd():
@@ -72,7 +89,7 @@ def test_random_expressions_differentiate_like_autograd():
         assert lib.mpChainLeaves(expr.encode()) == k
         src = lib.mpChainSource(expr.encode(), 2)
         assert src, (expr, lib.mpChainError())
-        bodies = _functor_bodies(src.decode())
+        bodies = {name: _with_literals(lines, expr) for name, lines in _functor_bodies(src.decode()).items()}
         xs = [r.uniform(-2, 2, 200) for _ in range(k)]
         up = r.normal(0, 1, 200)
         old = [r.normal(0, 1, 200) for _ in range(k)]
@@ -116,7 +133,9 @@ def test_every_dtype_compiles_and_is_cached_once(dtype):
     ("add(1,0)", "order of first appearance"), ("add(0,2)", "order of first appearance"),
     ("add(0,1))", "trailing text"), ("add(0 1)", "expected ','"), ("", "unknown op"),
     ("add(add(add(add(0,1),add(2,3)),add(add(4,5),add(6,7))),8)", "more than 8 leaves"),
-    ("scale(0)", "expected ','"), ("scale(0,x1)", "finite number"), ("shift(0,abc)", "finite number"), ("scale(0,inf)", "finite number")])
+    ("scale(0)", "expected ','"), ("scale(0,x1)", "finite number"), ("shift(0,abc)", "finite number"), ("scale(0,inf)", "finite number"),
+    ("shift(" * 9 + "0" + ",1)" * 9, "more than 8 constants"),
+    ("neg(" * 65 + "0" + ")" * 65, "more than 64 nodes"), ("neg(" * 100000 + "0" + ")" * 100000, "more than 64 nodes")])
 def test_bad_expressions_are_refused_with_a_reason(bad, why):
     lib = ffi.load_fusion()
     n = lib.mpChainCacheSize()
@@ -137,7 +156,8 @@ def test_the_fusion_library_exports_what_its_header_declares():
     lib = ffi.load_fusion()
     names = [n for _, n, _ in ffi.parse_declarations(ffi.os.path.join(ffi.ROOT, "include", "chain_fusion.h"))]
     assert sorted(names) == sorted(["mpChainForward", "mpChainReverse", "mpChainCompile", "mpChainLeaves",
-                                    "mpChainSource", "mpChainCodeObject", "mpChainCacheSize", "mpChainError"])
+                                    "mpChainSource", "mpChainCodeObject", "mpChainCacheSize", "mpChainCompilations",
+                                    "mpChainError"])
     for n in names:
         assert getattr(lib, n)
 
@@ -147,7 +167,7 @@ def test_several_threads_compile_at_once():
     expression is compiled once, and a thread's error text is its own."""
     import threading
     lib = ffi.load_fusion()
-    exprs = [f"relu(shift(mul(0,1),{k}.25))".encode() for k in range(4)]
+    exprs = [f"relu(shift({op}(0,1),0.25))".encode() for op in ("mul", "add", "sub")] + [b"neg(shift(mul(0,1),0.25))"]
     before = lib.mpChainCacheSize()
     results = [None] * 8
 
@@ -176,3 +196,44 @@ def test_missing_operand_arrays_are_refused():
     assert "operand array" in lib.mpChainError().decode()
     assert lib.mpChainReverse(b"add(0,1)", 1, None, None, None, 0.0, 16, ctx) != 0
     assert "operand array" in lib.mpChainError().decode()
+
+
+def test_constants_are_arguments_not_part_of_the_kernel():
+    """Expressions that differ in their constants only are one cache entry and one compilation."""
+    lib = ffi.load_fusion()
+    assert lib.mpChainCompile(b"selu(scale(add(0,1),0.5))", 1) == 0, lib.mpChainError()
+    n, started = lib.mpChainCacheSize(), lib.mpChainCompilations()
+    for value in ("0.25", "-3", "1e-3", "7.5e2"):
+        assert lib.mpChainCompile(f"selu(scale(add(0,1),{value}))".encode(), 1) == 0
+    assert lib.mpChainCacheSize() == n and lib.mpChainCompilations() == started
+    a = lib.mpChainSource(b"selu(scale(add(0,1),0.5))", 1)
+    b = lib.mpChainSource(b"selu(scale(add(0,1),-3))", 1)
+    assert a == b and b"c[0]" in a and b"0.5" not in a.split(b"namespace {")[1].split(b"}  // namespace")[0]
+
+
+def test_a_failed_compilation_is_not_tried_again():
+    """With the library's test hook set every compilation fails; the second call for the same
+    expression returns the first one's reason without starting another compilation. Run in a child
+    process so that the hook does not reach the other tests."""
+    import subprocess
+    import sys
+    code = (
+        "import os, sys\n"
+        "os.environ['MP_CHAIN_BREAK_COMPILE'] = '1'\n"
+        f"sys.path.insert(0, {ffi.ROOT!r})\n"
+        "from metaphor_amd import ffi\n"
+        "lib = ffi.load_fusion()\n"
+        "e = b'relu(mul(neg(0),add(1,0)))'\n"
+        "assert lib.mpChainCompile(e, 1) != 0\n"
+        "first = lib.mpChainError().decode()\n"
+        "assert 'MP_CHAIN_BREAK_COMPILE' in first, first\n"
+        "started = lib.mpChainCompilations()\n"
+        "assert started == 1\n"
+        "assert lib.mpChainCompile(e, 1) != 0 and lib.mpChainError().decode() == first\n"
+        "assert lib.mpChainCodeObject(e, 1, None) is None\n"
+        "assert lib.mpChainCompilations() == started\n"
+        "assert lib.mpChainCacheSize() == 0\n"
+        "assert lib.mpChainSource(e, 1)\n"
+        "print('ok')\n")
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0 and "ok" in res.stdout, res.stderr[-2000:]

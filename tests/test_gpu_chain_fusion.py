@@ -151,9 +151,40 @@ def test_output_may_alias_a_leaf_and_empty_and_null_calls_enqueue_nothing():
     assert torch.equal(a.t, before)
 
 
-def test_fusion_at_full_rate_of_the_build_time_chain():
-    """2^26 r32 elements: the run-time kernel of the benchmark chain takes the time of the build-time
-    one (same engine, same functor), measured with events around 10 launches each."""
+def test_one_kernel_serves_every_value_of_a_constant():
+    """relu(c1 * (a * b) + c2) with four pairs of constants: one compilation, every result against
+    fp64 numpy on the storage-rounded inputs (a constant reaches the kernel as an argument)."""
+    r = np.random.default_rng(9)
+    f = G.ffi.load_fusion()
+    for dtype in DTYPES:
+        n = 30011
+        a, b = G.dev(r.uniform(-2, 2, n), dtype), G.dev(r.uniform(-2, 2, n), dtype)
+        up = G.dev(r.normal(0, 1, n), dtype)
+        ha, hb, hup = (G.host(t.t).astype(np.float64) for t in (a, b, up))
+        sizes = set()
+        for c1, c2 in [(0.125, 0.5), (-0.75, 0.25), (3.0, -1e-3), (1e-2, 7.0)]:
+            expr = f"relu(shift(scale(mul(0,1),{c1!r}),{c2!r}))"
+            G.say(f"chain constants dtype={dtype} c1={c1} c2={c2}")
+            out = G.Guarded((n,), dtype)
+            ga, gb = G.Guarded((n,), dtype), G.Guarded((n,), dtype)
+            assert G.chain_forward(expr, [a.t, b.t], out.t) == 0, G.chain_error()
+            assert G.chain_reverse(expr, [a.t, b.t], up.t, [ga.t, gb.t], 0.0) == 0, G.chain_error()
+            sizes.add(int(f.mpChainCacheSize()))
+            pre = c1 * (ha * hb) + c2
+            on = (pre >= 0) * hup
+            mag = abs(c1) * np.abs(ha * hb) + abs(c2)
+            G.compare(out.t, np.where(pre >= 0, pre, 0.0), dtype, f"{expr} value", rowwise=False, scale=mag)
+            G.compare(ga.t, on * c1 * hb, dtype, f"{expr} da", rowwise=False, scale=np.abs(hup * c1 * hb))
+            G.compare(gb.t, on * c1 * ha, dtype, f"{expr} db", rowwise=False, scale=np.abs(hup * c1 * ha))
+            for g in (out, ga, gb):
+                g.check(expr)
+        assert len(sizes) == 1, "another value of a constant must not be another compilation"
+
+
+def test_rate_of_a_run_time_kernel_beside_the_build_time_one():
+    """2^26 r32 elements: the run-time kernel of the benchmark chain beside the build-time one (same
+    engine, same functor), events around 10 launches each. Printed, not asserted: wall-clock checks
+    belong to bench.py (its `chain` workload records the ratio and fails --strict on more than 10 %)."""
     n = 1 << 26
     xs = [torch.empty(n, device="cuda").uniform_(-2, 2) for _ in range(4)]
     out = torch.empty(n, device="cuda")
@@ -174,5 +205,4 @@ def test_fusion_at_full_rate_of_the_build_time_chain():
     t_run = timed(lambda: G.chain_forward(expr, xs, out))
     t_build = timed(lambda: G.fused(*xs, out))
     print(f"[chain-rate] run-time {t_run * 1e3:.1f} us, build-time {t_build * 1e3:.1f} us, "
-          f"{20 * n / t_run / 1e6:.0f} GB/s")
-    assert t_run < 1.1 * t_build + 0.02
+          f"ratio {t_run / t_build:.3f}, {20 * n / t_run / 1e6:.0f} GB/s")

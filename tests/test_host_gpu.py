@@ -70,6 +70,12 @@ def test_host_library_end_to_end(tmp_path):
     _cmp(_load(d, "any_affine"), np.where(pre >= 0, pre, 0.0), "run-time chain with constants", rowwise=False)
     _cmp(_load(d, "any_affine_da"), on * 0.125 * c64_, "run-time chain with constants da", rowwise=False)
     _cmp(_load(d, "any_affine_dc"), on * 0.125 * a64_, "run-time chain with constants dc", rowwise=False)
+    # the same kernel with other constants (host_check asserts that nothing was compiled for it)
+    pre2 = -0.75 * (a64_ * c64_) + 0.25
+    on2 = (pre2 >= 0).astype(np.float64)
+    _cmp(_load(d, "any_affine2"), np.where(pre2 >= 0, pre2, 0.0), "run-time chain, other constants", rowwise=False)
+    _cmp(_load(d, "any_affine2_da"), on2 * -0.75 * c64_, "run-time chain, other constants da", rowwise=False)
+    _cmp(_load(d, "any_affine2_dc"), on2 * -0.75 * a64_, "run-time chain, other constants dc", rowwise=False)
 
     # other generated chains (fp64 compositions of the pinned oracle pieces; upstream gradient = 1)
     a64, b64, c64, d64 = (z.astype(np.float64) for z in (a, b, c, dd))
