@@ -51,8 +51,30 @@ inline void mpHandleHipError(hipError_t err, const char* file, int line) {
   }
 }
 
+#ifdef MP_DIAGNOSTICS
+/* Test build only: what a row launcher decided, recorded instead of launched. With `dry` set a
+ * launcher runs its whole dispatch (with `cus` in place of the GPU's compute-unit count), notes the
+ * kernel it would enqueue and returns before the launch, so the dispatch can be swept on a machine
+ * without a GPU. kind: 0 short rows, 1 resident, 2 rows in pairs, 3 wavefront groups, 4 shared rows,
+ * 5 shared rows pipelined, 6 two passes, 7 rows that peel differently. */
+struct MpPlanNote {
+  long long kind, group, packs_per_thread, rows_per_block, grid, block, cluster, chunk_packs, workspace_bytes;
+};
+struct MpPlanProbe {
+  bool dry = false, noted = false;
+  int cus = 0;
+  MpPlanNote note{};
+};
+inline MpPlanProbe& mp_plan_probe() {
+  static thread_local MpPlanProbe probe;
+  return probe;
+}
+/* a launch that the runtime rejects (bad grid, missing code object) must not pass silently */
+#define MP_CHECK_LAUNCH() do { if (!mp_plan_probe().dry) HIP_ASSERT(hipGetLastError()); } while (0)
+#else
 /* a launch that the runtime rejects (bad grid, missing code object) must not pass silently */
 #define MP_CHECK_LAUNCH() HIP_ASSERT(hipGetLastError())
+#endif
 #endif /* MP_HOST_SIDE */
 
 namespace mp {
@@ -466,6 +488,26 @@ template <class T, int W, int G, int NV, bool RAGGED> struct RowTile {
  * ------------------------------------------------------------------------------------- */
 
 #ifdef MP_HOST_SIDE
+/* Before every launch of a row kernel: `if (note_plan(...)) return;`. Nothing in the library as
+ * shipped; in the test build it records the decision and, on a dry run, says "do not launch". */
+#ifdef MP_DIAGNOSTICS
+inline bool note_plan(int kind, int group, int packs_per_thread, int rows_per_block, size_t grid, size_t block,
+                      int cluster = 1, int chunk_packs = 0, size_t workspace_bytes = 0) {
+  MpPlanProbe& p = mp_plan_probe();
+  if (!p.dry) return false;
+  p.note = MpPlanNote{kind, group, packs_per_thread, rows_per_block, (long long)grid, (long long)block, cluster, chunk_packs,
+                      (long long)workspace_bytes};
+  p.noted = true;
+  return true;
+}
+inline bool plan_dry_run() { return mp_plan_probe().dry; }
+#else
+template <class... A> constexpr bool note_plan(A...) { return false; }
+constexpr bool plan_dry_run() { return false; }
+#endif
+enum PlanKind { PLAN_SHORT = 0, PLAN_RESIDENT = 1, PLAN_PAIRED = 2, PLAN_ANY = 3, PLAN_CLUSTER = 4, PLAN_DEEP = 5,
+                PLAN_STREAM = 6, PLAN_LOOSE = 7 };
+
 /* Packs a thread must hold so that a G-thread group covers `packs` packs; 0 = too long. */
 inline int packs_per_thread(size_t packs, int G, int max_nv) {
   for (int nv = 1; nv <= max_nv; nv *= 2)
@@ -475,6 +517,9 @@ inline int packs_per_thread(size_t packs, int G, int max_nv) {
 
 /* The GPU's compute-unit count, read once per process. */
 inline int compute_units() {
+#ifdef MP_DIAGNOSTICS
+  if (mp_plan_probe().dry && mp_plan_probe().cus > 0) return mp_plan_probe().cus;
+#endif
   static int cus = [] {
     int dev = 0, n = 0;
     HIP_ASSERT(hipGetDevice(&dev));

@@ -97,4 +97,49 @@ extern "C" void mpSetClusterWords(len_t own) {
   mp::require(own <= 1, "mpSetClusterWords: 0 or 1");
   mp::cluster_tuning().own_words = (int)own;
 }
+
+// Diagnostic: what the row launchers decide for [m, n] rows of a dtype on a GPU of `cus` compute
+// units, for every n in [n_lo, n_hi), without a GPU: each launcher runs its whole dispatch on a dry
+// run (kernel_header.h: MpPlanNote) and the kernel it would enqueue is written to notes[n - n_lo],
+// the bytes the matching workspace-size function asks for to sizes[n - n_lo]. op: 0 softmax
+// forward, 1 softmax reverse, 2 RMSNorm forward, 3 RMSNorm reverse. shift: 0 every operand 16-byte
+// aligned, 1 every operand one element past that, 2 the output one element past the inputs.
+// Operands are made-up addresses that nothing dereferences. Returns how many n were noted.
+#include "kernel_decls.h"
+extern "C" len_t mpDescribeRowPlans(len_t op, len_t dtype, len_t m, len_t n_lo, len_t n_hi, len_t cus, len_t shift,
+                                    MpPlanNote* notes, len_t* sizes) {
+  mp::require(op <= 3 && dtype <= 2 && shift <= 2 && cus >= 1 && n_lo <= n_hi, "mpDescribeRowPlans: bad arguments");
+  const size_t elem = dtype == MP_R16 ? 2 : dtype == MP_R32 ? 4 : 8;
+  auto at = [&](int k, bool shifted) {
+    return reinterpret_cast<void*>((uintptr_t)0x100000000000ull + (uintptr_t)k * 0x4000000000ull + (shifted ? elem : 0));
+  };
+  const bool in_shift = shift == 1, out_shift = shift >= 1;
+  void *a = at(0, in_shift), *b = at(1, in_shift), *g = at(2, in_shift), *o = at(3, out_shift), *o2 = at(4, false), *ws = at(5, false);
+  StreamContext ctx{};
+  MpPlanProbe& probe = mp_plan_probe();
+  probe.dry = true;
+  probe.cus = (int)cus;
+  len_t noted = 0;
+  for (len_t n = n_lo; n < n_hi; ++n) {
+    probe.noted = false;
+    probe.note = MpPlanNote{-1, 0, 0, 0, 0, 0, 0, 0, 0};
+    len_t need = 0;
+#define MP_BY_DTYPE(STEM, ...) \
+    do { if (dtype == MP_R16) launch_##STEM##_r16(__VA_ARGS__); else if (dtype == MP_R32) launch_##STEM##_r32(__VA_ARGS__); \
+         else launch_##STEM##_r64(__VA_ARGS__); } while (0)
+    switch (op) {
+      case 0: need = mpSoftmaxScratchBytes(dtype, m, n); MP_BY_DTYPE(softmax_ij_j, a, o, ws, m, n, ctx); break;
+      case 1: need = mpSoftmaxReverseScratchBytes(dtype, m, n); MP_BY_DTYPE(softmax_ij_j_reverse, a, b, o, ws, 0.0, m, n, ctx); break;
+      case 2: need = mpRmsnormScratchBytes(dtype, m, n); MP_BY_DTYPE(rmsnorm_ij_j, a, g, o, ws, 1e-6, m, n, ctx); break;
+      default: need = mpRmsnormReverseScratchBytes(dtype, m, n); MP_BY_DTYPE(rmsnorm_ij_j_reverse, a, g, b, o, o2, ws, 1e-6, 0.0, m, n, ctx); break;
+    }
+#undef MP_BY_DTYPE
+    notes[n - n_lo] = probe.note;
+    sizes[n - n_lo] = need;
+    noted += probe.noted ? 1 : 0;
+  }
+  probe.dry = false;
+  probe.cus = 0;
+  return noted;
+}
 #endif

@@ -1429,6 +1429,7 @@ template <class T>
 inline void sum_partial_rows(const typename precision<T>::type* partials, T* dst, double alpha, unsigned rows,
                              size_t n, hipStream_t stream) {
   using P = typename precision<T>::type;
+  if (plan_dry_run()) return;
   /* wide loads need 16-byte aligned partial rows: fp32 accumulators, n % 4 == 0, aligned scratch */
   const bool wide = sizeof(P) == 4 && (n % 4) == 0 && aligned16(partials);
   if (wide) {
@@ -1576,6 +1577,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   const size_t cap = (size_t)compute_units() * 2;
   if (rmsnorm_short_rows<T>(n, false)) {
     for_short_row(n, W, [&]<int G, bool CUT>() {
+      if (note_plan(PLAN_SHORT, G, 1, SHORT_THREADS / G, short_row_grid(m, G), SHORT_THREADS)) return;
       rmsnorm_fwd_short<T, W, G, CUT><<<dim3(short_row_grid(m, G)), dim3(SHORT_THREADS), 0, stream>>>(
           x, gain, y, (P)eps, m, (unsigned)n, short_rows_share_lines<T>(n, G));
     });
@@ -1595,6 +1597,9 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
       Word* slots = static_cast<Word*>(scratch);
       const int ppb = cluster_chunk_packs((n + W - 1) / W, C, (size_t)CLUSTER_THREADS * NORM_CLUSTER_NV, CLUSTER_SKEW_MAX);
       require(ppb <= CLUSTER_THREADS * NORM_CLUSTER_NV, "rmsnorm: cluster chunk exceeds the register tile");
+      if (note_plan(PLAN_CLUSTER, CLUSTER_THREADS, NORM_CLUSTER_NV, 1, m * C, CLUSTER_THREADS, C, ppb,
+                    C > 1 ? m * (size_t)C * sizeof(Word) : 0))
+        return;
       if (C > 1) {
         const size_t words = m * (size_t)C;
         cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
@@ -1628,6 +1633,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   if (eight_rows) {
     const size_t need = (m + NORM_BLOCK / 128 - 1) / (NORM_BLOCK / 128);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
+    if (note_plan(PLAN_RESIDENT, 128, 2, NORM_BLOCK / 128, grid.x, block.x)) return;
     rmsnorm_fwd_resident<T, W, 128, 2, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
     MP_CHECK_LAUNCH();
     return;
@@ -1639,6 +1645,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
       const int rpb = NORM_BLOCK / WAVE / gw;
       const size_t need = (m + rpb - 1) / rpb;
       const dim3 grid((unsigned)(need < cap ? need : cap)), block(rpb * gw * WAVE);
+      if (note_plan(PLAN_ANY, gw * WAVE, shot.NV, rpb, grid.x, block.x)) return;
       if (shot.NV == 1) rmsnorm_fwd_any<T, W, 1><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
       else rmsnorm_fwd_any<T, W, 2><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
       MP_CHECK_LAUNCH();
@@ -1653,6 +1660,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
         const size_t need = (m + ONESHOT / G - 1) / (ONESHOT / G);
         require(need < 0x7fffffffull, "rmsnorm: too many rows for one grid");
         const dim3 grid((unsigned)need), block(ONESHOT);
+        if (note_plan(PLAN_RESIDENT, G, NV, ONESHOT / G, grid.x, block.x)) return;
         if (loose) rmsnorm_fwd_resident<T, W, G, NV, true, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
         else rmsnorm_fwd_resident<T, W, G, NV, false, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
       }
@@ -1670,10 +1678,11 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
+    if (note_plan(PLAN_RESIDENT, G, NV, NORM_BLOCK / G, grid.x, block.x)) return;
     if (loose) rmsnorm_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
     else rmsnorm_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
   });
-  if (!resident) {
+  if (!resident && !note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, m < cap ? m : cap, STREAM_THREADS)) {
     const size_t grid = m < cap ? m : cap;
     if (mismatch) rmsnorm_fwd_stream<T, W, true><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
     else rmsnorm_fwd_stream<T, W><<<dim3((unsigned)grid), dim3(STREAM_THREADS), 0, stream>>>(x, gain, y, (P)eps, m, n);
@@ -1739,6 +1748,7 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
         const size_t need_any = (m + rpb - 1) / rpb, one_per_cu = (size_t)compute_units();
         rows = (unsigned)(need_any < one_per_cu ? need_any : one_per_cu);
         const dim3 grid(rows), block(rpb * gw * WAVE);
+        if (note_plan(PLAN_ANY, gw * WAVE, 2, rpb, grid.x, block.x, 1, 0, (size_t)rows * n * sizeof(P))) return;
         if (blend) rmsnorm_rev_paired_any<T, W, 2, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
         else rmsnorm_rev_paired_any<T, W, 2, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, gw);
         return;
@@ -1755,6 +1765,7 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
         const size_t need_any = (m + rpb - 1) / rpb, one_per_cu = (size_t)compute_units();
         rows = (unsigned)(need_any < one_per_cu ? need_any : one_per_cu);
         const dim3 grid(rows), block(rpb * gw * WAVE);
+        if (note_plan(PLAN_ANY, gw * WAVE, NV, rpb, grid.x, block.x, 1, 0, (size_t)rows * n * sizeof(P))) return;
         /* a third register set for two-byte types and for the shortest rows of four-byte ones (interleaved
          * repeats: r16 n = 1280 4.71 -> 5.99 TB/s, 3072 5.55 -> 5.87, 2560 equal; r32 n = 640 5.36 -> 5.71,
          * 1280 equal, 1536 5.86 -> 5.68) */
@@ -1773,6 +1784,7 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
       const size_t one_per_cu = (size_t)compute_units();
       rows = (unsigned)(need < one_per_cu ? need : one_per_cu);
       const dim3 grid(rows), block(NORM_BLOCK);
+      if (note_plan(PLAN_PAIRED, G, NV, NORM_BLOCK / G, grid.x, block.x, 1, 0, (size_t)rows * n * sizeof(P))) return;
       const bool exact = n == (size_t)G * NV * W;
       /* a third register set where a row is short enough that two sets in flight do not cover the
        * memory latency (interleaved repeats: r16 n = 1024 5.45 -> 6.09 TB/s, 2048 5.89 -> 6.08, 4096
@@ -1787,6 +1799,7 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
     } else {
       rows = (unsigned)(need < max_rows ? need : max_rows);
       const dim3 grid(rows), block(NORM_BLOCK);
+      if (note_plan(PLAN_RESIDENT, G, NV, NORM_BLOCK / G, grid.x, block.x, 1, 0, (size_t)rows * n * sizeof(P))) return;
       if (blend) rmsnorm_rev_resident<T, W, G, NV, true, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, rows_share_lines<T>(n));
       else rmsnorm_rev_resident<T, W, G, NV, false, LOOSE><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n, rows_share_lines<T>(n));
     }
@@ -1802,6 +1815,10 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
     const int ppb = cluster_chunk_packs(packs, C, norm_rev_cluster_tile<T>(packs));
     require((size_t)ppb <= norm_rev_cluster_tile<T>(packs), "rmsnorm reverse: cluster chunk exceeds the register tile");
     Word* slots = reinterpret_cast<Word*>(partials + rmsnorm_reverse_partial_rows(m) * n);
+    if (note_plan(deep ? PLAN_DEEP : PLAN_CLUSTER, CLUSTER_THREADS, (int)((norm_rev_cluster_tile<T>(packs) + CLUSTER_THREADS - 1) / CLUSTER_THREADS), 1, S * C,
+                  CLUSTER_THREADS, C, ppb,
+                  (rmsnorm_reverse_partial_rows(m) * n + (C > 1 || deep ? m * (size_t)C * 2 : 0)) * sizeof(P)))
+      return;
     if (C > 1 || deep) { /* the pipelined kernel hands its sums over through the words also when a row is one chunk (test build only) */
       const size_t words = m * (size_t)C * 2;
       cluster_zero_slots<Word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(slots, words);
@@ -1824,6 +1841,7 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
   if (!resident && !shared) {
     rows = (unsigned)max_rows;
     const dim3 grid(rows), block(STREAM_THREADS);
+    if (note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, grid.x, block.x, 1, 0, (size_t)rows * n * sizeof(P))) return;
     constexpr int NA = stream_acc_packs<T>();
     const bool sums_fit = packs <= (size_t)STREAM_THREADS * NA;
     if (sums_fit) {
@@ -1854,6 +1872,7 @@ inline void rmsnorm_reverse(const T* x, const T* gain, const T* dy, T* dx, T* dg
       const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
       rows = (unsigned)(need < max_rows ? need : max_rows);
       const dim3 grid(rows), block(NORM_BLOCK);
+      if (note_plan(PLAN_SHORT, G, 1, NORM_BLOCK / G, grid.x, block.x, 1, 0, (size_t)rows * n * sizeof(P))) return;
       if (alpha != 0.0) rmsnorm_rev_short<T, W, G, CUT, true><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, (unsigned)n);
       else rmsnorm_rev_short<T, W, G, CUT, false><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, (unsigned)n);
     });

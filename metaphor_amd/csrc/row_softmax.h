@@ -865,6 +865,7 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   require(n <= 0x40000000ull, "softmax: row length must not exceed 2^30");
   if (softmax_short_rows<T>(n)) {
     for_short_row(n, W, [&]<int G, bool CUT>() {
+      if (note_plan(PLAN_SHORT, G, 1, SHORT_THREADS / G, short_row_grid(m, G), SHORT_THREADS)) return;
       softmax_fwd_short<T, W, G, CUT><<<dim3(short_row_grid(m, G)), dim3(SHORT_THREADS), 0, stream>>>(
           x, y, m, (unsigned)n, short_rows_share_lines<T>(n, G));
     });
@@ -874,9 +875,10 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   if (misalign16(x) != misalign16(y)) { /* rows of x and y peel differently */
     constexpr int MAXNV = max_nv_for<T>(64);
     const bool resident = for_row_plan<MAXNV, true>(plan_row((n + W - 1) / W, MAXNV, 2, 16), [&]<int G, int NV>() {
+      if (note_plan(PLAN_LOOSE, G, NV, G < WAVE ? WAVE / G : 1, row_grid(m, G), G < WAVE ? WAVE : G)) return;
       softmax_fwd_loose<T, W, G, NV><<<dim3(row_grid(m, G)), dim3(G < WAVE ? WAVE : G), 0, stream>>>(x, y, m, n);
     });
-    if (!resident) /* rows beyond the registers of a workgroup */
+    if (!resident && !note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, stream_grid(m), STREAM_THREADS)) /* rows beyond the registers of a workgroup */
       softmax_fwd_stream<T, W, true><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
     MP_CHECK_LAUNCH();
     return;
@@ -894,6 +896,10 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
     constexpr int WPS = 2 * share_parts<P>();
     share_word* callers = nullptr;
     long long region = 0;
+    /* what the launch may touch of the caller's workspace: the words, when the library has none of its own for it */
+    if (note_plan(PLAN_CLUSTER, CLUSTER_THREADS, cluster_nv<T>(), 1, m * C, CLUSTER_THREADS, C, ppb,
+                  C > 1 ? m * (size_t)C * WPS * sizeof(share_word) : 0))
+      return;
     if (C > 1) {
       region = share_region(scratch, m, C, WPS);
       if (region < 0) {
@@ -927,10 +933,11 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
     plan = RowPlan{plan.G / 2, 4};
   const bool resident = for_row_plan<MAXNV, true, FIT>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
+    if (note_plan(PLAN_RESIDENT, G, NV, G < WAVE ? WAVE / G : 1, grid.x, block.x)) return;
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
     else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
   });
-  if (!resident)
+  if (!resident && !note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, stream_grid(m), STREAM_THREADS))
     softmax_fwd_stream<T, W><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
   MP_CHECK_LAUNCH();
 }
@@ -973,6 +980,7 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
     for_short_row(n, W, [&]<int G, bool CUT>() {
       const dim3 grid(short_row_grid(m, G)), block(SHORT_THREADS);
       const unsigned by_xcd = short_rows_share_lines<T>(n, G);
+      if (note_plan(PLAN_SHORT, G, 1, SHORT_THREADS / G, grid.x, block.x)) return;
       if (blend) softmax_rev_short<T, W, G, CUT, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, (unsigned)n, by_xcd);
       else softmax_rev_short<T, W, G, CUT, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, (unsigned)n, by_xcd);
     });
@@ -983,10 +991,11 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
     constexpr int MAXNV = max_nv_for<T>(32);
     const bool resident = for_row_plan<MAXNV, true>(plan_row((n + W - 1) / W, MAXNV, 2, 16), [&]<int G, int NV>() {
       const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
+      if (note_plan(PLAN_LOOSE, G, NV, G < WAVE ? WAVE / G : 1, grid.x, block.x)) return;
       if (blend) softmax_rev_loose<T, W, G, NV, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
       else softmax_rev_loose<T, W, G, NV, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
     });
-    if (!resident) { /* rows beyond the registers of a workgroup */
+    if (!resident && !note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, stream_grid(m), STREAM_THREADS)) { /* rows beyond the registers of a workgroup */
       const dim3 grid(stream_grid(m)), block(STREAM_THREADS);
       if (blend) softmax_rev_stream<T, W, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
       else softmax_rev_stream<T, W, false, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
@@ -1003,6 +1012,9 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
     constexpr int WPS = share_parts<P>();
     share_word* callers = nullptr;
     long long region = 0;
+    if (note_plan(PLAN_CLUSTER, CLUSTER_THREADS, CLUSTER_REV_NV, 1, m * C, CLUSTER_THREADS, C, ppb,
+                  C > 1 ? m * (size_t)C * WPS * sizeof(share_word) : 0))
+      return;
     if (C > 1) { /* as in the forward: the library's own words for this workspace and geometry, else the caller's, cleared */
       region = share_region(scratch, m, C, WPS);
       if (region < 0) {
@@ -1033,6 +1045,7 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
   const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, one_pack ? 1 : 2, 16);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
+    if (note_plan(PLAN_RESIDENT, G, NV, G < WAVE ? WAVE / G : 1, grid.x, block.x)) return;
     if (ragged) {
       if (blend) softmax_rev_resident<T, W, G, NV, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
       else softmax_rev_resident<T, W, G, NV, true, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
@@ -1041,7 +1054,7 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
       else softmax_rev_resident<T, W, G, NV, false, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
     }
   });
-  if (!resident) {
+  if (!resident && !note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, stream_grid(m), STREAM_THREADS)) {
     const dim3 grid(stream_grid(m)), block(STREAM_THREADS);
     if (blend) softmax_rev_stream<T, W, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
     else softmax_rev_stream<T, W, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n);
