@@ -24,6 +24,7 @@ import re
 PKG = os.path.dirname(os.path.abspath(__file__))
 SRC_DIR = os.path.join(PKG, "csrc", "hipcc_src")
 HOST_DIR = os.path.join(PKG, "host")
+ZIG_OPS = os.path.join(os.path.dirname(PKG), "zig", "src", "ops")
 CHAINS = os.path.join(PKG, "chains.json")
 
 ARITY = {"add": 2, "sub": 2, "mul": 2, "neg": 1, "relu": 1, "selu": 1, "scale": 1, "shift": 1}
@@ -318,6 +319,44 @@ def host_table(chains):
     return "\n".join(out)
 
 
+def zig_table(chains):
+    """The same table for the Zig op layer (zig/src/ops/fused_chains.zig): one pair of functions per
+    listed chain that spreads the leaf pointers into the launcher's argument list, and the table
+    that src/ops/fused.zig looks a pending expression's signature up in."""
+    out = [
+        "// GENERATED by metaphor_amd/chaingen.py from chains.json -- do not edit.",
+        "// Fused elementwise chains a pending expression can run as: its signature (leaves numbered in",
+        "// order of first appearance), its leaf count, and the launchers of both directions.",
+        'const core = @import("core");',
+        "const StreamContext = core.utils.StreamContext;",
+        "",
+        "pub const Chain = struct {",
+        "    signature: []const u8,",
+        "    leaves: usize,",
+        "    forward: *const fn (key: usize, x: []const *anyopaque, out: *anyopaque, n: usize, ctx: StreamContext) void,",
+        "    reverse: *const fn (key: usize, x: []const *anyopaque, out_grads: *anyopaque, g: []const *anyopaque, alpha: f64, n: usize, ctx: StreamContext) void,",
+        "};",
+        "",
+    ]
+    rows = []
+    for c in chains:
+        root, k = parse(c["expr"])
+        name = c["name"]
+        xs = ", ".join(f"x[{i}]" for i in range(k))
+        gs = ", ".join(f"g[{i}]" for i in range(k))
+        out += [
+            f"fn fwd_{name}(key: usize, x: []const *anyopaque, out: *anyopaque, n: usize, ctx: StreamContext) void {{",
+            f"    core.invoke(core.kernels.{name}, key, .{{ {xs}, out, n, ctx }});",
+            "}",
+            f"fn rev_{name}(key: usize, x: []const *anyopaque, out_grads: *anyopaque, g: []const *anyopaque, alpha: f64, n: usize, ctx: StreamContext) void {{",
+            f"    core.invoke(core.kernels.{name}_reverse, key, .{{ {xs}, out_grads, {gs}, alpha, n, ctx }});",
+            "}",
+        ]
+        rows.append(f'    .{{ .signature = "{root.signature()}", .leaves = {k}, .forward = fwd_{name}, .reverse = rev_{name} }},')
+    out += ["", "pub const table = [_]Chain{"] + rows + ["};", ""]
+    return "\n".join(out)
+
+
 def load_chains():
     with open(CHAINS) as f:
         chains = json.load(f)
@@ -349,6 +388,8 @@ def generate():
                 changed.append(path)
     if _write_if_changed(os.path.join(HOST_DIR, "chains.hpp"), host_table(chains)):
         changed.append(os.path.join(HOST_DIR, "chains.hpp"))
+    if os.path.isdir(ZIG_OPS) and _write_if_changed(os.path.join(ZIG_OPS, "fused_chains.zig"), zig_table(chains)):
+        changed.append(os.path.join(ZIG_OPS, "fused_chains.zig"))
     # a chain taken out of chains.json takes its generated sources with it
     wanted = {c["name"] + suffix for c in chains for suffix in (".hip", "_reverse.hip")}
     for name in sorted(os.listdir(SRC_DIR)):

@@ -12,12 +12,16 @@ const core = @import("core");
 const OpDatum = core.OpDatum;
 const Tensor = core.Tensor;
 const Graph = core.Graph;
+const fused = @import("fused.zig");
 
 pub fn forward(x: Tensor) Tensor {
     return forward_impl(x.ptr, x);
 }
 
 pub fn forward_impl(graph: *Graph, x: Tensor) Tensor {
+    // recorded, not launched: the expression it ends up in runs as one kernel (fused.zig)
+    if (fused.enabled) return fused.record(graph, .selu, x, null, 0.0);
+
     const out = graph.tensor(.{ .class = .hid, .dtype = x.dtype(), .sizes = x.sizes() });
 
     core.invoke(core.kernels.selu, core.dkey(out), .{ x.data_ptr(), out.data_ptr(), out.len(), out.context() });
