@@ -23,11 +23,27 @@ static __device__ __align__(256) unsigned char scratch[MP_NOALLOC_SCRATCH_BYTES]
 namespace {
 constexpr int MP_NOALLOC_MAX_DEVICES = 64;
 std::atomic<void*> scratch_on_device[MP_NOALLOC_MAX_DEVICES];
+/* the stream of the last call on each device, and whether the warning below has been printed */
+std::atomic<void*> last_stream[MP_NOALLOC_MAX_DEVICES];
+std::atomic<bool> warned{false};
 
-void* noalloc_scratch() {
+/* Calls on different streams of one device share the array and must not overlap in time, which
+ * only the caller can see to. A change of stream is where that can go wrong: say so once. */
+void note_stream(int dev, hipStream_t stream) {
+  void* now = static_cast<void*>(stream);
+  void* before = last_stream[dev].exchange(now, std::memory_order_relaxed);
+  if (before != now && before != nullptr && !warned.exchange(true, std::memory_order_relaxed))
+    fprintf(stderr,
+            "mpRmsnormReverseR32NoAlloc: called on two streams of device %d; every call on a device uses the same "
+            "built-in workspace, so calls on different streams must be ordered by the caller (an event or a "
+            "synchronisation between them), or their gain gradients corrupt each other. Said once.\n", dev);
+}
+
+void* noalloc_scratch(hipStream_t stream) {
   int dev = 0;
   HIP_ASSERT(hipGetDevice(&dev));
   mp::require(dev >= 0 && dev < MP_NOALLOC_MAX_DEVICES, "mpRmsnormReverseR32NoAlloc: device index beyond 63");
+  note_stream(dev, stream);
   void* ptr = scratch_on_device[dev].load(std::memory_order_acquire);
   if (ptr == nullptr) { /* two threads racing here both get the same answer */
     HIP_ASSERT(hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch)));
@@ -40,8 +56,11 @@ void* noalloc_scratch() {
 
 // Same computation and same kernels as launch_rmsnorm_ij_j_reverse_r32 (bit-identical results),
 // without the scratch argument. Returns 0 after enqueueing, 1 (with a message on stderr, nothing
-// enqueued) when [m, n] needs more workspace than the built-in 16 MiB: rows of up to 8192
-// elements always fit. The array is shared by every call on a device and keeps the last call's
+// enqueued) when [m, n] needs more workspace than the built-in 16 MiB. What a call needs is one
+// row of n fp32 sums per workgroup of the row pass, at most two workgroups a compute unit:
+// min(m, 2 * CUs) * n * 4 bytes, so rows of up to 4194304 / min(m, 2 * CUs) elements fit (8192 on
+// the MI355X's 256 compute units, whatever m); rows shared by several workgroups add two words per
+// row and workgroup. The array is shared by every call on a device and keeps the last call's
 // contents; every word a launch reads it has written before (the partial rows by the row pass,
 // the words of shared long rows by the clearing kernel), so nothing needs to start at zero, but
 // two calls that overlap in time on one device (two streams, two threads) race on it.
@@ -56,7 +75,7 @@ extern "C" int mpRmsnormReverseR32NoAlloc(const void* src, const void* gain, con
             (unsigned long)m, (unsigned long)n, need, MP_NOALLOC_SCRATCH_BYTES);
     return 1;
   }
-  void* ptr = noalloc_scratch();
+  void* ptr = noalloc_scratch(get_stream(stream));
   mp::rmsnorm_reverse<r32>(static_cast<const r32*>(src), static_cast<const r32*>(gain),
                            static_cast<const r32*>(dst_grads), static_cast<r32*>(src_grads),
                            static_cast<r32*>(gain_grads), ptr, eps, alpha, m, n, get_stream(stream));

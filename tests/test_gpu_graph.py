@@ -51,9 +51,14 @@ def test_replays_of_a_captured_forward_and_reverse_sequence_match_eager():
     for t in (x, gain, dy, y, dx, dg, logits, p, dp, dl, a, b, c, d, e, e2, up, *grads):
         assert t.dtype == f32
 
+    # the entry point that brings its own workspace: its first (eager) call looks the built-in array up
+    dx_na, dg_na = torch.empty_like(x), torch.empty_like(gain)
+
     def sequence():
         W.rmsnorm_forward(x, gain, y, 1e-6)
         W.rmsnorm_reverse(x, gain, dy, dx, dg, nscratch, 1e-6)
+        assert kernels.mpRmsnormReverseR32NoAlloc(x.data_ptr(), gain.data_ptr(), dy.data_ptr(), dx_na.data_ptr(),
+                                                  dg_na.data_ptr(), 1e-6, 0.0, m, n, W._ctx()) == 0
         W.softmax_forward(logits, p, fs)
         W.softmax_reverse(p, dp, dl, 0.0, rs)
         W.rmsnorm_forward(logits, lgain, ly, 1e-6, lf)
@@ -63,7 +68,7 @@ def test_replays_of_a_captured_forward_and_reverse_sequence_match_eager():
         assert G.chain_forward(chain, [a, b, c, d], e2) == 0, G.chain_error()
         assert G.chain_reverse(chain, [a, b, c, d], up, grads, 0.0) == 0, G.chain_error()
 
-    outputs = (y, dx, dg, p, dl, ly, ldx, ldg, sums, e, e2, *grads)
+    outputs = (y, dx, dg, dx_na, dg_na, p, dl, ly, ldx, ldg, sums, e, e2, *grads)
     G.say("eager sequence")
     sequence()
     torch.cuda.synchronize()
@@ -81,6 +86,7 @@ def test_replays_of_a_captured_forward_and_reverse_sequence_match_eager():
         torch.cuda.synchronize()
         for got, ref in zip(outputs, eager):
             assert torch.equal(got, ref), f"replay {replay} differs from the eager result"
+        assert torch.equal(dx_na, dx) and torch.equal(dg_na, dg), "the no-alloc entry point differs from the launcher"
         # eager work of the program between replays
         W.softmax_forward(logits, p, fs)
         torch.cuda.synchronize()

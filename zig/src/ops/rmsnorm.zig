@@ -10,7 +10,8 @@
 //! behind one launcher: the row pass, which leaves one partial row of gain-gradient sums per
 //! workgroup in the workspace, and a fixed-order sum of those rows, so g.grad does not depend on
 //! scheduling. The workspace comes from the stream's scratch (src/core/utils.zig:20-36) and is
-//! sized by mpRmsnormReverseScratchBytes; the forward wants one only for rows beyond 128 KiB.
+//! sized by mpRmsnormReverseScratchBytes; whether the forward wants one is for mpRmsnormScratchBytes to say
+//! (0 for rows that one workgroup holds).
 const std = @import("std");
 const core = @import("core");
 const OpDatum = core.OpDatum;
