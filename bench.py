@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the row-reduction / elementwise hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--regions R] [--workload cfg2]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--regions R] [--prewarm-ms P] [--workload cfg2]
                     [--no-extra] [--no-cpu] [--no-ceilings] [--strict]
 
 A step is one pass of the hot path over one batch of the headline workload (cfg2: RMSNorm
@@ -490,6 +490,8 @@ def main():
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--regions", type=int, default=7, help="timed regions of --steps steps each; value = the median one")
+    ap.add_argument("--prewarm-ms", type=float, default=250.0,
+                    help="wall time of the disclosed pre-warm in front of the regions (counter runs under rocprofv3 use 0)")
     ap.add_argument("--workload", default="cfg2", choices=sorted(SETS))
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity check")
@@ -512,7 +514,7 @@ def main():
     name = args.workload
     sets = make_sets(name)
     w = sets[0]
-    times, in_region_ms, prewarm = time_regions(sets, args.steps, args.warmup, args.regions)
+    times, in_region_ms, prewarm = time_regions(sets, args.steps, args.warmup, args.regions, args.prewarm_ms * 1e-3)
     step_bytes = w.fwd_bytes + w.rev_bytes
     region_values = [args.steps * step_bytes / t / 1e9 for t in times]
     dt = _median(times)  # the median region: `value` and `ms_per_step` describe the same region

@@ -11,7 +11,10 @@
  * constant as second argument, scale (the reference's dilate: x * c) and shift (its translate:
  * x + c), with its leaves written as 0, 1, ... (or x0, x1, ...) and numbered in order of first
  * appearance; a leaf may appear more than once. Examples: "selu(mul(add(0,1),add(2,3)))",
- * "relu(scale(mul(0,1),0.125))". At most 8 leaves, 8 constants, 64 nodes. The constants are
+ * "relu(scale(mul(0,1),0.125))". Up to four results over the same leaves are written one after the
+ * other with ';' between them, leaves numbered across all of them
+ * ("selu(mul(add(0,1),2));relu(sub(add(0,1),3))"): one kernel computes them all and reads every
+ * leaf once (mpChainForwardMany / mpChainReverseMany). At most 8 leaves, 8 constants, 64 nodes. The constants are
  * arguments of the kernels, read from the text at every call: an expression is compiled once,
  * whatever the values (a learning rate that changes every step costs nothing).
  * dtype is MP_R16, MP_R32 or MP_R64 (tensor_types.h).
@@ -48,6 +51,16 @@ EXTERN_C int mpChainForward(const char* expression, int dtype, const void* const
  * (2k + 1 reads). g: k device pointers, distinct from each other. */
 EXTERN_C int mpChainReverse(const char* expression, int dtype, const void* const* x, const void* out_grads,
                             void* const* g, double alpha, len_t n, StreamContext);
+
+/* The same for an expression with R results: outs holds R device pointers, out_grads R upstream
+ * gradients; g[j] receives the sum over all results of d result_r / d x[j] * out_grads[r]. A leaf
+ * that no result depends on gets 0 (+ alpha * g). mpChainForward / mpChainReverse refuse an
+ * expression with more than one result. */
+EXTERN_C int mpChainForwardMany(const char* expressions, int dtype, const void* const* x, void* const* outs, len_t n, StreamContext);
+EXTERN_C int mpChainReverseMany(const char* expressions, int dtype, const void* const* x, const void* const* out_grads,
+                                void* const* g, double alpha, len_t n, StreamContext);
+/* How many results an expression has, -1 when it does not parse. */
+EXTERN_C int mpChainRoots(const char* expressions);
 
 /* Compile now rather than at the first launch. Needs no GPU. */
 EXTERN_C int mpChainCompile(const char* expression, int dtype);

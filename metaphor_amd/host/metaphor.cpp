@@ -356,6 +356,104 @@ static const FusedChain* find_chain(const std::string& signature) {
   return nullptr;
 }
 
+/* The pending nodes of this graph inside the expression below t (t itself included when pending). */
+static void pending_below(Graph* g, Tensor t, std::vector<size_t>& out, int& budget) {
+  if (--budget < 0 || !(is_pending(t) && t.ptr == g)) return;
+  out.push_back(t.idx);
+  const Graph::Node& node = g->nodes_[t.idx];
+  pending_below(g, node.in0, out, budget);
+  if (node.pending != Pending::selu && node.pending != Pending::relu && node.pending != Pending::dilate &&
+      node.pending != Pending::translate)
+    pending_below(g, node.in1, out, budget);
+}
+
+/* Several results in one kernel: other pending results of this graph (pending nodes that no pending
+ * node consumes) whose expressions share a pending subexpression with t's are computed with it, as
+ * one forward launch with as many output streams (mpChainForwardMany), so that what they share is
+ * read and computed once: u = a + b; e1 = selu(u * c); e2 = relu(u - d) is one launch. Each result
+ * keeps a reverse of its own (its own expression, one launch each): the graph's reverse walk
+ * reaches the results one at a time. True when t was computed this way. */
+static bool materialise_with_siblings(Graph* g, Tensor t, const std::string& signature, const std::vector<Tensor>& leaves) {
+  int budget = 64;
+  std::vector<size_t> mine;
+  pending_below(g, t, mine, budget);
+  if (mine.size() < 2) return false; /* nothing below t that another result could share */
+  std::vector<char> consumed(g->nodes_.size(), 0), shared(g->nodes_.size(), 0);
+  size_t first = g->nodes_.size();
+  for (size_t i = 0; i < g->nodes_.size(); ++i) {
+    const Graph::Node& node = g->nodes_[i];
+    if (node.pending == Pending::none) continue;
+    for (const Tensor& in : {node.in0, node.in1})
+      if (in.ptr == g && in.cls == TensorClass::hid && in.idx < consumed.size()) consumed[in.idx] = 1;
+  }
+  for (size_t i : mine)
+    if (i != t.idx) {
+      shared[i] = 1;
+      first = i < first ? i : first;
+    }
+  struct Root { Tensor t; std::string own; std::vector<Tensor> own_leaves; };
+  std::vector<Root> roots{{t, signature, leaves}};
+  std::string combined = signature;
+  std::vector<Tensor> all = leaves;
+  for (size_t i = first + 1; i < g->nodes_.size() && roots.size() < 4; ++i) {
+    const Graph::Node& node = g->nodes_[i];
+    if (i == t.idx || node.pending == Pending::none || consumed[i]) continue;
+    if (node.data.len != g->nodes_[t.idx].data.len || node.data.dtype != g->nodes_[t.idx].data.dtype) continue;
+    const Tensor other{g, i, TensorClass::hid};
+    std::vector<size_t> theirs;
+    int room = 64;
+    pending_below(g, other, theirs, room);
+    bool overlap = false;
+    for (size_t j : theirs) overlap = overlap || shared[j];
+    if (!overlap) continue;
+    std::string text, own;
+    std::vector<Tensor> together = all, own_leaves;
+    int b1 = 64, b2 = 64;
+    if (!spell(g, other, text, together, b1) || !spell(g, other, own, own_leaves, b2)) continue; /* too many leaves: it stays by itself */
+    combined += ";" + text;
+    all = together;
+    roots.push_back({other, own, own_leaves});
+  }
+  if (roots.size() < 2 || mpChainCompile(combined.c_str(), (int)t.dtype()) != 0) return false;
+  void* x[8];
+  void* outs[4];
+  for (size_t i = 0; i < all.size(); ++i) {
+    if (all[i].len() == 0) panic("materialise: an input of a pending node was freed");
+    x[i] = all[i].data_ptr();
+  }
+  { /* the shape this graph had compiled */
+    std::string shape;
+    std::vector<Tensor> again;
+    int room = 64;
+    for (size_t r = 0; r < roots.size(); ++r) {
+      if (r) shape += ';';
+      room = 64;
+      spell(g, roots[r].t, shape, again, room, true);
+    }
+    size_t idx = 0;
+    while (idx < g->runtime_chains_.size() && g->runtime_chains_[idx] != shape) ++idx;
+    if (idx == g->runtime_chains_.size()) g->runtime_chains_.push_back(shape);
+  }
+  const size_t n = g->nodes_[t.idx].data.len;
+  const Tag dt = g->nodes_[t.idx].data.dtype;
+  for (size_t r = 0; r < roots.size(); ++r) {
+    TensorData d = g->allocator_.alloc(dt, n, g->stream);
+    g->nodes_[roots[r].t.idx].data = d;
+    g->nodes_[roots[r].t.idx].pending = Pending::none;
+    outs[r] = d.ptr;
+  }
+  if (mpChainForwardMany(combined.c_str(), (int)dt, x, outs, (len_t)n, g->stream->context) != 0) panic(mpChainError());
+  g->launches++;
+  if (g->mode == Mode::train)
+    for (const Root& root : roots) {
+      std::vector<OpDatum> args(root.own_leaves.begin(), root.own_leaves.end());
+      args.push_back(OpDatum(root.own));
+      args.push_back(root.t);
+      attach_op(root.t, runtime_chain_reverse, std::move(args));
+    }
+  return true;
+}
+
 void materialise(Tensor t) {
   if (!is_pending(t)) return;
   Graph* g = t.ptr;
@@ -403,6 +501,7 @@ void materialise(Tensor t) {
      * (a single op is already one kernel). A refusal (too many leaves, a compile failure) falls
      * through to one launch per op. */
     const bool several = signature.find('(') != signature.rfind('(');
+    if (g->fusion == Fusion::any && spelled && materialise_with_siblings(g, t, signature, leaves)) return;
     if (g->fusion == Fusion::any && spelled && several &&
         mpChainCompile(signature.c_str(), (int)key) == 0) {
       void* x[8];

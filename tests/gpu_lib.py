@@ -301,6 +301,19 @@ def chain_reverse(expr, xs, out_grads, grads, alpha=0.0):
                             _pointer_array(grads), float(alpha), out_grads.numel(), ctx())
 
 
+def chain_forward_many(exprs, xs, outs):
+    """Several results over the same leaves ("e1;e2") in one kernel."""
+    f = ffi.load_fusion()
+    return f.mpChainForwardMany(exprs.encode(), KEY[outs[0].dtype], _pointer_array(xs), _pointer_array(outs),
+                                outs[0].numel(), ctx())
+
+
+def chain_reverse_many(exprs, xs, out_grads, grads, alpha=0.0):
+    f = ffi.load_fusion()
+    return f.mpChainReverseMany(exprs.encode(), KEY[grads[0].dtype], _pointer_array(xs), _pointer_array(out_grads),
+                                _pointer_array(grads), float(alpha), grads[0].numel(), ctx())
+
+
 def chain_error():
     return ffi.load_fusion().mpChainError().decode()
 

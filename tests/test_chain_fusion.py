@@ -135,7 +135,9 @@ def test_every_dtype_compiles_and_is_cached_once(dtype):
     ("add(add(add(add(0,1),add(2,3)),add(add(4,5),add(6,7))),8)", "more than 8 leaves"),
     ("scale(0)", "expected ','"), ("scale(0,x1)", "finite number"), ("shift(0,abc)", "finite number"), ("scale(0,inf)", "finite number"),
     ("shift(" * 9 + "0" + ",1)" * 9, "more than 8 constants"),
-    ("neg(" * 65 + "0" + ")" * 65, "more than 64 nodes"), ("neg(" * 100000 + "0" + ")" * 100000, "more than 64 nodes")])
+    ("neg(" * 65 + "0" + ")" * 65, "more than 64 nodes"), ("neg(" * 100000 + "0" + ")" * 100000, "more than 64 nodes"),
+    ("add(0,1);", "unknown op"), ("add(0,1);0", "bare leaf"), ("add(0,1);add(0,3)", "order of first appearance"),
+    (";".join(["neg(0)"] * 5), "more than 4 results")])
 def test_bad_expressions_are_refused_with_a_reason(bad, why):
     lib = ffi.load_fusion()
     n = lib.mpChainCacheSize()
@@ -157,7 +159,7 @@ def test_the_fusion_library_exports_what_its_header_declares():
     names = [n for _, n, _ in ffi.parse_declarations(ffi.os.path.join(ffi.ROOT, "include", "chain_fusion.h"))]
     assert sorted(names) == sorted(["mpChainForward", "mpChainReverse", "mpChainCompile", "mpChainLeaves",
                                     "mpChainSource", "mpChainCodeObject", "mpChainCacheSize", "mpChainCompilations",
-                                    "mpChainError"])
+                                    "mpChainError", "mpChainForwardMany", "mpChainReverseMany", "mpChainRoots"])
     for n in names:
         assert getattr(lib, n)
 
@@ -237,3 +239,82 @@ def test_a_failed_compilation_is_not_tried_again():
         "print('ok')\n")
     res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, timeout=300)
     assert res.returncode == 0 and "ok" in res.stdout, res.stderr[-2000:]
+
+
+def test_expressions_with_several_results_differentiate_like_autograd():
+    """Up to four results over shared leaves in one text: the forward functor writes every result, the
+    reverse functor adds every result's contribution to each leaf (upstream gradient r is in[k + r]),
+    a leaf that only some results use gets only theirs; executed line by line against torch autograd."""
+    lib = ffi.load_fusion()
+    r = np.random.default_rng(11)
+    fixed = ["selu(mul(add(x0,x1),x2));relu(sub(add(x0,x1),x3))", "neg(x0);neg(x1)", "mul(x0,x0);add(x0,x1);scale(x1,0.5)"]
+    for case in range(30):
+        if case < len(fixed):
+            text = fixed[case]
+        else:  # random trees, leaves renumbered across the whole text as the parser wants them
+            roots = int(r.integers(2, 5))
+            parts, seen = [], []
+            for _ in range(roots):
+                e = random_expression(r, int(r.integers(1, 4)), int(r.integers(1, 4)))
+                pick = {}
+                def renumber(m):
+                    old = int(m.group(1))
+                    if old not in pick:  # reuse a leaf of an earlier result half of the time
+                        pick[old] = int(r.choice(seen)) if seen and r.random() < 0.5 else None
+                    if pick[old] is None:
+                        pick[old] = len(seen)
+                        seen.append(len(seen))
+                    return f"x{pick[old]}"
+                parts.append(re.sub(r"x(\d+)", renumber, e))
+            if len(seen) > 8:
+                continue
+            text = ";".join(parts)
+        exprs = text.split(";")
+        assert lib.mpChainRoots(text.encode()) == len(exprs), (text, lib.mpChainError())
+        k = lib.mpChainLeaves(text.encode())
+        assert k >= 1, (text, lib.mpChainError())
+        src = lib.mpChainSource(text.encode(), 2)
+        assert src, (text, lib.mpChainError())
+        bodies = {name: _with_literals(lines, text) for name, lines in _functor_bodies(src.decode()).items()}
+        R = len(exprs)
+        xs = [r.uniform(-2, 2, 100) for _ in range(k)]
+        ups = [r.normal(0, 1, 100) for _ in range(R)]
+        old = [r.normal(0, 1, 100) for _ in range(k)]
+        ts = [torch.from_numpy(x.copy()).requires_grad_(True) for x in xs]
+        outs = []
+        for e in exprs:  # each result parsed by the build-time parser with its own leaf numbering
+            names = []
+            def local(m):
+                g = int(m.group(1))
+                if g not in names:
+                    names.append(g)
+                return f"x{names.index(g)}"
+            e_x = e
+            root, _ = chaingen.parse(re.sub(r"x(\d+)", local, e_x))
+            outs.append(_torch_eval(root, [ts[g] for g in names]))
+        total = sum((o * torch.from_numpy(u)).sum() for o, u in zip(outs, ups))
+        total.backward()
+
+        fwd_lines = bodies["ChainForward"]
+        env = _run_lines([l for l in fwd_lines if not l.startswith("out[")], xs)
+        got = [eval(re.sub(r"\bin\[", "inp[", l.split("=", 1)[1].rstrip(";")), {}, env) for l in fwd_lines if l.startswith("out[")]
+        assert len(got) == R
+        for o, ref in zip(got, outs):
+            np.testing.assert_allclose(o, ref.detach().numpy(), rtol=1e-12, atol=1e-14, err_msg=text)
+        alpha = 0.25
+        rev = bodies["ChainReverseBlend"]
+        env = _run_lines([l for l in rev if not l.startswith("out[") and not l.startswith("const P al")], xs + ups + old)
+        env["al"] = alpha
+        grads = [l for l in rev if l.startswith("out[")]
+        assert len(grads) == k
+        for i, line in enumerate(grads):
+            g = eval(re.sub(r"\bin\[", "inp[", line.split("=", 1)[1].rstrip(";").replace("(P)0", "0.0")), {}, env)
+            ref = (ts[i].grad.numpy() if ts[i].grad is not None else 0.0) + alpha * old[i]
+            np.testing.assert_allclose(g, ref, rtol=1e-12, atol=1e-13, err_msg=f"{text} leaf {i}")
+    # one compilation for the lot, and the single-result entry points refuse it
+    assert lib.mpChainCompile(fixed[0].encode(), 1) == 0, lib.mpChainError()
+    ctx = ffi.StreamContext()
+    import ctypes
+    ptrs = (ctypes.c_void_p * 4)()
+    assert lib.mpChainForward(fixed[0].encode(), 1, ptrs, None, 16, ctx) != 0
+    assert "mpChainForwardMany" in lib.mpChainError().decode()

@@ -181,6 +181,65 @@ def test_one_kernel_serves_every_value_of_a_constant():
         assert len(sizes) == 1, "another value of a constant must not be another compilation"
 
 
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_several_results_in_one_kernel_match_autograd(dtype):
+    """u = a + b; e1 = selu(u * c); e2 = relu(u - d) (and two more texts) as ONE forward kernel with
+    as many output streams and ONE reverse kernel that takes both upstream gradients; against torch
+    autograd in fp64 on the storage-rounded inputs, overwrite and blend, aligned and shifted."""
+    r = np.random.default_rng(23)
+    texts = ["selu(mul(add(0,1),2));relu(sub(add(0,1),3))", "mul(0,0);add(0,1);scale(1,0.5)",
+             "neg(0);relu(1);selu(mul(0,1));shift(sub(2,0),-0.25)"]
+    for text in texts:
+        exprs = text.split(";")
+        k, R = G.ffi.load_fusion().mpChainLeaves(text.encode()), len(exprs)
+        assert G.ffi.load_fusion().mpChainRoots(text.encode()) == R
+        for n, shift, alpha in [(5, 0, 0.0), (70001, 0, 0.0), (70001, 1, -0.5), (1 << 20, 0, 1.0)]:
+            G.say(f"several results {text} dtype={dtype} n={n} shift={shift} alpha={alpha}")
+            xs = [G.dev(r.uniform(-1.5, 1.5, n), dtype, shift) for _ in range(k)]
+            ups = [G.dev(r.normal(0, 1, n), dtype, shift) for _ in range(R)]
+            old = [G.dev(r.normal(0, 1, n), dtype, shift) for _ in range(k)]
+            outs = [G.Guarded((n,), dtype, shift) for _ in range(R)]
+            hx, hup, hold = [G.host(x.t) for x in xs], [G.host(u.t) for u in ups], [G.host(o.t).copy() for o in old]
+            assert G.chain_forward_many(text, [x.t for x in xs], [o.t for o in outs]) == 0, G.chain_error()
+            assert G.chain_reverse_many(text, [x.t for x in xs], [u.t for u in ups], [o.t for o in old], alpha) == 0, G.chain_error()
+            ts = [torch.from_numpy(x.astype(np.float64)).requires_grad_(True) for x in hx]
+            gmag = [np.zeros(n) for _ in range(k)]
+            refs = []
+            for e, up in zip(exprs, hup):  # each result with its own leaf numbering for the build-time parser
+                names = []
+                def local(m):
+                    g = int(m.group(1))
+                    if g not in names:
+                        names.append(g)
+                    return f"x{names.index(g)}"
+                import re
+                root, _ = chaingen.parse(re.sub(r"(?<=[(,])(\d+)(?=[,)])(?!\.)", lambda m: local(m), _leaves_only(e)))
+                val = _torch_eval(root, [ts[g] for g in names])
+                refs.append(val)
+                vmag, gm = _magnitudes(root, [hx[g] for g in names], up)
+                for j, g in enumerate(names):
+                    gmag[g] = gmag[g] + gm[j]
+                refs[-1] = (val, vmag)
+            total = sum((v * torch.from_numpy(u.astype(np.float64))).sum() for (v, _), u in zip(refs, hup))
+            total.backward()
+            for o, (v, vmag) in zip(outs, refs):
+                G.compare(o.t, v.detach().numpy(), dtype, f"{text} value", rowwise=False, scale=vmag)
+            for i in range(k):
+                g = ts[i].grad.numpy() if ts[i].grad is not None else np.zeros(n)
+                want = g + alpha * hold[i].astype(np.float64)
+                G.compare(old[i].t, want, dtype, f"{text} gradient of leaf {i}", rowwise=False,
+                          scale=gmag[i] + abs(alpha) * np.abs(hold[i].astype(np.float64)))
+            for b in xs + ups + outs + old:
+                b.check(text)
+
+
+def _leaves_only(e):
+    """The text of one result with its constants protected from the leaf renumbering: a constant is the
+    second argument of scale / shift."""
+    import re
+    return re.sub(r"((?:scale|shift)\((?:[^()]|\([^()]*\))*),(-?[\d.]+(?:e-?\d+)?)\)", lambda m: f"{m.group(1)},{float(m.group(2))!r}e0)", e)
+
+
 def test_rate_of_a_run_time_kernel_beside_the_build_time_one():
     """2^26 r32 elements: the run-time kernel of the benchmark chain beside the build-time one (same
     engine, same functor), events around 10 launches each. Printed, not asserted: wall-clock checks

@@ -77,6 +77,20 @@ def test_host_library_end_to_end(tmp_path):
     _cmp(_load(d, "any_affine2_da"), on2 * -0.75 * c64_, "run-time chain, other constants da", rowwise=False)
     _cmp(_load(d, "any_affine2_dc"), on2 * -0.75 * a64_, "run-time chain, other constants dc", rowwise=False)
 
+    # two results out of one forward kernel: u = a + b; e1 = selu(u * c); e2 = relu(u - d); each reversed
+    # with an upstream gradient of 1, the leaf gradients accumulate over the two reverses
+    b64_, d64_ = b.astype(np.float64), dd.astype(np.float64)
+    u_ = a64_ + b64_
+    w1, w2 = u_ * c64_, u_ - d64_
+    g1 = O.selu_reverse(w1, np.ones_like(w1))
+    g2 = (w2 >= 0).astype(np.float64)
+    _cmp(_load(d, "two_e1"), O.selu(w1), "two results e1", rowwise=False, scale=np.abs(w1))
+    _cmp(_load(d, "two_e2"), np.where(w2 >= 0, w2, 0.0), "two results e2", rowwise=False)
+    _cmp(_load(d, "two_da"), g1 * c64_ + g2, "two results da", rowwise=False)
+    _cmp(_load(d, "two_db"), g1 * c64_ + g2, "two results db", rowwise=False)
+    _cmp(_load(d, "two_dc"), g1 * u_, "two results dc", rowwise=False)
+    _cmp(_load(d, "two_dd"), -g2, "two results dd", rowwise=False)
+
     # other generated chains (fp64 compositions of the pinned oracle pieces; upstream gradient = 1)
     a64, b64, c64, d64 = (z.astype(np.float64) for z in (a, b, c, dd))
     u, v = a64 + b64, c64 + d64
