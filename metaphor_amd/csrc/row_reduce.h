@@ -16,6 +16,7 @@
 #ifndef MP_ROW_REDUCE_H
 #define MP_ROW_REDUCE_H
 
+#include <atomic>
 #include "row_rmsnorm.h" /* sum_partial_rows */
 
 #if defined(__cplusplus) && defined(__HIPCC__)
@@ -353,6 +354,17 @@ template <class T> inline size_t reduce_cols_scratch_bytes(size_t m, size_t n) {
   return chunks > 1 ? chunks * n * sizeof(typename precision<T>::type) : 0;
 }
 
+/* A stream context put together by hand has no workspace: say once what that costs, since nothing
+ * in the launcher's signature does. */
+inline void note_missing_workspace(size_t m, size_t n, size_t blocks) {
+  static std::atomic<bool> told{false};
+  if (!told.exchange(true))
+    fprintf(stderr,
+            "note: column sums of [%zu, %zu] run on %zu workgroups because they were given no workspace (a stream "
+            "context from mpInitStream / mpAdoptStream carries one, launch_reduce_ij_j_scratch takes one); said once\n",
+            m, n, blocks);
+}
+
 /* dst[j] = scale * sum_i (weight[i] *) src[i,j] + blend * dst[j].
  * scratch: reduce_cols_scratch_bytes(m, n) bytes or NULL (then one workgroup per column strip
  * walks every row, which leaves most of the GPU idle on tall, narrow matrices). */
@@ -398,6 +410,8 @@ inline void reduce_cols(const T* src, const T* weight, T* dst, void* scratch, do
   size_t blocks = ((n + W - 1) / W + lanes - 1) / lanes;
   require(blocks < 0x7fffffffull, "column sums: too many columns for one grid");
   size_t chunks = scratch != nullptr ? reduce_cols_chunks<T>(m, n) : 1;
+  if (scratch == nullptr && blocks * 4 < (size_t)compute_units() && reduce_cols_chunks<T>(m, n) > 1)
+    note_missing_workspace(m, n, blocks);
   const size_t fit = scratch_bytes / (n * sizeof(P)); /* partial rows the workspace holds */
   if (chunks > fit) chunks = fit;
   /* without a workspace the strips are all the workgroups there are: an aligned matrix too narrow
