@@ -5,9 +5,11 @@
                     [--no-extra] [--no-cpu] [--no-ceilings] [--strict]
 
 A step is one pass of the hot path over one batch of the headline workload (cfg2: RMSNorm
-forward + reverse, r32, [8192, 4096]) with all inputs resident in HBM. Successive steps
-rotate over several buffer sets, and the reverse of a step works on a different set than its
-forward, so the 256 MiB memory-side cache cannot serve repeats.
+forward + reverse, r32, [8192, 4096]) with all inputs resident in HBM: the forward of a buffer
+set and then the reverse of the same set, as a training step runs them. Successive steps rotate
+over several buffer sets, so that a set comes back only after the other sets' steps have passed
+through the 256 MiB memory-side cache: what a reverse finds there was put there by the forward of
+its own step, never by an earlier step.
 
 Timing: W untimed warm-up steps, then a pre-warm of the same steps for a stated wall time (a
 GPU that has idled runs its first milliseconds below its sustained clocks; `prewarm_ms` and
@@ -16,8 +18,11 @@ by synchronisations. `value` is the median region's K * bytes / time, `ms_per_st
 region's time / K; all R per-region values are in the line (`region_values_GBps`), the first
 among them. Inside each region one launch of the dominant launcher is bracketed by a pair of
 events on the launch stream (`in_region_launch_ms`: it includes the cost of the pair itself,
-2-3 us); the roofline object's launch duration comes from groups of 8 back-to-back launches of
-that launcher between one pair, timed right after the regions, which takes the pair's cost out.
+2-3 us). The roofline object's launch duration takes the pair's cost out: right after the regions,
+groups of 8 steps, of 8 forwards and of 8 reverses are each timed between one pair. The reverse
+inside a step is a group of steps minus a group of forwards (`roofline`), the reverse on tensors
+that nothing touched recently is the third kind of group (`roofline.on_its_own`); they differ
+where the reverse re-reads a tensor that its forward left in the memory-side cache.
 
 One JSON line is printed: whole-step throughput, the roofline of the dominant launcher, and for
 every workload its forward/reverse rates, roofline objects, the CPU oracle timed on the host
@@ -37,7 +42,7 @@ sys.path.insert(0, ROOT)
 sys.path.insert(0, os.path.join(ROOT, "tests"))
 
 HBM_PEAK_GBPS = 8000.0
-SETS = {"cfg1": 16, "cfg2": 4, "cfg3": 2, "cfg4": 2, "cfg5a": 3, "cfg5b": 3, "copy": 2, "permutate": 2, "gemm": 2,
+SETS = {"cfg1": 16, "cfg2": 6, "cfg3": 2, "cfg4": 2, "cfg5a": 3, "cfg5b": 3, "copy": 2, "permutate": 2, "gemm": 2,
         "chain": 2, "normvocab": 3}
 ON_REQUEST = {"normvocab"}  # workloads outside BASELINE's configurations: run with --workload, not beside the headline
 MFMA_PEAK_TFLOPS = {"gemm": 2500.0}  # dense fp16 matrix rate of the MI355X
@@ -86,10 +91,14 @@ BATCH = 8  # launches between a pair of events: a pair costs 2-3 us of stream ti
 
 
 def _step(sets, i):
-    S = len(sets)
-    sets[i % S].forward()
-    if sets[0].has_reverse:
-        sets[(i + S // 2) % S].reverse()
+    """One step: the forward of a buffer set and then the reverse of the same set, as a training
+    step runs them (the reverse re-reads what its forward read or wrote a moment ago). Steps rotate
+    over the buffer sets, so a set comes back only after the other sets' steps have passed through
+    the 256 MiB memory-side cache: nothing a step finds there was left by an earlier step."""
+    s = sets[i % len(sets)]
+    s.forward()
+    if s.has_reverse:
+        s.reverse()
 
 
 def time_regions(sets, steps, warmup, regions=7, prewarm_s=0.25):
@@ -124,7 +133,7 @@ def time_regions(sets, steps, warmup, regions=7, prewarm_s=0.25):
             elif has_rev:
                 sets[i % S].forward()
                 a.record()
-                sets[(i + S // 2) % S].reverse()
+                sets[i % S].reverse()
                 b.record()
             else:
                 a.record()
@@ -137,14 +146,17 @@ def time_regions(sets, steps, warmup, regions=7, prewarm_s=0.25):
 
 
 def time_each(sets, iters, batch=BATCH):
-    """Per-launch durations in ms of the forward and of the reverse launcher: groups of `batch`
-    back-to-back launches (rotating over the buffer sets) between one pair of events, one value
-    per group. A reverse works on the set half a rotation away from the last forward's."""
+    """Per-launch durations in ms: groups of `batch` back-to-back launches (rotating over the buffer
+    sets) between one pair of events, one value per group. Three kinds of group take turns: forwards
+    only; reverses only (the rotation over the sets goes on through all groups, so a reverse works on
+    a set that launches on all the other sets have passed since: nothing of it is cached); whole steps (a forward and the reverse of the same set). Returns
+    the three lists (forward, reverse on its own, step); the reverse as it runs inside a step is a
+    step minus a forward."""
     import torch
     S = len(sets)
     has_rev = sets[0].has_reverse
     groups = max(3, iters // batch)
-    fwd, rev = [], []
+    fwd, rev, step = [], [], []
     k = 0
     for _ in range(groups):
         a, b = _events(2)
@@ -157,12 +169,21 @@ def time_each(sets, iters, batch=BATCH):
         if has_rev:
             c, d = _events(2)
             c.record()
-            for j in range(batch):
-                sets[(k + j + S // 2) % S].reverse()
+            for _ in range(batch):  # the rotation goes on: each set was last touched S - 1 launches ago
+                sets[k % S].reverse()
+                k += 1
             d.record()
             rev.append((c, d))
+            e, f = _events(2)
+            e.record()
+            for _ in range(batch):
+                _step(sets, k)
+                k += 1
+            f.record()
+            step.append((e, f))
     torch.cuda.synchronize()
-    return [a.elapsed_time(b) / batch for a, b in fwd], [a.elapsed_time(b) / batch for a, b in rev]
+    per = lambda pairs: [a.elapsed_time(b) / batch for a, b in pairs]
+    return per(fwd), per(rev), per(step)
 
 
 def graph_forward_ms(sets, replays=50):
@@ -208,7 +229,7 @@ def native_launch_cost(launches=4000):
     return json.loads(res.stdout.strip().splitlines()[-1])
 
 
-def rates(w, fwd_ms, rev_ms):
+def rates(w, fwd_ms, rev_ms, step_ms=None):
     out = {"fwd_ms": round(_median(fwd_ms), 5),
            "fwd_GBps": round(w.fwd_bytes / (_median(fwd_ms) * 1e-3) / 1e9, 1)}
     out["fwd_frac"] = round(out["fwd_GBps"] / HBM_PEAK_GBPS, 4)
@@ -218,6 +239,10 @@ def rates(w, fwd_ms, rev_ms):
         out["rev_GBps"] = round(w.rev_bytes / (_median(rev_ms) * 1e-3) / 1e9, 1)
         out["rev_frac"] = round(out["rev_GBps"] / HBM_PEAK_GBPS, 4)
         out["rev_rows_per_s"] = round(w.rows / (_median(rev_ms) * 1e-3), 1)
+    if step_ms:  # a forward and the reverse of the same tensors, back to back
+        out["step_ms"] = round(_median(step_ms), 5)
+        out["step_GBps"] = round((w.fwd_bytes + w.rev_bytes) / (_median(step_ms) * 1e-3) / 1e9, 1)
+        out["step_vs_apart"] = round(_median(step_ms) / (_median(fwd_ms) + _median(rev_ms)), 4)
     if hasattr(w, "fwd_flops"):
         out["fwd_TFLOPs"] = round(w.fwd_flops / (_median(fwd_ms) * 1e-3) / 1e12, 1)
         if rev_ms:
@@ -225,12 +250,22 @@ def rates(w, fwd_ms, rev_ms):
     return out
 
 
-def roofline_of(name, direction, nbytes, launch_ms, ceiling=None):
+def reverse_in_step(fwd_ms, step_ms):
+    """Durations of the reverse launcher as it runs inside a step, behind the forward of the same
+    tensors: each group of steps minus the group of forwards timed next to it."""
+    return [max(s - f, 1e-6) for f, s in zip(fwd_ms, step_ms)]
+
+
+def roofline_of(name, direction, nbytes, launch_ms, ceiling=None, on_its_own_ms=None):
     """The roofline object of one launcher: algorithmic bytes over the average launch duration
     (events on the launch stream), against the 8 TB/s peak; `traffic` from the committed
     FETCH_SIZE / WRITE_SIZE summary (reverse launcher of workloads that have one, else forward);
     `copy_ceiling` is a plain pass with the same reads, writes and footprint, timed the same way
-    in this run."""
+    in this run. With on_its_own_ms, launch_ms are the durations of a reverse inside a step (a
+    step minus a forward) and on_its_own_ms those of the same launcher on tensors that nothing
+    touched recently: the first is what the timed step contains, the second is the launcher against
+    HBM alone (where the two differ, the reverse found a tensor of its forward in the memory-side
+    cache; the plain pass of the copy ceiling never does)."""
     # an event pair also spans whatever the host does between recording the first event and
     # enqueueing the launch; a sample several times the median is such a host stall, not a launch
     med = _median(launch_ms)
@@ -250,6 +285,17 @@ def roofline_of(name, direction, nbytes, launch_ms, ceiling=None):
     if ceiling:
         out["copy_ceiling"] = ceiling
         out["frac_of_copy_ceiling"] = round(achieved / ceiling["GBps"], 4)
+    if on_its_own_ms:
+        out["kernel"] = f"{name} {direction} launcher inside a step (behind the forward of the same tensors)"
+        out["timing"] = (f"{len(kept)} groups of {BATCH} steps minus {BATCH} forwards, one event pair a group of "
+                         "steps and one a group of forwards")
+        own = _median(on_its_own_ms)
+        alone = {"avg_launch_ms": round(sum(on_its_own_ms) / len(on_its_own_ms), 5), "median_launch_ms": round(own, 5),
+                 "achieved": round(nbytes / (own * 1e-3) / 1e9, 1)}
+        alone["frac"] = round(alone["achieved"] / HBM_PEAK_GBPS, 4)
+        if ceiling:
+            alone["frac_of_copy_ceiling"] = round(alone["achieved"] / ceiling["GBps"], 4)
+        out["on_its_own"] = alone
     return out
 
 
@@ -493,6 +539,7 @@ def main():
     ap.add_argument("--prewarm-ms", type=float, default=250.0,
                     help="wall time of the disclosed pre-warm in front of the regions (counter runs under rocprofv3 use 0)")
     ap.add_argument("--workload", default="cfg2", choices=sorted(SETS))
+    ap.add_argument("--sets", type=int, default=0, help="buffer sets the steps rotate over (default: the workload's own number)")
     ap.add_argument("--no-extra", action="store_true", help="skip the other workloads")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline and parity check")
     ap.add_argument("--no-ceilings", action="store_true", help="skip the plain-copy ceilings of each stream mix")
@@ -512,22 +559,22 @@ def main():
 
     import contextlib
     name = args.workload
-    sets = make_sets(name)
+    sets = make_sets(name, args.sets or None)
     w = sets[0]
     times, in_region_ms, prewarm = time_regions(sets, args.steps, args.warmup, args.regions, args.prewarm_ms * 1e-3)
     step_bytes = w.fwd_bytes + w.rev_bytes
     region_values = [args.steps * step_bytes / t / 1e9 for t in times]
     dt = _median(times)  # the median region: `value` and `ms_per_step` describe the same region
     value = args.steps * step_bytes / dt / 1e9
-    fwd_ms, rev_ms = time_each(sets, max(24, min(args.steps, 96)))
+    fwd_ms, rev_ms, step_ms = time_each(sets, max(24, min(args.steps, 96)))
 
-    dom_bytes, dom_name, dom_ms = (w.rev_bytes, "reverse", rev_ms) if w.has_reverse else (w.fwd_bytes, "forward", fwd_ms)
+    dom_bytes, dom_name, dom_ms = (w.rev_bytes, "reverse", reverse_in_step(fwd_ms, step_ms)) if w.has_reverse else (w.fwd_bytes, "forward", fwd_ms)
     checks_failed = []
     cpu_line = parity = None
     if not args.no_cpu:
         with contextlib.redirect_stdout(sys.stderr):  # stdout carries the one JSON line only
             cpu_line, parity = cpu_and_parity(name, w, CPU_BUDGET_S.get(name, 3.0))
-    per_workload = rates(w, fwd_ms, rev_ms)
+    per_workload = rates(w, fwd_ms, rev_ms, step_ms)
     del sets
     torch.cuda.empty_cache()
     fwd_ceiling, rev_ceiling = (None, None) if args.no_ceilings else ceilings_for(w)
@@ -545,7 +592,7 @@ def main():
         "vs_baseline": None,
         "dtype": {"cfg3": "f16", "gemm": "f16"}.get(name, "f32"),
         "data": "synthetic",
-        "config": {"workload": f"{name}: {W.DESCRIPTION[name]}", "buffer_sets": SETS[name],
+        "config": {"workload": f"{name}: {W.DESCRIPTION[name]}", "buffer_sets": args.sets or SETS[name],
                    "bytes_per_step": step_bytes},
         # how `value` was taken: median of `regions` regions of `steps` steps each, after the warm-up
         # steps and a disclosed pre-warm of the same steps; the first region is region_values_GBps[0]
@@ -555,7 +602,8 @@ def main():
         "frac_of_hbm_peak": round(value / HBM_PEAK_GBPS, 4),
         "rows_per_s": round(args.steps * w.rows / dt, 1),
         # the dominant launcher: groups of back-to-back launches between event pairs, right after the regions
-        "roofline": roofline_of(name, dom_name, dom_bytes, dom_ms, rev_ceiling if w.has_reverse else fwd_ceiling),
+        "roofline": roofline_of(name, dom_name, dom_bytes, dom_ms, rev_ceiling if w.has_reverse else fwd_ceiling,
+                                on_its_own_ms=rev_ms if w.has_reverse else None),
         name: per_workload,
     }
     # one launch of the dominant launcher inside each timed region, events around it (pair included)
@@ -597,8 +645,8 @@ def main():
                 for i in range(4):
                     _step(osets, i)
                 torch.cuda.synchronize()
-            f_ms, r_ms = time_each(osets, k)
-            extra[other] = rates(o, f_ms, r_ms)
+            f_ms, r_ms, s_ms = time_each(osets, k)
+            extra[other] = rates(o, f_ms, r_ms, s_ms)
             extra[other]["workload"] = W.DESCRIPTION[other]
             if other == "cfg1":  # launch-bound: also the rate with the host out of the loop
                 g_ms, same = graph_forward_ms(osets)
@@ -618,7 +666,8 @@ def main():
             if other.startswith("cfg") or other == "chain":  # the same roofline object as the headline workload carries
                 f_ceil, r_ceil = (None, None) if args.no_ceilings or other == "cfg1" else ceilings_for(o)
                 if o.has_reverse:
-                    extra[other]["roofline"] = roofline_of(other, "reverse", o.rev_bytes, r_ms, r_ceil)
+                    extra[other]["roofline"] = roofline_of(other, "reverse", o.rev_bytes, reverse_in_step(f_ms, s_ms), r_ceil,
+                                                           on_its_own_ms=r_ms)
                     extra[other]["roofline_fwd"] = roofline_of(other, "forward", o.fwd_bytes, f_ms, f_ceil)
                 else:
                     extra[other]["roofline"] = roofline_of(other, "forward", o.fwd_bytes, f_ms, f_ceil)

@@ -218,6 +218,16 @@ __device__ __forceinline__ void store_pack_nt(T* p, const P (&in)[W]) {
   }
 }
 
+/* An output that another kernel reads again soon (a forward's result, read by its reverse): an
+ * ordinary store leaves it in the memory-side cache, a non-temporal one does not. A template
+ * parameter and not a branch: the compiler merges two stores that differ in the hint alone, and
+ * drops the hint. */
+template <bool KEEP, class T, int W, class P>
+__device__ __forceinline__ void store_pack_kept(T* p, const P (&in)[W]) {
+  if constexpr (KEEP) store_pack<T, W>(p, in);
+  else store_pack_nt<T, W>(p, in);
+}
+
 /* The four accessors above for packs that start at any element (see loose_vec_of). */
 template <class T, int W, class P>
 __device__ __forceinline__ void load_pack_loose(const T* p, P (&out)[W]) {
@@ -459,12 +469,12 @@ template <class T, int W, int G, int NV, bool RAGGED> struct RowTile {
     }
   }
 
-  __device__ __forceinline__ void store(T* row, const RowGeom<T, W>& g, int lane) const {
+  template <bool KEEP = false> __device__ __forceinline__ void store(T* row, const RowGeom<T, W>& g, int lane) const {
     T* body = row + g.head;
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = k * G + lane;
-      if (p < g.nvec) store_pack_nt<T, W>(body + (size_t)p * W, v[k]);
+      if (p < g.nvec) store_pack_kept<KEEP, T, W>(body + (size_t)p * W, v[k]);
     }
     if constexpr (RAGGED) {
       if (lane < g.head) row[lane] = (T)edge;

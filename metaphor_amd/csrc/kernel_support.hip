@@ -98,6 +98,14 @@ extern "C" void mpSetClusterWords(len_t own) {
   mp::cluster_tuning().own_words = (int)own;
 }
 
+// Diagnostic: what the forward kernels leave in the memory-side cache for their reverse (the RMSNorm
+// forward's loads of x, the softmax forward's stores of y): 0 nothing (streaming accesses whatever the
+// size), 1 always, 2 (as shipped) by the size of the tensor. Process-wide.
+extern "C" void mpSetKeepInput(len_t mode) {
+  mp::require(mode <= 2, "mpSetKeepInput: 0, 1 or 2");
+  mp::cluster_tuning().keep_input = mode == 2 ? -1 : (int)mode;
+}
+
 // Diagnostic: what the row launchers decide for [m, n] rows of a dtype on a GPU of `cus` compute
 // units, for every n in [n_lo, n_hi), without a GPU: each launcher runs its whole dispatch on a dry
 // run (kernel_header.h: MpPlanNote) and the kernel it would enqueue is written to notes[n - n_lo],

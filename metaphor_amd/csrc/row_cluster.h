@@ -55,6 +55,7 @@ struct ClusterTuning {
   unsigned spin_limit = 1u << 22;
   int deep = 0; /* the RMSNorm reverse's shared rows: 0 by the launcher's rule, 1 always the pipelined kernel, 2 never */
   int own_words = 1; /* stamped exchange words: 1 in the library's own memory where a region is to be had, 0 always in the caller's workspace */
+  int keep_input = -1; /* what a forward leaves in the memory-side cache for its reverse (keep_input, keep_output): -1 by tensor size, 0 nothing, 1 always */
 };
 #ifdef MP_DIAGNOSTICS
 inline ClusterTuning& cluster_tuning() {
@@ -64,6 +65,32 @@ inline ClusterTuning& cluster_tuning() {
 #else
 constexpr ClusterTuning cluster_tuning() { return ClusterTuning{}; }
 #endif
+
+/* What a forward leaves in the memory-side cache (256 MiB in front of the HBM stacks, shared by the
+ * eight XCDs) for the reverse that follows it. Streaming (non-temporal) accesses leave nothing
+ * there, ordinary ones do, and a streaming load that finds its line there is served from it. So a
+ * forward whose input the reverse reads again (RMSNorm: x) loads it with ordinary loads, a forward
+ * whose output the reverse reads (softmax: y) stores it with ordinary stores, and everything else
+ * stays streaming (ordinary stores of the rest push the kept tensor out again). Measured as steps
+ * of a forward and its reverse on tensors not touched for several steps, against the same with
+ * streaming accesses throughout, and the forward on its own:
+ *   RMSNorm r32 [8192, 4096] (128 MiB a tensor): step 110.4 -> 103.4 us, forward 43.3 -> 44.2;
+ *     [16384, 4096] (256 MiB): 214.8 -> 202.1, 85.8 -> 87.8; [32768, 4096] (512 MiB): 435.4 -> 418.9, 179.4 -> 182.1;
+ *   softmax r32 [8192, 4096]: step 105.7 -> 96.9, forward 42.5 -> 43.8; [512, 151936] (296 MiB):
+ *     246.6 -> 236.9, 99.0 -> 107.1; r16 [16384, 16384] (512 MiB): 424.7 -> 414.7, 173.2 -> 179.5.
+ * A forward that no reverse follows pays for it, little for kept loads, more for kept stores of
+ * tensors beyond the cache; the launchers cannot know what follows and keep by tensor size:
+ * inputs up to the size of the cache, outputs up to half of it. */
+constexpr size_t KEEP_INPUT_BYTES = 256u << 20;
+constexpr size_t KEEP_OUTPUT_BYTES = 128u << 20;
+inline bool keep_input(size_t tensor_bytes) {
+  const int mode = cluster_tuning().keep_input;
+  return mode < 0 ? tensor_bytes <= KEEP_INPUT_BYTES : mode != 0;
+}
+inline bool keep_output(size_t tensor_bytes) {
+  const int mode = cluster_tuning().keep_input;
+  return mode < 0 ? tensor_bytes <= KEEP_OUTPUT_BYTES : mode != 0;
+}
 
 /* Workgroups per row that a workspace must provide words for, given the number c the launcher
  * would use now. As shipped that is c itself (nothing can change it between the size query and

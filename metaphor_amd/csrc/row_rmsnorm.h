@@ -47,11 +47,13 @@ __device__ __forceinline__ void group_allreduce_sum2(P& a, P& b, P* slots_a, P* 
 
 /* ------------------------------------------------------------------ resident forward */
 
+/* KEEP: x through ordinary loads, which leave it in the memory-side cache for the reverse
+ * (keep_input, row_cluster.h). */
 /* LOOSE = false: x, gain and y 16-byte aligned and n % W == 0. LOOSE = true: any alignment of the
  * three and any n; the packs start at the row's first element (see RowPacks), so a thread's
  * columns, and with them its gain, are the same in every row (gain read element by element for
  * rows that each peel differently: r32 n = 257 3.3 TB/s). */
-template <class T, int W, int G, int NV, bool LOOSE, int BLOCK = NORM_BLOCK>
+template <class T, int W, int G, int NV, bool LOOSE, int BLOCK = NORM_BLOCK, bool KEEP = false>
 __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
   using P = typename precision<T>::type;
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
     for (int k = 0; k < NV; ++k) {
       const int p = k * G + lane;
       if (live && p < rp.npk) {
-        rp.template load<true>(xr, p, xv[k]);
+        rp.template load<!KEEP>(xr, p, xv[k]);
       } else {
 #pragma unroll
         for (int i = 0; i < W; ++i) xv[k][i] = (P)0;
@@ -134,7 +136,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
  * repeats: r16 n = 1152 5.26 -> 5.67 TB/s, r32 n = 1280 5.78 -> 5.94, six other widths -2 ... +1 %). */
 constexpr int ANY_MAX_ROWS = 8; /* groups per workgroup the LDS of the wavefront-group kernels is sized for */
 
-template <class T, int W, int NV>
+template <class T, int W, int NV, bool KEEP = false>
 __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_fwd_any(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n, int gw) {
   using P = typename precision<T>::type;
@@ -161,7 +163,8 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_fwd_any(
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = k * G + lane;
-      xs[k] = __builtin_nontemporal_load(reinterpret_cast<const V*>(xr + (size_t)(p < npk ? p : 0) * W));
+      const V* at = reinterpret_cast<const V*>(xr + (size_t)(p < npk ? p : 0) * W);
+      xs[k] = KEEP ? *at : __builtin_nontemporal_load(at);
     }
   };
   auto finish = [&](const V (&xs)[NV], size_t base, P (*sl)[NW]) {
@@ -1616,6 +1619,8 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
    * two packs per thread for the same effect (n = 1024: 5.6 -> 6.1) and
    * nothing beats the persistent kernel below 32 packs a row. Measured on the MI355X. */
   constexpr int ONESHOT = 256;
+  /* aligned rows of whole packs: x through loads that leave it in the memory-side cache for the reverse */
+  const bool keep = keep_input(m * n * sizeof(T));
   /* rows whose packs start at any element: two packs a thread, so that a row one pack over a power
    * of two does not idle half of a group twice as wide (r32 n = 257: 4.1 -> 5.1 TB/s, n = 130: 3.8 -> 4.9) */
   const int nv_target = sizeof(T) == 2 || loose ? 2 : 1;
@@ -1634,7 +1639,8 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
     const size_t need = (m + NORM_BLOCK / 128 - 1) / (NORM_BLOCK / 128);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
     if (note_plan(PLAN_RESIDENT, 128, 2, NORM_BLOCK / 128, grid.x, block.x)) return;
-    rmsnorm_fwd_resident<T, W, 128, 2, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+    if (keep) rmsnorm_fwd_resident<T, W, 128, 2, false, NORM_BLOCK, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+    else rmsnorm_fwd_resident<T, W, 128, 2, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
     MP_CHECK_LAUNCH();
     return;
   }
@@ -1646,8 +1652,13 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
       const size_t need = (m + rpb - 1) / rpb;
       const dim3 grid((unsigned)(need < cap ? need : cap)), block(rpb * gw * WAVE);
       if (note_plan(PLAN_ANY, gw * WAVE, shot.NV, rpb, grid.x, block.x)) return;
-      if (shot.NV == 1) rmsnorm_fwd_any<T, W, 1><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
-      else rmsnorm_fwd_any<T, W, 2><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
+      if (shot.NV == 1) {
+        if (keep) rmsnorm_fwd_any<T, W, 1, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
+        else rmsnorm_fwd_any<T, W, 1><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
+      } else {
+        if (keep) rmsnorm_fwd_any<T, W, 2, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
+        else rmsnorm_fwd_any<T, W, 2><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
+      }
       MP_CHECK_LAUNCH();
       return;
     }
@@ -1662,6 +1673,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
         const dim3 grid((unsigned)need), block(ONESHOT);
         if (note_plan(PLAN_RESIDENT, G, NV, ONESHOT / G, grid.x, block.x)) return;
         if (loose) rmsnorm_fwd_resident<T, W, G, NV, true, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+        else if (keep) rmsnorm_fwd_resident<T, W, G, NV, false, ONESHOT, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
         else rmsnorm_fwd_resident<T, W, G, NV, false, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
       }
     });
@@ -1680,6 +1692,8 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
     if (note_plan(PLAN_RESIDENT, G, NV, NORM_BLOCK / G, grid.x, block.x)) return;
     if (loose) rmsnorm_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
+    else if (keep)
+      rmsnorm_fwd_resident<T, W, G, NV, false, NORM_BLOCK, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
     else rmsnorm_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
   });
   if (!resident && !note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, m < cap ? m : cap, STREAM_THREADS)) {

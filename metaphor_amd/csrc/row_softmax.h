@@ -87,7 +87,10 @@ __global__ __launch_bounds__(SHORT_THREADS) void softmax_rev_short(
 
 /* ------------------------------------------------------------------ resident forward */
 
-template <class T, int W, int G, int NV, bool RAGGED>
+/* KEEP: y through ordinary stores, which leave it in the memory-side cache for the reverse
+ * (keep_output, row_cluster.h). */
+
+template <class T, int W, int G, int NV, bool RAGGED, bool KEEP = false>
 __global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_fwd_resident(
     const T* x, T* y, size_t m, size_t n, unsigned by_xcd) {
   using P = typename precision<T>::type;
@@ -116,7 +119,7 @@ __global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_fwd_resident(
 
   const P inv = (P)1 / s;
   t.each([&](P& e) { e *= inv; });
-  if (live) t.store(y + row * n, g, lane);
+  if (live) t.template store<KEEP>(y + row * n, g, lane);
 }
 
 /* ------------------------------------------------------------------ resident reverse */
@@ -423,7 +426,7 @@ template <class T> constexpr int cluster_nv() {
   return 24 / ((PACK_BYTES / (int)sizeof(T)) * (int)(sizeof(typename precision<T>::type) / 4));
 }
 
-template <class T, int W>
+template <class T, int W, bool KEEP = false>
 __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
     const T* x, T* y, share_word* callers_words, size_t region,
     size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
@@ -570,7 +573,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
         P out[W];
 #pragma unroll
         for (int i = 0; i < W; ++i) out[i] = exp_shifted((P)v[k][i], shM) * inv;
-        store_pack_nt<T, W>(ybody + (size_t)p * W, out);
+        store_pack_kept<KEEP, T, W>(ybody + (size_t)p * W, out);
       }
     }
     if (edge_at != (size_t)-1) yr[edge_at] = (T)(exp_shifted(edge_x, shM) * inv);
@@ -581,7 +584,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
       if (p >= 0 && p < hi) {
 #pragma unroll
         for (int i = 0; i < W; ++i) v[k][i] *= scale;
-        store_pack_nt<T, W>(ybody + (size_t)p * W, v[k]);
+        store_pack_kept<KEEP, T, W>(ybody + (size_t)p * W, v[k]);
       }
     }
     if (edge_at != (size_t)-1) yr[edge_at] = (T)(edge * scale);
@@ -909,8 +912,12 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
         cluster_zero_slots<share_word><<<dim3((unsigned)((words + 255) / 256)), dim3(256), 0, stream>>>(callers, words);
       }
     }
-    softmax_fwd_cluster<T, W><<<dim3((unsigned)(m * C)), dim3(CLUSTER_THREADS), 0, stream>>>(
-        x, y, callers, (size_t)region, m, n, C, ppb, cluster_tuning().spin_limit);
+    if (keep_output(m * n * sizeof(T)))
+      softmax_fwd_cluster<T, W, true><<<dim3((unsigned)(m * C)), dim3(CLUSTER_THREADS), 0, stream>>>(
+          x, y, callers, (size_t)region, m, n, C, ppb, cluster_tuning().spin_limit);
+    else
+      softmax_fwd_cluster<T, W><<<dim3((unsigned)(m * C)), dim3(CLUSTER_THREADS), 0, stream>>>(
+          x, y, callers, (size_t)region, m, n, C, ppb, cluster_tuning().spin_limit);
     MP_CHECK_LAUNCH();
     return;
   }
@@ -931,11 +938,14 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   else if (FIT && row_regime_override() == REGIME_AUTO && plan.NV == 2 && plan.G >= 128 && plan.G <= 512 && MAXNV >= 4 &&
            packs * 16 <= (size_t)plan.G * 2 * 11)
     plan = RowPlan{plan.G / 2, 4};
+  const unsigned flags = rows_share_lines<T>(n);
+  const bool keep = keep_output(m * n * sizeof(T));
   const bool resident = for_row_plan<MAXNV, true, FIT>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (note_plan(PLAN_RESIDENT, G, NV, G < WAVE ? WAVE / G : 1, grid.x, block.x)) return;
-    if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
-    else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n, rows_share_lines<T>(n));
+    if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n, flags);
+    else if (keep) softmax_fwd_resident<T, W, G, NV, false, true><<<grid, block, 0, stream>>>(x, y, m, n, flags);
+    else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n, flags);
   });
   if (!resident && !note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, stream_grid(m), STREAM_THREADS))
     softmax_fwd_stream<T, W><<<dim3(stream_grid(m)), dim3(STREAM_THREADS), 0, stream>>>(x, y, m, n);
@@ -1043,15 +1053,16 @@ inline void softmax_reverse(const T* y, const T* dy, T* dx, void* scratch, doubl
    * 401 ... 512 packs take one pack on 512 threads (against two on 256: n = 3584 6.02 -> 6.25, 3840 5.98 ->
    * 6.46, 4096 6.10 -> 6.33; 3328 equal, 3072 better at two) */
   const RowPlan plan = row_regime_override() == REGIME_CLUSTER ? RowPlan{0, 0} : plan_row(packs, MAXNV, one_pack ? 1 : 2, 16);
+  const unsigned rev_flags = rows_share_lines<T>(n);
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
     if (note_plan(PLAN_RESIDENT, G, NV, G < WAVE ? WAVE / G : 1, grid.x, block.x)) return;
     if (ragged) {
-      if (blend) softmax_rev_resident<T, W, G, NV, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
-      else softmax_rev_resident<T, W, G, NV, true, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
+      if (blend) softmax_rev_resident<T, W, G, NV, true, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rev_flags);
+      else softmax_rev_resident<T, W, G, NV, true, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rev_flags);
     } else {
-      if (blend) softmax_rev_resident<T, W, G, NV, false, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
-      else softmax_rev_resident<T, W, G, NV, false, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rows_share_lines<T>(n));
+      if (blend) softmax_rev_resident<T, W, G, NV, false, true><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rev_flags);
+      else softmax_rev_resident<T, W, G, NV, false, false><<<grid, block, 0, stream>>>(y, dy, dx, al, m, n, rev_flags);
     }
   });
   if (!resident && !note_plan(PLAN_STREAM, STREAM_THREADS, 0, 1, stream_grid(m), STREAM_THREADS)) {

@@ -43,7 +43,7 @@ def lib():
 ROW_STEMS = ("softmax_ij_j", "softmax_ij_j_reverse", "rmsnorm_ij_j", "rmsnorm_ij_j_reverse")
 ROW_SIZE_FNS = ("mpSoftmaxScratchBytes", "mpSoftmaxReverseScratchBytes", "mpRmsnormScratchBytes",
                 "mpRmsnormReverseScratchBytes")
-_diag = {"lib": None, "regime": 0, "tuned": False, "deep": 0, "own_words": 1}
+_diag = {"lib": None, "regime": 0, "tuned": False, "deep": 0, "own_words": 1, "keep_input": 2}
 
 
 def diag_lib():
@@ -69,12 +69,14 @@ def diag_lib():
         d.mpSetClusterDeep.restype = None
         d.mpSetClusterWords.argtypes = [ffi.len_t]
         d.mpSetClusterWords.restype = None
+        d.mpSetKeepInput.argtypes = [ffi.len_t]
+        d.mpSetKeepInput.restype = None
         _diag["lib"] = d
     return _diag["lib"]
 
 
 def _override_active():
-    return _diag["regime"] != 0 or _diag["tuned"] or _diag["deep"] != 0 or _diag["own_words"] != 1
+    return _diag["regime"] != 0 or _diag["tuned"] or _diag["deep"] != 0 or _diag["own_words"] != 1 or _diag["keep_input"] != 2
 
 
 def row_size(fn, dtype, m, n):
@@ -423,6 +425,13 @@ def set_cluster_words(own=1):
     library's own memory (as shipped), 0 in the caller's workspace, cleared before every launch."""
     diag_lib().mpSetClusterWords(int(own))
     _diag["own_words"] = int(own)
+
+
+def set_keep_input(mode=2):
+    """How the resident RMSNorm forward of the test build loads x: 0 streaming loads, 1 loads that
+    leave x in the memory-side cache, 2 by the size of the tensor (as shipped)."""
+    diag_lib().mpSetKeepInput(int(mode))
+    _diag["keep_input"] = int(mode)
 
 
 def permutate(src, dst, alpha=0.0):

@@ -313,6 +313,26 @@ def test_column_sums_with_workspace(dtype):
     assert used > 0, "no shape took the two-stage path"
 
 
+def test_column_sums_without_a_workspace_say_so_at_most_once(capfd):
+    """launch_reduce_ij_j through a bare stream context has no workspace to split a tall, narrow
+    matrix through: the result is the same, and the library says what that costs once a process."""
+    r = rng(18)
+    f32 = torch.float32
+    notes = 0
+    for (m, n) in [(60000, 8), (90001, 12)]:
+        G.say(f"reduce_ij_j through a bare context shape=({m},{n})")
+        src, dst = G.dev(r.normal(0, 1, (m, n)), f32), G.Guarded((n,), f32)
+        capfd.readouterr()
+        G.matrix_op("reduce_ij_j", src.t, dst.t, 0.0, m, n)
+        torch.cuda.synchronize()
+        notes += capfd.readouterr().err.count("given no workspace")
+        ref = O.reduce_ij_j(G.host(src.t), None, 0.0)
+        G.compare(dst.t, ref, f32, f"reduce_ij_j bare ({m},{n})", rowwise=False,
+                  scale=np.abs(G.host(src.t).astype(np.float64)).sum(axis=0))
+        dst.check("column sums")
+    assert notes <= 1, "the note about the missing workspace was printed more than once"
+
+
 @pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
 def test_column_sums_on_a_library_stream(dtype):
     """launch_reduce_ij_j has the reference's signature (no workspace): on a stream made by
@@ -428,6 +448,39 @@ def test_softmax_forward_cluster_path(dtype, packs, spin):
                     assert bool((y.t[torch.isinf(x.t)] == 0).all())
                 x.check("x")
                 y.check("y")
+
+
+@pytest.mark.parametrize("dtype", DTYPES, ids=IDS)
+def test_forward_results_do_not_depend_on_what_is_left_in_the_cache(dtype):
+    """The forward kernels come in two flavours that differ in a cache hint alone: the RMSNorm forward
+    loads x, and the softmax forward stores y, so that the tensor stays in the memory-side cache
+    for the reverse (tensors up to a size) or streams past it (larger ones). Both flavours of every
+    kernel that has them, forced through the test build: the same bits, and within the bound of the
+    oracle. Row lengths: one per forward path (one-shot groups, persistent groups, groups of whole
+    wavefronts, eight rows a workgroup, rows shared by workgroups)."""
+    r = rng(53)
+    eps = 1e-6
+    try:
+        for (m, n) in [(37, 512), (19, 1152), (23, 1280), (9, 4096), (5, 16384), (3, 50257), (2, 151936)]:
+            x = G.dev(r.normal(0, 2, (m, n)), dtype)
+            g = G.dev(1 + 0.1 * r.normal(0, 1, n), dtype)
+            xh, gh = G.host(x.t), G.host(g.t)
+            got = {}
+            for mode in (0, 1):
+                G.set_keep_input(mode)
+                G.say(f"cache policy {mode} dtype={dtype} shape=({m},{n})")
+                y, z = G.Guarded((m, n), dtype), G.Guarded((m, n), dtype)
+                G.rmsnorm(x.t, g.t, y.t, eps)
+                G.softmax(x.t, z.t)
+                G.compare(y.t, O.rmsnorm_ij_j(xh, gh, eps), dtype, f"rmsnorm policy {mode} ({m},{n})")
+                G.compare(z.t, O.softmax_ij_j(xh), dtype, f"softmax policy {mode} ({m},{n})", **G.softmax_tol(dtype))
+                y.check("y")
+                z.check("z")
+                got[mode] = (y.t.clone(), z.t.clone())
+            assert torch.equal(got[0][0], got[1][0]), f"rmsnorm ({m},{n}): the two flavours differ"
+            assert torch.equal(got[0][1], got[1][1]), f"softmax ({m},{n}): the two flavours differ"
+    finally:
+        G.set_keep_input(2)
 
 
 @pytest.mark.parametrize("own", [1, 0], ids=["library-words", "caller-words"])
