@@ -120,8 +120,22 @@ __device__ __forceinline__ float shift_of(float m) { return m * 1.44269504088896
 __device__ __forceinline__ double exp_shifted(double x, double m) { return ::exp(x - m); }
 __device__ __forceinline__ double shift_of(double m) { return m; }
 
-__device__ __forceinline__ float rsqrt_of(float x) { return 1.0f / __builtin_sqrtf(x); }
+/* 1 / sqrt(x) from the hardware's reciprocal square root (good to one ulp) instead of an IEEE
+ * square root and an IEEE division, some forty instructions that every lane of a row would spend
+ * on the same number. The instruction reads denormal arguments as zero: tiny ones are scaled
+ * into range first (x = 0 still gives +inf). */
+__device__ __forceinline__ float rsqrt_of(float x) {
+  const bool tiny = x < 0x1p-100f;
+  const float r = __builtin_amdgcn_rsqf(tiny ? x * 0x1p+100f : x);
+  return tiny ? r * 0x1p+50f : r;
+}
 __device__ __forceinline__ double rsqrt_of(double x) { return 1.0 / ::sqrt(x); }
+
+/* 1 / x for a row's sum (x >= 1 for a softmax row that has a finite element; 0 gives +inf as the
+ * division does): the hardware's reciprocal, good to one ulp, instead of the ten instructions of
+ * an IEEE division that every lane of the row would spend on the same number. */
+__device__ __forceinline__ float reciprocal_of(float x) { return __builtin_amdgcn_rcpf(x); }
+__device__ __forceinline__ double reciprocal_of(double x) { return 1.0 / x; }
 
 /* e^x - 1 for x <= 0, accurate near 0: an 8-term series inside (-0.25, 0], exp-1 below. */
 __device__ __forceinline__ float expm1_nonpos(float x) {

@@ -57,6 +57,7 @@ template <class T, int W, int G, int NV, bool LOOSE, int BLOCK = NORM_BLOCK, boo
 __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   constexpr int RPB = BLOCK / G;
   static_assert(G >= W, "the first lanes of a group hold the elements behind the last whole pack");
   __shared__ P slots[2][G < WAVE ? 1 : RPB][G < WAVE ? 1 : G / WAVE];
@@ -106,7 +107,7 @@ __global__ __launch_bounds__(BLOCK) void rmsnorm_fwd_resident(
 #pragma unroll
       for (int i = 0; i < W; ++i) ss += xv[k][i] * xv[k][i];
     ss = group_allreduce<AddOP, G>(ss, slots[parity][G < WAVE ? 0 : sub], lane);
-    const P r = rsqrt_of(ss / (P)n + eps);
+    const P r = rsqrt_of(ss * inv_n + eps);
 
     if (live) {
       T* yr = y + row * n;
@@ -140,6 +141,7 @@ template <class T, int W, int NV, bool KEEP = false>
 __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_fwd_any(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n, int gw) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   using V = typename vec_of<T, W>::type;
   constexpr int NW = NORM_BLOCK / WAVE;
   __shared__ P slots[2][ANY_MAX_ROWS][NW];
@@ -182,7 +184,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_fwd_any(
     lds_barrier();
     const int slot = lane & (NW - 1);
     ss = fold_partials<AddOP, NW>(slot < gw ? sl[sub][slot] : (P)0);
-    const P r = rsqrt_of(ss / (P)n + eps);
+    const P r = rsqrt_of(ss * inv_n + eps);
     if (row < m) {
       T* yr = y + row * n;
 #pragma unroll
@@ -222,6 +224,7 @@ template <class T, int W, bool APART = false>
 __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_fwd_stream(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, size_t n) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   constexpr int G = STREAM_THREADS, U = 4;
   __shared__ P slots[2][G / WAVE];
   const int lane = threadIdx.x;
@@ -259,7 +262,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_fwd_stream(
       if (edge != (size_t)-1) ss += (P)xr[edge] * (P)xr[edge];
     }
     ss = group_allreduce<AddOP, G>(ss, slots[parity], lane);
-    const P r = rsqrt_of(ss / (P)n + eps);
+    const P r = rsqrt_of(ss * inv_n + eps);
 
     for (int p = lane; p < g.nvec; p += G) {
       P buf[W], gv[W];
@@ -288,6 +291,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void rmsnorm_fwd_cluster(
     typename slot_word<typename precision<T>::type>::type* slots,
     size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   using V = typename vec_of<T, W>::type;
   constexpr int G = CLUSTER_THREADS, NV = NORM_CLUSTER_NV;
   __shared__ P red[2][G / WAVE];
@@ -352,7 +356,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void rmsnorm_fwd_cluster(
     }
   }
 
-  const P r = rsqrt_of(ss / (P)n + eps);
+  const P r = rsqrt_of(ss * inv_n + eps);
   T* ybody = yr + g.head;
   const T* gbody = gain + g.head;
   const bool gain_packed = (reinterpret_cast<uintptr_t>(gbody) & 15u) == 0;
@@ -405,6 +409,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n, unsigned by_xcd) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   constexpr int RPB = NORM_BLOCK / G;
   __shared__ P slots[2][2][G < WAVE ? 1 : RPB][G < WAVE ? 1 : G / WAVE];
   __shared__ P comb[RPB > 1 ? NORM_BLOCK * NV * W : 1]; /* one row of dg sums per group of the workgroup */
@@ -450,8 +455,8 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_resident(
         c += dv[k][i] * gv[k][i] * xv[k][i];
       }
     group_allreduce_sum2<G>(ss, c, slots[parity][0][G < WAVE ? 0 : sub], slots[parity][1][G < WAVE ? 0 : sub], lane);
-    const P r = rsqrt_of(ss / (P)n + eps);
-    const P cc = c / (P)n * r * r;
+    const P r = rsqrt_of(ss * inv_n + eps);
+    const P cc = c * inv_n * r * r;
 
     if (live) {
 #pragma unroll
@@ -538,11 +543,12 @@ __device__ __forceinline__ void group_allreduce_sum2_lds(P& a, P& b, P* slots_a,
  * many partial rows. EXACT: every thread's NV packs lie inside the row (n == G * NV * W).
  * DEPTH 3: three register sets, two rows on their way while a third is reduced; the launcher says
  * where that pays. */
-template <class T, int W, int G, int NV, bool BLEND, bool EXACT, int DEPTH = 2>
-__global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
+template <class T, int W, int G, int NV, bool BLEND, bool EXACT, int DEPTH = 2, int WPE = 1>
+__global__ __launch_bounds__(NORM_BLOCK, WPE) void rmsnorm_rev_paired(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   using V = typename vec_of<T, W>::type;
   static_assert(G > WAVE && G <= NORM_BLOCK, "groups of 128 ... 1024 threads");
   constexpr int RPB = NORM_BLOCK / G;
@@ -593,8 +599,8 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
       }
     }
     group_allreduce_sum2_lds<G>(ss, c, sl[0][sub], sl[1][sub], lane);
-    const P r = rsqrt_of(ss / (P)n + eps);
-    const P cc = c / (P)n * r * r;
+    const P r = rsqrt_of(ss * inv_n + eps);
+    const P cc = c * inv_n * r * r;
     if (live) {
       T* out_row = dx + row * n;
 #pragma unroll
@@ -690,6 +696,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n, int gw) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   using V = typename vec_of<T, W>::type;
   constexpr int NW = NORM_BLOCK / WAVE;
   __shared__ P slots[DEPTH][2][ANY_MAX_ROWS][NW];
@@ -751,8 +758,8 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired_any(
     const int slot = lane & (NW - 1);
     ss = fold_partials<AddOP, NW>(slot < gw ? sl[0][sub][slot] : (P)0);
     c = fold_partials<AddOP, NW>(slot < gw ? sl[1][sub][slot] : (P)0);
-    const P r = rsqrt_of(ss / (P)n + eps);
-    const P cc = c / (P)n * r * r;
+    const P r = rsqrt_of(ss * inv_n + eps);
+    const P cc = c * inv_n * r * r;
     if (live) {
       T* out_row = dx + row * n;
 #pragma unroll
@@ -841,6 +848,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   constexpr int G = STREAM_THREADS, U = 2;
   __shared__ P slots[2][2][G / WAVE];
   const int lane = threadIdx.x;
@@ -880,8 +888,8 @@ __global__ __launch_bounds__(STREAM_THREADS) void rmsnorm_rev_stream(
         }
     }
     group_allreduce_sum2<G>(ss, c, slots[parity][0], slots[parity][1], lane);
-    const P r = rsqrt_of(ss / (P)n + eps);
-    const P cc = c / (P)n * r * r;
+    const P r = rsqrt_of(ss * inv_n + eps);
+    const P cc = c * inv_n * r * r;
 
     auto finish_pack = [&](int p, P (&sum)[W], bool in_registers) {
       P xv[W], dv[W], gv[W], out[W];
@@ -957,6 +965,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
     typename slot_word<typename precision<T>::type>::type* slots,
     size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   using V = typename vec_of<T, W>::type;
   constexpr int G = CLUSTER_THREADS, NV = norm_rev_cluster_nv<T>();
   __shared__ P red[2][2][G / WAVE];
@@ -1064,8 +1073,8 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 4 * norm_rev_cluster_per_cu<T>()) 
     if constexpr (AHEAD) {
       if (fetch_late && row + S < m) fetch(row + S, xn, dn);
     }
-    const P r = rsqrt_of(ss / (P)n + eps);
-    const P cc = c / (P)n * r * r;
+    const P r = rsqrt_of(ss * inv_n + eps);
+    const P cc = c * inv_n * r * r;
 
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
@@ -1147,6 +1156,7 @@ __global__ __launch_bounds__(CLUSTER_THREADS) void rmsnorm_rev_cluster_deep(
     typename slot_word<typename precision<T>::type>::type* slots,
     size_t m, size_t n, int C, int packs_per_block, unsigned spin_limit) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   using V = typename vec_of<T, W>::type;
   using Word = typename slot_word<P>::type;
   constexpr int G = CLUSTER_THREADS, D = DEEP_LANES, NV = 2, NW = G / WAVE;
@@ -1284,8 +1294,8 @@ __global__ __launch_bounds__(CLUSTER_THREADS) void rmsnorm_rev_cluster_deep(
       c = fold_partials<AddOP, NW>(fb[1][lane & (NW - 1)]);
       __syncthreads(); /* fb is free again */
     }
-    const P r = rsqrt_of(ss / (P)n + eps);
-    const P cc = c / (P)n * r * r;
+    const P r = rsqrt_of(ss * inv_n + eps);
+    const P cc = c * inv_n * r * r;
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = lo + k * D + lane;
@@ -1455,6 +1465,7 @@ template <class T, int W, int G, bool CUT>
 __global__ __launch_bounds__(SHORT_THREADS) void rmsnorm_fwd_short(
     const T* x, const T* gain, T* y, typename precision<T>::type eps, size_t m, unsigned n, unsigned by_xcd) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   const int lane = threadIdx.x % G;
   bool live;
   const size_t row = short_row_of<G>(m, by_xcd, live);
@@ -1465,7 +1476,7 @@ __global__ __launch_bounds__(SHORT_THREADS) void rmsnorm_fwd_short(
 #pragma unroll
   for (int i = 0; i < W; ++i) ss += t.v[i] * t.v[i];
   ss = fold_partials<AddOP, G>(ss);
-  const P r = rsqrt_of(ss / (P)n + eps);
+  const P r = rsqrt_of(ss * inv_n + eps);
 #pragma unroll
   for (int i = 0; i < W; ++i) t.v[i] *= r * g.v[i];
   if (live) t.store(y + row * n, n, lane);
@@ -1479,6 +1490,7 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_short(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, unsigned n) {
   using P = typename precision<T>::type;
+  const P inv_n = (P)1 / (P)n; /* one division a thread, not two a row */
   constexpr int RPB = NORM_BLOCK / G, WAVES = NORM_BLOCK / WAVE;
   __shared__ P comb[WAVES][G * W];
   const int lane = threadIdx.x % G, sub = threadIdx.x / G;
@@ -1503,8 +1515,8 @@ __global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_short(
     }
     ss = fold_partials<AddOP, G>(ss);
     c = fold_partials<AddOP, G>(c);
-    const P r = rsqrt_of(ss / (P)n + eps);
-    const P cc = c / (P)n * r * r;
+    const P r = rsqrt_of(ss * inv_n + eps);
+    const P cc = c * inv_n * r * r;
     if (live) {
       ShortRow<T, W, G, CUT> out;
 #pragma unroll
@@ -1806,6 +1818,16 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
        * 4096 5.99 -> 5.81) */
       constexpr int DEPTH = NV == 1 && ((sizeof(T) == 2 && G <= 512) || G == 128) ? 3 : 2;
       auto go = [&]<bool BLEND, bool EXACT>() {
+#ifdef MP_DIAGNOSTICS
+        if constexpr (DEPTH == 2 && NV == 1 && sizeof(T) == 4 && G == 1024) {
+          if (cluster_tuning().deep == 1) { /* experiment: two workgroups a CU */
+            const size_t two = 2 * one_per_cu;
+            rows = (unsigned)(need < two ? need : two);
+            rmsnorm_rev_paired<T, W, G, NV, BLEND, EXACT, 2, 8><<<dim3(rows), block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
+            return;
+          }
+        }
+#endif
         rmsnorm_rev_paired<T, W, G, NV, BLEND, EXACT, DEPTH><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
       };
       if (blend) { if (exact) go.template operator()<true, true>(); else go.template operator()<true, false>(); }

@@ -52,7 +52,7 @@ __global__ __launch_bounds__(SHORT_THREADS) void softmax_fwd_short(const T* x, T
   }
   s = fold_partials<AddOP, G>(s);
 
-  const P inv = (P)1 / s;
+  const P inv = reciprocal_of(s);
 #pragma unroll
   for (int i = 0; i < W; ++i) t.v[i] *= inv;
   if (live) t.store(y + row * n, n, lane);
@@ -117,7 +117,7 @@ __global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_fwd_resident(
   t.each([&](P& e) { e = exp_shifted(e, sh); s += e; });
   s = group_allreduce<AddOP, G>(s, slots[1], lane);
 
-  const P inv = (P)1 / s;
+  const P inv = reciprocal_of(s);
   t.each([&](P& e) { e *= inv; });
   if (live) t.template store<KEEP>(y + row * n, g, lane);
 }
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(G < WAVE ? WAVE : G) void softmax_fwd_loose(const T
     }
   s = group_allreduce<AddOP, G>(s, slots[1], lane);
 
-  const P inv = (P)1 / s;
+  const P inv = reciprocal_of(s);
   if (!live) return;
 #pragma unroll
   for (int k = 0; k < NV; ++k) {
@@ -369,7 +369,7 @@ __global__ __launch_bounds__(STREAM_THREADS) void softmax_fwd_stream(
     const P sh = shift_of(mx);
     const P scaled = run_max > neg_inf<P>() ? run_sum * exp_shifted(run_max, sh) : (P)0;
     const P s = group_allreduce<AddOP, G>(scaled, slots[parity][1], lane);
-    const P inv = (P)1 / s;
+    const P inv = reciprocal_of(s);
 
     /* pass 2: the row again, normally still in cache */
     T* ybody = yr + g.head;
@@ -562,10 +562,10 @@ __global__ __launch_bounds__(CLUSTER_THREADS, 8) void softmax_fwd_cluster(
     }
   }
 
-  const P scale = exp_shifted(base_mx, shift_of(M)) / S;
+  const P scale = exp_shifted(base_mx, shift_of(M)) * reciprocal_of(S);
   T* ybody = yr + g.head;
   if constexpr (RAW) {
-    const P shM = shift_of(M), inv = (P)1 / S;
+    const P shM = shift_of(M), inv = reciprocal_of(S);
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
       const int p = lo + k * G + lane;
