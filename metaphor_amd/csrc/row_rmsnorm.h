@@ -543,8 +543,8 @@ __device__ __forceinline__ void group_allreduce_sum2_lds(P& a, P& b, P* slots_a,
  * many partial rows. EXACT: every thread's NV packs lie inside the row (n == G * NV * W).
  * DEPTH 3: three register sets, two rows on their way while a third is reduced; the launcher says
  * where that pays. */
-template <class T, int W, int G, int NV, bool BLEND, bool EXACT, int DEPTH = 2, int WPE = 1>
-__global__ __launch_bounds__(NORM_BLOCK, WPE) void rmsnorm_rev_paired(
+template <class T, int W, int G, int NV, bool BLEND, bool EXACT, int DEPTH = 2>
+__global__ __launch_bounds__(NORM_BLOCK) void rmsnorm_rev_paired(
     const T* x, const T* gain, const T* dy, T* dx, typename precision<T>::type* partials,
     typename precision<T>::type eps, typename precision<T>::type alpha, size_t m, size_t n) {
   using P = typename precision<T>::type;
@@ -1818,16 +1818,6 @@ inline void rmsnorm_reverse_as(const T* x, const T* gain, const T* dy, T* dx, T*
        * 4096 5.99 -> 5.81) */
       constexpr int DEPTH = NV == 1 && ((sizeof(T) == 2 && G <= 512) || G == 128) ? 3 : 2;
       auto go = [&]<bool BLEND, bool EXACT>() {
-#ifdef MP_DIAGNOSTICS
-        if constexpr (DEPTH == 2 && NV == 1 && sizeof(T) == 4 && G == 1024) {
-          if (cluster_tuning().deep == 1) { /* experiment: two workgroups a CU */
-            const size_t two = 2 * one_per_cu;
-            rows = (unsigned)(need < two ? need : two);
-            rmsnorm_rev_paired<T, W, G, NV, BLEND, EXACT, 2, 8><<<dim3(rows), block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
-            return;
-          }
-        }
-#endif
         rmsnorm_rev_paired<T, W, G, NV, BLEND, EXACT, DEPTH><<<grid, block, 0, stream>>>(x, gain, dy, dx, partials, (P)eps, (P)alpha, m, n);
       };
       if (blend) { if (exact) go.template operator()<true, true>(); else go.template operator()<true, false>(); }
