@@ -7,6 +7,9 @@
 // mpSoftmaxScratchBytes(dtype, m, n) bytes (0 for rows that fit one workgroup) that lets several
 // workgroups share a long row; the reference's own softmax call sites already pass a scratch
 // buffer (src/loss/loss.zig:204,226). With scratch == NULL long rows are read twice instead.
+// An output of up to 128 MiB is written so that it stays in the GPU's memory-side cache, where the
+// reverse that reads it finds it (a step of forward and reverse gains 8 %, a forward on its own
+// pays 3 %); larger outputs stream past the cache.
 extern "C" void launch_softmax_ij_j_Scalar(
   const void* src,
   void* dst,

@@ -49,10 +49,12 @@ def test_shipped_libraries_export_no_process_wide_switches():
         out = subprocess.run(["nm"] + flags + [os.path.join(ffi.LIB_DIR, name)],
                              capture_output=True, text=True, check=True).stdout
         assert "mpSetRowRegime" not in out and "mpSetClusterTuning" not in out and "mpSetClusterDeep" not in out, name
+        assert "mpSetClusterWords" not in out and "mpSetKeepInput" not in out and "mpDescribeRowPlans" not in out, name
         assert "row_regime_override" not in out and "cluster_tuning" not in out, name
     diag = subprocess.run(["nm", "-D", "--defined-only", os.path.join(ffi.LIB_DIR, "libmp_kernels_diag.so")],
                           capture_output=True, text=True, check=True).stdout
     assert " T mpSetRowRegime" in diag and " T mpSetClusterTuning" in diag and " T mpSetClusterDeep" in diag
+    assert " T mpSetClusterWords" in diag and " T mpSetKeepInput" in diag and " T mpDescribeRowPlans" in diag
 
 
 def test_dispatch_arrays_are_r16_r32_r64_in_scalar_tag_order():
