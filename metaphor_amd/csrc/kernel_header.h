@@ -59,6 +59,7 @@ inline void mpHandleHipError(hipError_t err, const char* file, int line) {
  * 5 shared rows pipelined, 6 two passes, 7 rows that peel differently. */
 struct MpPlanNote {
   long long kind, group, packs_per_thread, rows_per_block, grid, block, cluster, chunk_packs, workspace_bytes;
+  long long kept; /* 1: the forward's variant that leaves a tensor in the memory-side cache */
 };
 struct MpPlanProbe {
   bool dry = false, noted = false;
@@ -516,11 +517,11 @@ template <class T, int W, int G, int NV, bool RAGGED> struct RowTile {
  * shipped; in the test build it records the decision and, on a dry run, says "do not launch". */
 #ifdef MP_DIAGNOSTICS
 inline bool note_plan(int kind, int group, int packs_per_thread, int rows_per_block, size_t grid, size_t block,
-                      int cluster = 1, int chunk_packs = 0, size_t workspace_bytes = 0) {
+                      int cluster = 1, int chunk_packs = 0, size_t workspace_bytes = 0, bool kept = false) {
   MpPlanProbe& p = mp_plan_probe();
   if (!p.dry) return false;
   p.note = MpPlanNote{kind, group, packs_per_thread, rows_per_block, (long long)grid, (long long)block, cluster, chunk_packs,
-                      (long long)workspace_bytes};
+                      (long long)workspace_bytes, kept ? 1 : 0};
   p.noted = true;
   return true;
 }

@@ -130,7 +130,7 @@ extern "C" len_t mpDescribeRowPlans(len_t op, len_t dtype, len_t m, len_t n_lo, 
   len_t noted = 0;
   for (len_t n = n_lo; n < n_hi; ++n) {
     probe.noted = false;
-    probe.note = MpPlanNote{-1, 0, 0, 0, 0, 0, 0, 0, 0};
+    probe.note = MpPlanNote{-1, 0, 0, 0, 0, 0, 0, 0, 0, 0};
     len_t need = 0;
 #define MP_BY_DTYPE(STEM, ...) \
     do { if (dtype == MP_R16) launch_##STEM##_r16(__VA_ARGS__); else if (dtype == MP_R32) launch_##STEM##_r32(__VA_ARGS__); \

@@ -1650,7 +1650,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   if (eight_rows) {
     const size_t need = (m + NORM_BLOCK / 128 - 1) / (NORM_BLOCK / 128);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
-    if (note_plan(PLAN_RESIDENT, 128, 2, NORM_BLOCK / 128, grid.x, block.x)) return;
+    if (note_plan(PLAN_RESIDENT, 128, 2, NORM_BLOCK / 128, grid.x, block.x, 1, 0, 0, keep)) return;
     if (keep) rmsnorm_fwd_resident<T, W, 128, 2, false, NORM_BLOCK, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
     else rmsnorm_fwd_resident<T, W, 128, 2, false><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
     MP_CHECK_LAUNCH();
@@ -1663,7 +1663,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
       const int rpb = NORM_BLOCK / WAVE / gw;
       const size_t need = (m + rpb - 1) / rpb;
       const dim3 grid((unsigned)(need < cap ? need : cap)), block(rpb * gw * WAVE);
-      if (note_plan(PLAN_ANY, gw * WAVE, shot.NV, rpb, grid.x, block.x)) return;
+      if (note_plan(PLAN_ANY, gw * WAVE, shot.NV, rpb, grid.x, block.x, 1, 0, 0, keep)) return;
       if (shot.NV == 1) {
         if (keep) rmsnorm_fwd_any<T, W, 1, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
         else rmsnorm_fwd_any<T, W, 1><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n, gw);
@@ -1683,7 +1683,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
         const size_t need = (m + ONESHOT / G - 1) / (ONESHOT / G);
         require(need < 0x7fffffffull, "rmsnorm: too many rows for one grid");
         const dim3 grid((unsigned)need), block(ONESHOT);
-        if (note_plan(PLAN_RESIDENT, G, NV, ONESHOT / G, grid.x, block.x)) return;
+        if (note_plan(PLAN_RESIDENT, G, NV, ONESHOT / G, grid.x, block.x, 1, 0, 0, keep && !loose)) return;
         if (loose) rmsnorm_fwd_resident<T, W, G, NV, true, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
         else if (keep) rmsnorm_fwd_resident<T, W, G, NV, false, ONESHOT, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
         else rmsnorm_fwd_resident<T, W, G, NV, false, ONESHOT><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
@@ -1702,7 +1702,7 @@ inline void rmsnorm_forward(const T* x, const T* gain, T* y, void* scratch, doub
   const bool resident = for_row_plan<MAXNV, true>(plan, [&]<int G, int NV>() {
     const size_t need = (m + NORM_BLOCK / G - 1) / (NORM_BLOCK / G);
     const dim3 grid((unsigned)(need < cap ? need : cap)), block(NORM_BLOCK);
-    if (note_plan(PLAN_RESIDENT, G, NV, NORM_BLOCK / G, grid.x, block.x)) return;
+    if (note_plan(PLAN_RESIDENT, G, NV, NORM_BLOCK / G, grid.x, block.x, 1, 0, 0, keep && !loose)) return;
     if (loose) rmsnorm_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);
     else if (keep)
       rmsnorm_fwd_resident<T, W, G, NV, false, NORM_BLOCK, true><<<grid, block, 0, stream>>>(x, gain, y, (P)eps, m, n);

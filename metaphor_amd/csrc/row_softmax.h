@@ -901,7 +901,7 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
     long long region = 0;
     /* what the launch may touch of the caller's workspace: the words, when the library has none of its own for it */
     if (note_plan(PLAN_CLUSTER, CLUSTER_THREADS, cluster_nv<T>(), 1, m * C, CLUSTER_THREADS, C, ppb,
-                  C > 1 ? m * (size_t)C * WPS * sizeof(share_word) : 0))
+                  C > 1 ? m * (size_t)C * WPS * sizeof(share_word) : 0, keep_output(m * n * sizeof(T))))
       return;
     if (C > 1) {
       region = share_region(scratch, m, C, WPS);
@@ -942,7 +942,7 @@ inline void softmax_forward(const T* x, T* y, void* scratch, size_t m, size_t n,
   const bool keep = keep_output(m * n * sizeof(T));
   const bool resident = for_row_plan<MAXNV, true, FIT>(plan, [&]<int G, int NV>() {
     const dim3 grid(row_grid(m, G)), block(G < WAVE ? WAVE : G);
-    if (note_plan(PLAN_RESIDENT, G, NV, G < WAVE ? WAVE / G : 1, grid.x, block.x)) return;
+    if (note_plan(PLAN_RESIDENT, G, NV, G < WAVE ? WAVE / G : 1, grid.x, block.x, 1, 0, 0, keep && !ragged)) return;
     if (ragged) softmax_fwd_resident<T, W, G, NV, true><<<grid, block, 0, stream>>>(x, y, m, n, flags);
     else if (keep) softmax_fwd_resident<T, W, G, NV, false, true><<<grid, block, 0, stream>>>(x, y, m, n, flags);
     else softmax_fwd_resident<T, W, G, NV, false><<<grid, block, 0, stream>>>(x, y, m, n, flags);

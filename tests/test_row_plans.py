@@ -16,7 +16,7 @@ import pytest
 from metaphor_amd import ffi
 
 SHORT, RESIDENT, PAIRED, ANY, CLUSTER, DEEP, STREAM, LOOSE = range(8)
-KIND, GROUP, PPT, RPB, GRID, BLOCK, PER_ROW, CHUNK, WORKSPACE = range(9)
+KIND, GROUP, PPT, RPB, GRID, BLOCK, PER_ROW, CHUNK, WORKSPACE, KEPT = range(10)
 OPS = {"softmax": 0, "softmax_reverse": 1, "rmsnorm": 2, "rmsnorm_reverse": 3}
 ELEM = {0: 2, 1: 4, 2: 8}            # bytes of r16, r32, r64
 ACC = {0: 4, 1: 4, 2: 8}             # bytes of precision<T>
@@ -37,7 +37,7 @@ def _lib():
 
 
 def _plans(lib, op, dtype, m, cus, shift):
-    notes = np.zeros((N_HI - 1, 9), dtype=np.int64)
+    notes = np.zeros((N_HI - 1, 10), dtype=np.int64)
     sizes = np.zeros(N_HI - 1, dtype=np.uint64)
     noted = lib.mpDescribeRowPlans(op, dtype, m, 1, N_HI, cus, shift, notes.ctypes.data, sizes.ctypes.data)
     return int(noted), notes, sizes.astype(np.int64)
@@ -98,7 +98,7 @@ def test_the_benchmark_shapes_take_the_kernels_the_design_names():
     lib = _lib()
 
     def one(op, dtype, m, n, cus=256):
-        notes = np.zeros((1, 9), dtype=np.int64)
+        notes = np.zeros((1, 10), dtype=np.int64)
         sizes = np.zeros(1, dtype=np.uint64)
         assert lib.mpDescribeRowPlans(OPS[op], dtype, m, n, n + 1, cus, 0, notes.ctypes.data, sizes.ctypes.data) == 1
         return notes[0], int(sizes[0])
@@ -117,3 +117,31 @@ def test_the_benchmark_shapes_take_the_kernels_the_design_names():
         assert (p[KIND], p[PER_ROW]) == (CLUSTER, fwd) and p[GRID] == m * fwd and 0 < p[WORKSPACE] <= size
         p, size = one("softmax_reverse", 1, m, n)
         assert (p[KIND], p[PER_ROW]) == (CLUSTER, rev) and 0 < p[WORKSPACE] <= size
+
+
+@pytest.mark.parametrize("dtype", [0, 1], ids=["r16", "r32"])
+def test_forwards_keep_a_tensor_for_their_reverse_by_its_size(dtype):
+    """The RMSNorm forward leaves an input of up to 256 MiB, the softmax forward an output of up to
+    128 MiB, in the memory-side cache (its kernels' KEEP variants), larger tensors stream past it;
+    only the kernels for aligned rows of whole packs have the variant, and no reverse has one."""
+    lib = _lib()
+    w = 16 // ELEM[dtype]
+    n = np.arange(1, N_HI, dtype=np.int64)
+    whole = n % w == 0
+    for m in (64, 512, 4096, 32768):
+        nbytes = m * n * ELEM[dtype]
+        _, p, _ = _plans(lib, OPS["rmsnorm"], dtype, m, 256, 0)
+        able = np.isin(p[:, KIND], (RESIDENT, ANY)) & whole
+        want = able & (nbytes <= 256 << 20)
+        assert (p[:, KEPT] == want).all(), f"rmsnorm m {m}: n = {n[p[:, KEPT] != want][:5]}"
+        assert want.any() or m * N_HI * ELEM[dtype] < (256 << 20) or not able.any()
+        _, p, _ = _plans(lib, OPS["softmax"], dtype, m, 256, 0)
+        able = ((p[:, KIND] == RESIDENT) & whole) | (p[:, KIND] == CLUSTER)
+        want = able & (nbytes <= 128 << 20)
+        assert (p[:, KEPT] == want).all(), f"softmax m {m}: n = {n[p[:, KEPT] != want][:5]}"
+        for op in ("softmax_reverse", "rmsnorm_reverse"):
+            _, p, _ = _plans(lib, OPS[op], dtype, m, 256, 0)
+            assert not p[:, KEPT].any(), f"{op} m {m}"
+    # operands shifted off their 16-byte alignment: no variant keeps anything but the shared-row softmax
+    _, p, _ = _plans(lib, OPS["rmsnorm"], dtype, 512, 256, 1)
+    assert not p[:, KEPT].any()
