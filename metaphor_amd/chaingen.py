@@ -218,7 +218,7 @@ extern "C" void launch_{name}_Scalar(
   StreamContext stream
 ) {{
   const mp::EwPtrs<{k}, 1> ptrs{{{{{ins}}}, {{out}}}};
-  mp::ew_launch<Scalar, {k}, 1, 1>(ptrs, N, {_camel(name)}Fn_Scalar{{}}, get_stream(stream));
+  mp::ew_launch_forward<Scalar, {k}, 1, 1>(ptrs, N, {_camel(name)}Fn_Scalar{{}}, get_stream(stream));
 }}
 """
 

@@ -358,6 +358,8 @@ std::string chain_source(Expr& e, int dtype) {
     for (int l = 0; l < 3; ++l)
       s += std::string("MP_CHAIN_KERNEL(") + kind.stem + "_" + std::to_string(l) + ", " + layouts[l] + ", " +
            std::to_string(kind.nin) + ", " + std::to_string(kind.nout) + ", " + kind.fn + ")\n";
+  /* the forward once more with loads that leave the inputs in the memory-side cache for the reverse */
+  s += std::string("MP_CHAIN_KERNEL(chain_forward_3, mp::EW_KEPT, ") + std::to_string(k) + ", " + std::to_string(R) + ", ChainForward)\n";
   return s;
 }
 
@@ -407,7 +409,7 @@ bool compile(const std::string& generated, std::vector<char>& code, std::string&
 struct Loaded {
   std::atomic<bool> ready{false}; /* set after module and fn are written, read before they are used */
   hipModule_t module = nullptr;
-  hipFunction_t fn[9] = {};
+  hipFunction_t fn[12] = {}; /* three kinds x (three layouts, and for the forward the one that keeps its inputs) */
 };
 
 /* `build` is held while this chain is compiled or loaded on a device, so that neither holds up
@@ -504,9 +506,9 @@ const Loaded* loaded_here(Chain* c) {
   }
   const char* stems[3] = {"chain_forward_", "chain_reverse_overwrite_", "chain_reverse_blend_"};
   for (int k = 0; k < 3; ++k)
-    for (int layout = 0; layout < 3; ++layout) {
+    for (int layout = 0; layout < (k == 0 ? 4 : 3); ++layout) { /* only the forward has the variant that keeps its inputs */
       const std::string name = stems[k] + std::to_string(layout);
-      r = hipModuleGetFunction(&l.fn[k * 3 + layout], module, name.c_str());
+      r = hipModuleGetFunction(&l.fn[k * 4 + layout], module, name.c_str());
       if (r != hipSuccess) {
         fail("hipModuleGetFunction(" + name + "): " + hipGetErrorString(r));
         (void)hipModuleUnload(module);
@@ -518,7 +520,7 @@ const Loaded* loaded_here(Chain* c) {
   return &l;
 }
 
-int layout_index(int layout) { return layout == mp::EW_ALIGNED ? 0 : layout == mp::EW_PEELED ? 1 : 2; }
+int layout_index(int layout) { return layout == mp::EW_ALIGNED ? 0 : layout == mp::EW_PEELED ? 1 : layout == mp::EW_LOOSE ? 2 : 3; }
 
 /* One launch: kind 0 forward, 1 reverse that overwrites, 2 reverse that blends. */
 int enqueue(Chain* c, int kind, int dtype, const void* const* in, int nin, void* const* out, int nout, double alpha,
@@ -532,7 +534,7 @@ int enqueue(Chain* c, int kind, int dtype, const void* const* in, int nin, void*
   const Loaded* l = loaded_here(c);
   if (l == nullptr) return 1;
   const size_t elem = dtype == MP_R16 ? 2 : dtype == MP_R32 ? 4 : 8;
-  const mp::EwPlan plan = mp::ew_plan(in, nin, out, nout, n, elem, mp::EW_BLOCK, 1);
+  const mp::EwPlan plan = mp::ew_plan(in, nin, out, nout, n, elem, mp::EW_BLOCK, 1, kind == 0);
   /* the kernel's first parameter is EwPtrs<nin, nout> by value: the inputs, then the outputs */
   const void* ptrs[2 * MAX_LEAVES + MAX_ROOTS + MAX_LEAVES];
   for (int s = 0; s < nin; ++s) ptrs[s] = in[s];
@@ -542,7 +544,7 @@ int enqueue(Chain* c, int kind, int dtype, const void* const* in, int nin, void*
   args.alpha = alpha;
   for (size_t i = 0; i < constants.size() && i < (size_t)MAX_CONSTANTS; ++i) args.c[i] = constants[i];
   void* params[4] = {ptrs, &n, &head, &args};
-  const hipError_t r = hipModuleLaunchKernel(l->fn[kind * 3 + layout_index(plan.layout)], plan.blocks, 1, 1, mp::EW_BLOCK, 1, 1,
+  const hipError_t r = hipModuleLaunchKernel(l->fn[kind * 4 + layout_index(plan.layout)], plan.blocks, 1, 1, mp::EW_BLOCK, 1, 1,
                                              0, stream, params, nullptr);
   if (r != hipSuccess) return fail(std::string("hipModuleLaunchKernel: ") + hipGetErrorString(r));
   return 0;

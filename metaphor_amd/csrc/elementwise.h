@@ -47,7 +47,18 @@ template <int NIN> constexpr int ew_block() { return NIN == 0 ? 256 : EW_BLOCK; 
  * against 6.4 TB/s); all 16-byte aligned; or anything else, and the packs then start at any element (see loose_vec_of),
  * which costs a streaming kernel 5-15 % where one-element accesses cost half (r32) or three
  * quarters (r16) of the bandwidth. */
-enum EwLayout { EW_ALIGNED, EW_PEELED, EW_LOOSE };
+enum EwLayout { EW_ALIGNED, EW_PEELED, EW_LOOSE, EW_KEPT };
+/* EW_KEPT is EW_ALIGNED with ordinary loads in place of non-temporal ones: the inputs stay in the
+ * memory-side cache (256 MiB in front of the HBM stacks), where the reverse of the same expression,
+ * which reads every input of its forward again (four of its nine streams for
+ * selu(hadamard(add, add))), finds them. launch_fused_selu_hadamard_add_add_r32 and its reverse in
+ * turn on operands that nothing touched for five steps, against the same with every operand one
+ * element further (the peeled layout, whose loads stream): 8 MiB a tensor 23.3 -> 18.9 us a step,
+ * 32 MiB 82.1 -> 74.1, 64 MiB 159.7 -> 145.3; the forward on its own pays for it from 16 MiB a
+ * tensor up (32 MiB: 28.2 -> 30.8 us, 64 MiB: 55.6 -> 59.2) and gains below (8 MiB: 8.5 -> 7.8).
+ * Taken by the forward launchers of fused chains whose inputs together are no larger than the
+ * cache. */
+constexpr size_t EW_KEEP_BYTES = 256u << 20;
 
 /* F::apply(const P (&in)[NIN], P (&out)[NOUT]) computes one element. head: the elements before the
  * first pack (EW_PEELED only, less than a cache line of them). */
@@ -55,7 +66,7 @@ template <class T, int W, int LAYOUT, int NIN, int NOUT, int UNROLL, class F>
 __device__ __forceinline__ void ew_body(const EwPtrs<NIN, NOUT>& ptrs, size_t n, unsigned head_arg, const F& f) {
   using P = typename precision<T>::type;
   constexpr int NA = NIN > 0 ? NIN : 1, EW_BLOCK = ew_block<NIN>();
-  constexpr bool LOOSE = LAYOUT == EW_LOOSE;
+  constexpr bool LOOSE = LAYOUT == EW_LOOSE, KEPT = LAYOUT == EW_KEPT;
   const size_t head = LAYOUT == EW_PEELED ? head_arg : 0;
   const size_t npacks = (n - head) / W;
   const size_t base = (size_t)blockIdx.x * (EW_BLOCK * UNROLL) + threadIdx.x;
@@ -68,6 +79,7 @@ __device__ __forceinline__ void ew_body(const EwPtrs<NIN, NOUT>& ptrs, size_t n,
 #pragma unroll
       for (int s = 0; s < NIN; ++s) {
         if constexpr (LOOSE) load_pack_nt_loose<T, W>(static_cast<const T*>(ptrs.in[s]) + head + p * W, in[u][s]);
+        else if constexpr (KEPT) load_pack<T, W>(static_cast<const T*>(ptrs.in[s]) + head + p * W, in[u][s]);
         else load_pack_nt<T, W>(static_cast<const T*>(ptrs.in[s]) + head + p * W, in[u][s]);
       }
     }
@@ -126,7 +138,7 @@ struct EwPlan {
 };
 #ifdef MP_HOST_SIDE
 inline EwPlan ew_plan(const void* const* in, int nin, void* const* out, int nout, size_t n, size_t elem_bytes,
-                      int block_threads, int unroll) {
+                      int block_threads, int unroll, bool keepable = false) {
   const int W = PACK_BYTES / (int)elem_bytes;
   /* the place in a cache line that the operands share, or ~0u when they differ */
   auto in_line = [](const void* p) { return (unsigned)(reinterpret_cast<uintptr_t>(p) & 127u); };
@@ -146,25 +158,36 @@ inline EwPlan ew_plan(const void* const* in, int nin, void* const* out, int nout
   const size_t per_block = (size_t)block_threads * unroll;
   size_t blocks = (npacks + per_block - 1) / per_block;
   if (blocks == 0) blocks = 1; /* only single elements */
-  return EwPlan{peel ? EW_PEELED : packed ? EW_ALIGNED : EW_LOOSE, head, (unsigned)blocks};
+  const bool keep = keepable && !peel && packed && (size_t)nin * n * elem_bytes <= EW_KEEP_BYTES;
+  return EwPlan{peel ? EW_PEELED : keep ? EW_KEPT : packed ? EW_ALIGNED : EW_LOOSE, head, (unsigned)blocks};
 }
 
 /* Enqueue f over n elements: one pack per stream per lane, laid out as EwLayout says.
- * n == 0 enqueues nothing. */
-template <class T, int NIN, int NOUT, int UNROLL, class F>
-inline void ew_launch(const EwPtrs<NIN, NOUT>& ptrs, size_t n, F f, hipStream_t stream) {
+ * n == 0 enqueues nothing. KEEPABLE: the launch is the forward of an expression whose reverse reads
+ * its inputs again (see EW_KEPT). */
+template <class T, int NIN, int NOUT, int UNROLL, bool KEEPABLE, class F>
+inline void ew_launch_as(const EwPtrs<NIN, NOUT>& ptrs, size_t n, F f, hipStream_t stream) {
   if (n == 0) return;
   constexpr int EW_BLOCK = ew_block<NIN>();
   require(n / EW_BLOCK < 0x7fffffffull, "elementwise launch: too many elements for one grid");
   constexpr int W = PACK_BYTES / (int)sizeof(T);
   static_assert(128 / sizeof(T) <= 64, "the first workgroup's threads cover the head");
-  const EwPlan plan = ew_plan(ptrs.in, NIN, ptrs.out, NOUT, n, sizeof(T), EW_BLOCK, UNROLL);
+  const EwPlan plan = ew_plan(ptrs.in, NIN, ptrs.out, NOUT, n, sizeof(T), EW_BLOCK, UNROLL, KEEPABLE);
   const unsigned head = plan.head;
   const dim3 grid(plan.blocks), block(EW_BLOCK);
   if (plan.layout == EW_PEELED) ew_kernel<T, W, EW_PEELED, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, head, f);
   else if (plan.layout == EW_ALIGNED) ew_kernel<T, W, EW_ALIGNED, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
-  else ew_kernel<T, W, EW_LOOSE, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
+  else if (plan.layout == EW_LOOSE) ew_kernel<T, W, EW_LOOSE, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
+  else if constexpr (KEEPABLE) ew_kernel<T, W, EW_KEPT, NIN, NOUT, UNROLL, F><<<grid, block, 0, stream>>>(ptrs, n, 0u, f);
   MP_CHECK_LAUNCH();
+}
+template <class T, int NIN, int NOUT, int UNROLL, class F>
+inline void ew_launch(const EwPtrs<NIN, NOUT>& ptrs, size_t n, F f, hipStream_t stream) {
+  ew_launch_as<T, NIN, NOUT, UNROLL, false, F>(ptrs, n, f, stream);
+}
+template <class T, int NIN, int NOUT, int UNROLL, class F>
+inline void ew_launch_forward(const EwPtrs<NIN, NOUT>& ptrs, size_t n, F f, hipStream_t stream) {
+  ew_launch_as<T, NIN, NOUT, UNROLL, true, F>(ptrs, n, f, stream);
 }
 #endif /* MP_HOST_SIDE */
 

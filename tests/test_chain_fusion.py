@@ -125,7 +125,11 @@ def test_every_dtype_compiles_and_is_cached_once(dtype):
     assert lib.mpChainCompile(b"relu( mul(sub(x0, x1), selu(add(x2,x0))) )", dtype) == 0
     assert lib.mpChainCacheSize() == n
     kinds = {0: "_Float16", 1: "float", 2: "double"}
-    assert f"typedef {kinds[dtype]} ChainT;" in lib.mpChainSource(expr, dtype).decode()
+    src = lib.mpChainSource(expr, dtype).decode()
+    assert f"typedef {kinds[dtype]} ChainT;" in src
+    # three operand layouts a direction, and the forward once more with loads that keep its inputs in cache
+    assert src.count("MP_CHAIN_KERNEL(chain_forward_") == 4 and "MP_CHAIN_KERNEL(chain_forward_3, mp::EW_KEPT" in src
+    assert src.count("MP_CHAIN_KERNEL(chain_reverse_overwrite_") == 3 and src.count("MP_CHAIN_KERNEL(chain_reverse_blend_") == 3
 
 
 @pytest.mark.parametrize("bad,why", [

@@ -240,6 +240,37 @@ def _leaves_only(e):
     return re.sub(r"((?:scale|shift)\((?:[^()]|\([^()]*\))*),(-?[\d.]+(?:e-?\d+)?)\)", lambda m: f"{m.group(1)},{float(m.group(2))!r}e0)", e)
 
 
+def test_forward_variants_that_keep_or_stream_their_inputs_give_the_same_bits():
+    """A chain's forward loads inputs that together fit the memory-side cache with ordinary loads (its
+    reverse then finds them there) and larger ones, or operands off their 16-byte alignment, with
+    streaming loads: the same values either way, build-time and run-time kernels alike. 2^20 elements
+    (kept when aligned, streaming one element further) and 17 * 2^20 (four inputs of 68 MiB: beyond
+    the cache, streaming)."""
+    f32 = torch.float32
+    expr = "selu(mul(add(0,1),add(2,3)))"
+    r = np.random.default_rng(11)
+    for n in (1 << 20, 17 << 20):
+        vals = [torch.from_numpy(r.uniform(-2, 2, n).astype(np.float32)).cuda() for _ in range(4)]
+        got = []
+        for shift in (0, 1):
+            xs = [G.Guarded((n,), f32, shift) for _ in range(4)]
+            for x, v in zip(xs, vals):
+                x.t.copy_(v)
+            run_time, build_time = G.Guarded((n,), f32, shift), G.Guarded((n,), f32, shift)
+            G.say(f"chain forward variants n={n} shift={shift}")
+            assert G.chain_forward(expr, [x.t for x in xs], run_time.t) == 0, G.chain_error()
+            _static("fused_selu_hadamard_add_add", f32, *[x.t.data_ptr() for x in xs], build_time.t.data_ptr(), n)
+            torch.cuda.synchronize()
+            for b in xs + [run_time, build_time]:
+                b.check("chain forward variants")
+            got.append((run_time.t.clone(), build_time.t.clone()))
+            del xs, run_time, build_time
+        assert torch.equal(got[0][0], got[1][0]), f"n={n}: the run-time kernel's forward variants differ"
+        assert torch.equal(got[0][1], got[1][1]), f"n={n}: the build-time kernel's forward variants differ"
+        del got, vals
+        torch.cuda.empty_cache()
+
+
 def test_rate_of_a_run_time_kernel_beside_the_build_time_one():
     """2^26 r32 elements: the run-time kernel of the benchmark chain beside the build-time one (same
     engine, same functor), events around 10 launches each. Printed, not asserted: wall-clock checks
