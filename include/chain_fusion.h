@@ -43,7 +43,9 @@
 
 /* out[i] = expression(x[0][i], ..., x[k-1][i]) for i < n: one read of each leaf, one write.
  * x: k device pointers (k = the expression's leaf count), any element alignment; out may alias
- * any x[j] exactly. */
+ * any x[j] exactly. Leaves that are 16-byte aligned and together no larger than 256 MiB are read so
+ * that they stay in the GPU's memory-side cache, where mpChainReverse, which reads them all again,
+ * finds them. */
 EXTERN_C int mpChainForward(const char* expression, int dtype, const void* const* x, void* out, len_t n, StreamContext);
 
 /* Every leaf gradient in one pass: g[j][i] = d expression / d x[j] * out_grads[i] + alpha * g[j][i].
