@@ -278,6 +278,13 @@ class Cfg4(Workload):
         fused_reverse(self.a, self.b, self.c, self.d, self.de, self.da, self.db, self.dc, self.dd, 0.0)
 
 
+class Cfg4Mid(Cfg4):
+    """cfg4's chain on tensors of 32 MiB: inputs that together fit the memory-side cache, which the
+    forward therefore leaves there for its reverse (not a BASELINE configuration)."""
+    name = "cfg4mid"
+    n = 1 << 23
+
+
 class RuntimeChain(Cfg4):
     """cfg4's size and stream mix (4 reads + 1 write forward, 5 + 4 reverse) for an expression no
     build listed: relu((a - b) * (c + d)) is compiled by the fusion library on first use."""
@@ -423,13 +430,14 @@ class NormVocab(Cfg2):
         rmsnorm_forward(self.x, self.gain, self.y, self.eps, self.fwd_scratch)
 
 
-WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg5a, Cfg5b, Copy, Permutate, Gemm, RuntimeChain, NormVocab)}
+WORKLOADS = {c.name: c for c in (Cfg1, Cfg2, Cfg3, Cfg4, Cfg4Mid, Cfg5a, Cfg5b, Copy, Permutate, Gemm, RuntimeChain, NormVocab)}
 
 DESCRIPTION = {
     "cfg1": "softmax fwd r32 [256,1024]",
     "cfg2": "RMSNorm fwd+rev r32 [8192,4096], gain [4096], eps 1e-6",
     "cfg3": "causal attention-score softmax fwd+rev r16 [524288,2048]",
     "cfg4": "fused selu((a+b)*(c+d)) fwd+rev r32 flat 2^28",
+    "cfg4mid": "fused selu((a+b)*(c+d)) fwd+rev r32 flat 2^23: the forward keeps its inputs in the memory-side cache (not a BASELINE configuration)",
     "cfg5a": "vocabulary softmax fwd (+rev) r32 [512,151936]",
     "cfg5b": "vocabulary softmax fwd (+rev) r32 [2048,50257]",
     "chain": "relu((a-b)*(c+d)) fwd+rev r32 flat 2^28, an expression no build listed, compiled at run time",
