@@ -1221,6 +1221,46 @@ def test_launchers_follow_the_stream_of_the_context():
     utils.mpDeinitStream(sc)
 
 
+def test_shared_rows_on_two_streams_at_once_with_a_workspace_each():
+    """Launches that may overlap in time get different workspaces: the workspace is the key under
+    which the library keeps a launch's exchange words. Two streams, each with its own workspace
+    and its own inputs, enqueue the shared-row softmax forward and reverse ten times without
+    waiting for each other; every result against the oracle."""
+    kernels, utils = G.lib()
+    r = rng(71)
+    f32 = torch.float32
+    m, n = 48, 50257
+    fwd_bytes = G.row_size("mpSoftmaxScratchBytes", f32, m, n)
+    rev_bytes = G.row_size("mpSoftmaxReverseScratchBytes", f32, m, n)
+    assert fwd_bytes > 0 and rev_bytes > 0
+    lanes = []
+    for _ in range(2):
+        lanes.append(dict(sc=utils.mpInitStream(), fs=G.Guarded((fwd_bytes,), torch.uint8), rs=G.Guarded((rev_bytes,), torch.uint8),
+                          x=[G.dev(r.normal(0, 3, (m, n)), f32) for _ in range(2)], dy=G.dev(r.normal(0, 1, (m, n)), f32),
+                          y=[G.Guarded((m, n), f32) for _ in range(2)], dx=[G.Guarded((m, n), f32) for _ in range(2)]))
+    torch.cuda.synchronize()
+    G.say(f"shared rows on two streams ({m},{n})")
+    for launch in range(10):
+        for ln in lanes:
+            k = launch % 2
+            kernels.softmax_ij_j[1](ln["x"][k].t.data_ptr(), ln["y"][k].t.data_ptr(), ln["fs"].t.data_ptr(), m, n, ln["sc"])
+            kernels.softmax_ij_j_reverse[1](ln["y"][k].t.data_ptr(), ln["dy"].t.data_ptr(), ln["dx"][k].t.data_ptr(),
+                                            ln["rs"].t.data_ptr(), 0.0, m, n, ln["sc"])
+    for ln in lanes:
+        utils.mpStreamSynchronize(ln["sc"])
+    for i, ln in enumerate(lanes):
+        dyh = G.host(ln["dy"].t)
+        for k in range(2):
+            yh = G.host(ln["y"][k].t)
+            G.compare(ln["y"][k].t, O.softmax_ij_j(G.host(ln["x"][k].t)), f32, f"stream {i} y{k}", atol=1e-6)
+            G.compare(ln["dx"][k].t, O.softmax_ij_j_reverse(yh, dyh), f32, f"stream {i} dx{k}", scale=G.softmax_reverse_scale(yh, dyh))
+            ln["y"][k].check("y")
+            ln["dx"][k].check("dx")
+        ln["fs"].check("forward workspace")
+        ln["rs"].check("reverse workspace")
+        utils.mpDeinitStream(ln["sc"])
+
+
 def test_device_utils_roundtrip():
     kernels, utils = G.lib()
     utils.mpInitDevice(0)
