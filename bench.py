@@ -242,6 +242,9 @@ def rates(w, fwd_ms, rev_ms, step_ms=None):
     if step_ms:  # a forward and the reverse of the same tensors, back to back
         out["step_ms"] = round(_median(step_ms), 5)
         out["step_GBps"] = round((w.fwd_bytes + w.rev_bytes) / (_median(step_ms) * 1e-3) / 1e9, 1)
+        # the same bytes over a forward and a reverse that have nothing to do with each other (other sets):
+        # what the step would run at if the reverse found nothing of its forward in the memory-side cache
+        out["apart_GBps"] = round((w.fwd_bytes + w.rev_bytes) / ((_median(fwd_ms) + _median(rev_ms)) * 1e-3) / 1e9, 1)
         out["step_vs_apart"] = round(_median(step_ms) / (_median(fwd_ms) + _median(rev_ms)), 4)
     if hasattr(w, "fwd_flops"):
         out["fwd_TFLOPs"] = round(w.fwd_flops / (_median(fwd_ms) * 1e-3) / 1e12, 1)
